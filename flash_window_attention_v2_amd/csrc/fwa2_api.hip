@@ -1,0 +1,191 @@
+// extern "C" surface of libfwa2 (declared in include/fwa2.h): argument
+// validation, workspace sizing and dispatch to the gfx950 kernels.  Nothing
+// here allocates device memory or synchronises.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "fwa2_common.hpp"
+
+namespace fwa2 {
+hipError_t launch_forward(FwdParams p, int dtype, bool has_bias, int mask_dt, hipStream_t st);
+hipError_t launch_mask_scan(const void* mask, int mask_dt, int64_t sw, int64_t sn, int n, int n_windows,
+                            uint8_t* live, hipStream_t st);
+hipError_t launch_backward(const BwdParams& p, int dtype, bool has_bias, int mask_dt, hipStream_t st);
+size_t backward_workspace_bytes(int heads, int n, int bw, bool has_bias, bool has_mask, int n_windows, int cus);
+int backward_supported(int n);
+}  // namespace fwa2
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+int check_t4(const char* name, const fwa2_tensor4& t) {
+    if (t.ptr == nullptr) return fail(FWA2_ERR_INVALID_ARGUMENT, "%s: null pointer", name);
+    if (!aligned16(t.ptr) || (t.stride_bw % 8) || (t.stride_h % 8) || (t.stride_n % 8))
+        return fail(FWA2_ERR_UNSUPPORTED,
+                    "%s: rows must start on 16-byte boundaries (pointer 16-byte aligned, strides multiples of 8 elements)",
+                    name);
+    if (t.stride_n < 32) return fail(FWA2_ERR_INVALID_ARGUMENT, "%s: row stride %lld overlaps rows", name, (long long)t.stride_n);
+    return FWA2_OK;
+}
+
+fwa2::T4 to_t4(const fwa2_tensor4& t) { return fwa2::T4{t.ptr, t.stride_bw, t.stride_h, t.stride_n}; }
+
+int cu_count() {
+    static int cus = [] {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess) return 256;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 256;
+        return n;
+    }();
+    return cus;
+}
+
+int validate(const fwa2_problem* p, int backward) {
+    if (p == nullptr) return fail(FWA2_ERR_INVALID_ARGUMENT, "problem is null");
+    if (p->struct_bytes != sizeof(fwa2_problem) || p->abi_version != FWA2_ABI_VERSION)
+        return fail(FWA2_ERR_INVALID_ARGUMENT, "fwa2_problem layout mismatch: caller %u bytes / abi %u, library %zu bytes / abi %d",
+                    p->struct_bytes, p->abi_version, sizeof(fwa2_problem), FWA2_ABI_VERSION);
+    if (p->dtype != FWA2_F16 && p->dtype != FWA2_BF16)
+        return fail(FWA2_ERR_INVALID_ARGUMENT, "Only support fp16 and bf16");
+    if (p->bw <= 0 || p->heads <= 0 || p->n <= 0 || p->head_dim <= 0)
+        return fail(FWA2_ERR_INVALID_ARGUMENT, "bw, heads, n and head_dim must be positive");
+    if (p->head_dim > 128)
+        return fail(FWA2_ERR_INVALID_ARGUMENT, "FlashAttention only support head dimensions up to 128");
+    if (p->head_dim != 32)
+        return fail(FWA2_ERR_UNSUPPORTED, "head_dim %d: this build implements head_dim 32 only", p->head_dim);
+    if ((int64_t)p->bw * p->heads * ((p->n + 255) / 256) > 0x7fffffffLL)
+        return fail(FWA2_ERR_UNSUPPORTED, "too many (batch*window, head) pairs for one launch");
+    int rc;
+    if ((rc = check_t4("q", p->q)) || (rc = check_t4("k", p->k)) || (rc = check_t4("v", p->v)) || (rc = check_t4("o", p->o)))
+        return rc;
+    if (p->scale_kind == FWA2_SCALE_TENSOR) {
+        if (p->logit_scale == nullptr) return fail(FWA2_ERR_INVALID_ARGUMENT, "logit_scale: null with FWA2_SCALE_TENSOR");
+    } else if (p->scale_kind != FWA2_SCALE_DEFAULT) {
+        return fail(FWA2_ERR_INVALID_ARGUMENT, "scale_kind %d unknown", p->scale_kind);
+    }
+    if (p->bias.ptr && p->bias.stride_n < p->n)
+        return fail(FWA2_ERR_INVALID_ARGUMENT, "bias: row stride %lld < n", (long long)p->bias.stride_n);
+    if (p->mask.ptr) {
+        if (p->mask_dtype != p->dtype && p->mask_dtype != FWA2_F32)
+            return fail(FWA2_ERR_INVALID_ARGUMENT, "mask dtype must be the input dtype or fp32");
+        if (p->n_windows <= 0 || p->bw % p->n_windows)
+            return fail(FWA2_ERR_INVALID_ARGUMENT, "bw %d is not a multiple of n_windows %d", p->bw, p->n_windows);
+        if (p->mask.stride_n < p->n)
+            return fail(FWA2_ERR_INVALID_ARGUMENT, "mask: row stride %lld < n", (long long)p->mask.stride_n);
+    }
+    if (p->lse == nullptr) return fail(FWA2_ERR_INVALID_ARGUMENT, "lse: null pointer");
+    if (p->lse_stride_h < p->n) return fail(FWA2_ERR_INVALID_ARGUMENT, "lse: head stride %lld < n", (long long)p->lse_stride_h);
+    if (backward) {
+        if ((rc = check_t4("do", p->d_o)) || (rc = check_t4("dq", p->dq)) || (rc = check_t4("dk", p->dk)) ||
+            (rc = check_t4("dv", p->dv)))
+            return rc;
+        if (p->bias.ptr && p->dbias == nullptr) return fail(FWA2_ERR_INVALID_ARGUMENT, "dbias: null although bias is given");
+        if (p->scale_kind == FWA2_SCALE_TENSOR && p->dscale == nullptr)
+            return fail(FWA2_ERR_INVALID_ARGUMENT, "dscale: null although logit_scale is given");
+        if (!fwa2::backward_supported(p->n))
+            return fail(FWA2_ERR_UNSUPPORTED, "backward: n = %d is not supported by this build", p->n);
+        const size_t need = fwa2_backward_workspace_bytes(p);
+        if (need && (p->workspace == nullptr || p->workspace_bytes < need))
+            return fail(FWA2_ERR_INVALID_ARGUMENT, "workspace: need %zu bytes, got %zu", need, p->workspace_bytes);
+        if (need && (reinterpret_cast<uintptr_t>(p->workspace) & 255))
+            return fail(FWA2_ERR_INVALID_ARGUMENT, "workspace must be 256-byte aligned");
+    }
+    return FWA2_OK;
+}
+
+bool row_vec_ok(const void* ptr, int64_t sa, int64_t sn, int n) {
+    return aligned16(ptr) && (sa % 8) == 0 && (sn % 8) == 0 && (n % 8) == 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int fwa2_abi_version(void) { return FWA2_ABI_VERSION; }
+
+const char* fwa2_last_error(void) { return g_err; }
+
+int fwa2_validate(const fwa2_problem* p, int backward) {
+    g_err[0] = 0;
+    return validate(p, backward);
+}
+
+size_t fwa2_backward_workspace_bytes(const fwa2_problem* p) {
+    if (p == nullptr) return 0;
+    return fwa2::backward_workspace_bytes(p->heads, p->n, p->bw, p->bias.ptr != nullptr, p->mask.ptr != nullptr,
+                                          p->n_windows, cu_count());
+}
+
+int fwa2_mask_scan(const void* mask, int mask_dtype, int n_windows, int n, int64_t stride_w, int64_t stride_n,
+                   uint8_t* live, void* stream) {
+    g_err[0] = 0;
+    if (mask == nullptr || live == nullptr || n_windows <= 0 || n <= 0)
+        return fail(FWA2_ERR_INVALID_ARGUMENT, "fwa2_mask_scan: bad argument");
+    if (mask_dtype != FWA2_F16 && mask_dtype != FWA2_BF16 && mask_dtype != FWA2_F32)
+        return fail(FWA2_ERR_INVALID_ARGUMENT, "fwa2_mask_scan: bad mask dtype");
+    hipError_t e = fwa2::launch_mask_scan(mask, mask_dtype, stride_w, stride_n, n, n_windows, live, (hipStream_t)stream);
+    if (e != hipSuccess) return fail(FWA2_ERR_HIP, "mask scan launch: %s", hipGetErrorString(e));
+    return FWA2_OK;
+}
+
+int fwa2_forward(const fwa2_problem* p) {
+    g_err[0] = 0;
+    int rc = validate(p, 0);
+    if (rc) return rc;
+    fwa2::FwdParams k;
+    memset(&k, 0, sizeof(k));
+    k.q = to_t4(p->q); k.k = to_t4(p->k); k.v = to_t4(p->v); k.o = to_t4(p->o);
+    k.logit_scale = p->logit_scale;
+    k.bias = p->bias.ptr; k.bias_sh = p->bias.stride_a; k.bias_sn = p->bias.stride_n;
+    k.mask = p->mask.ptr; k.mask_sw = p->mask.stride_a; k.mask_sn = p->mask.stride_n;
+    k.mask_live = p->mask.ptr ? p->mask_live : nullptr;
+    k.lse = p->lse; k.lse_sb = p->lse_stride_bw; k.lse_sh = p->lse_stride_h;
+    k.bw = p->bw; k.heads = p->heads; k.n = p->n; k.n_windows = p->mask.ptr ? p->n_windows : 1;
+    k.scale_kind = p->scale_kind;
+    k.default_scale = 1.0f / sqrtf((float)p->head_dim);
+    k.bias_vec = p->bias.ptr && row_vec_ok(p->bias.ptr, p->bias.stride_a, p->bias.stride_n, p->n);
+    k.mask_vec = p->mask.ptr && row_vec_ok(p->mask.ptr, p->mask.stride_a, p->mask.stride_n, p->n);
+    hipError_t e = fwa2::launch_forward(k, p->dtype, p->bias.ptr != nullptr, p->mask.ptr ? p->mask_dtype : -1,
+                                        (hipStream_t)p->stream);
+    if (e != hipSuccess) return fail(FWA2_ERR_HIP, "forward launch: %s", hipGetErrorString(e));
+    return FWA2_OK;
+}
+
+int fwa2_backward(const fwa2_problem* p) {
+    g_err[0] = 0;
+    int rc = validate(p, 1);
+    if (rc) return rc;
+    fwa2::BwdParams k;
+    memset(&k, 0, sizeof(k));
+    k.q = to_t4(p->q); k.k = to_t4(p->k); k.v = to_t4(p->v); k.o = to_t4(p->o);
+    k.d_o = to_t4(p->d_o); k.dq = to_t4(p->dq); k.dk = to_t4(p->dk); k.dv = to_t4(p->dv);
+    k.logit_scale = p->logit_scale;
+    k.bias = p->bias.ptr; k.bias_sh = p->bias.stride_a; k.bias_sn = p->bias.stride_n;
+    k.mask = p->mask.ptr; k.mask_sw = p->mask.stride_a; k.mask_sn = p->mask.stride_n;
+    k.mask_live = p->mask.ptr ? p->mask_live : nullptr;
+    k.lse = p->lse; k.lse_sb = p->lse_stride_bw; k.lse_sh = p->lse_stride_h;
+    k.bw = p->bw; k.heads = p->heads; k.n = p->n; k.n_windows = p->mask.ptr ? p->n_windows : 1;
+    k.scale_kind = p->scale_kind;
+    k.default_scale = 1.0f / sqrtf((float)p->head_dim);
+    k.dbias = p->dbias; k.dscale = p->dscale;
+    k.workspace = p->workspace;
+    k.cus = cu_count();
+    hipError_t e = fwa2::launch_backward(k, p->dtype, p->bias.ptr != nullptr, p->mask.ptr ? p->mask_dtype : -1,
+                                         (hipStream_t)p->stream);
+    if (e != hipSuccess) return fail(FWA2_ERR_HIP, "backward launch: %s", hipGetErrorString(e));
+    return FWA2_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,524 @@
+// Backward kernels: dq, dk, dv, dbias, dlogit_scale for gfx950.
+//
+// Replaces _bwd_preprocess_do_o_dot, _bwd_kernel and the host epilogue of the
+// reference (flash_win_attn_v2/kernels/attn_kernel_backward.py:6-51, 84-564,
+// 703-711).
+//
+// Work split.  A workgroup is PERSISTENT for one head: it walks over many
+// (batch*window) units of that head and keeps the bias-gradient tile in
+// registers for the whole walk, so dbias costs one register add per score and
+// one plain store per workgroup instead of one global atomic per score.
+// Inside a workgroup every wavefront owns 16 keys (16 wavefronts at N = 256)
+// and streams all queries of the unit past them, 32 at a time.
+//
+// Per unit:
+//   load     q, k (L2-normalised, q additionally times s*log2e), dO -> LDS in
+//            the input dtype; delta = rowsum(o*dO) and lse*log2e -> LDS.
+//   phase A  S = Q_hat K_hat^T and dP = dO V^T with v_mfma_f32_16x16x32
+//            (rows = queries, columns = this wave's keys), P = 2^(S+bias+mask-lse),
+//            dZ = P (dP - delta); dbias registers += dZ; the accumulators,
+//            rounded to the input dtype, are directly the B operands (k =
+//            queries) of dV^T += dO^T P and dK_hat^T += Q_hat^T dZ, whose A
+//            operands come out of the row-major LDS tiles with
+//            ds_read_b64_tr_b16.  dZ is also written to LDS, key-major.
+//   phase B  dQ_hat^T = K_hat^T dZ^T, the one product that contracts over keys:
+//            both operands are transposing LDS reads; the 4 partial sums per
+//            output tile meet in an fp32 LDS accumulator (ds_add_f32).
+//   epilogue back through the normalisation: dx = (dx_hat - x_hat (dx_hat.x_hat)) / |x|;
+//            dlogit_scale falls out of the same dot product because
+//            sum_j dC_ij c_ij = q_hat_i . dq_hat_i.
+//
+// bias and mask are read key-major (transposed once per call by a small
+// pre-pass into the workspace) so that a lane's 8 scores are one 16-byte load.
+#include "fwa2_common.hpp"
+
+namespace fwa2 {
+
+constexpr int kRow = 40;    // LDS row stride of 16-bit tiles, in elements (80 bytes)
+constexpr int kAccRow = 33; // LDS row stride of the fp32 dQ accumulator, in floats
+
+template <int DT, int MASK_DT> struct MaskElemB { typedef typename Elem<DT>::E E; };
+template <int DT> struct MaskElemB<DT, FWA2_F32> { typedef float E; };
+
+template <class V8>
+__device__ __forceinline__ void unpack8b(V8 v, float* x) {
+#pragma unroll
+    for (int j = 0; j < 8; j++) x[j] = (float)v[j];
+}
+
+__device__ __forceinline__ float wave_sum(float x) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) x += __shfl_xor(x, off);
+    return x;
+}
+
+template <int DT, bool HAS_BIAS, int MASK_DT, int NQB>
+__global__ void __launch_bounds__(NQB * 128) bwd_kernel(const BwdParams p) {
+    typedef typename Elem<DT>::E E;
+    typedef typename Elem<DT>::V8 V8;
+    typedef typename Elem<DT>::V4 V4;
+    typedef typename MaskElemB<DT, MASK_DT>::E ME;
+    typedef ME MV8 __attribute__((ext_vector_type(8)));
+
+    const int N = p.n;
+    const int R = (N + 31) & ~31;          // padded query rows (and LDS rows)
+    const int NPk = p.waves * 16;          // padded key rows
+    const int nqb = R >> 5;                // query blocks of 32
+    const int nks = R >> 5;                // key steps of 32 in phase B
+    const int ngroups = p.waves >= 4 ? (p.waves >> 2) : 1;
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    E* Qs = reinterpret_cast<E*>(smem_raw);
+    E* Ks = Qs + R * kRow;
+    E* dOs = Ks + R * kRow;
+    E* dZs = dOs + R * kRow;               // 2 buffers
+    float* dQacc = reinterpret_cast<float*>(dZs + 2 * R * kRow);
+    float* lse2s = dQacc + R * kAccRow;
+    float* deltas = lse2s + R;
+    float* red = deltas + R;               // [16]
+
+    const int tid = threadIdx.x;
+    const int nthreads = blockDim.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int l16 = lane & 15;
+    const int g = lane >> 4;
+
+    const int h = blockIdx.x / p.groups;
+    const int grp = blockIdx.x - h * p.groups;
+
+    float s_true;
+    if (p.scale_kind == FWA2_SCALE_TENSOR) {
+        float ls = (float)reinterpret_cast<const E*>(p.logit_scale)[h];
+        s_true = expf(fminf(ls, kLn100));
+    } else {
+        s_true = p.default_scale;
+    }
+    const float scale2 = s_true * kLog2e;
+
+    const int key = wave * 16 + l16;       // the key this lane owns in the score tiles
+    const bool key_ok = key < N;
+
+    float dbacc[NQB][8];
+#pragma unroll
+    for (int a = 0; a < NQB; a++)
+#pragma unroll
+        for (int j = 0; j < 8; j++) dbacc[a][j] = 0.f;
+    float ds_part = 0.f;
+
+    // dZ staging rows that no wavefront writes must read as zeros in phase B
+    for (int i = tid; i < 2 * R * kRow / 8; i += nthreads) st8<V8>(dZs + i * 8, zero8<V8>());
+
+    const E* bias_t = nullptr;
+    if (HAS_BIAS) bias_t = reinterpret_cast<const E*>(p.bias_t) + ((int64_t)h * NPk + key) * R;
+
+    for (int b = grp; b < p.bw; b += p.groups) {
+        const E* qptr = reinterpret_cast<const E*>(p.q.ptr) + b * p.q.sb + h * p.q.sh;
+        const E* kptr = reinterpret_cast<const E*>(p.k.ptr) + b * p.k.sb + h * p.k.sh;
+        const E* vptr = reinterpret_cast<const E*>(p.v.ptr) + b * p.v.sb + h * p.v.sh;
+        const E* optr = reinterpret_cast<const E*>(p.o.ptr) + b * p.o.sb + h * p.o.sh;
+        const E* doptr = reinterpret_cast<const E*>(p.d_o.ptr) + b * p.d_o.sb + h * p.d_o.sh;
+        const float* lseptr = p.lse + b * p.lse_sb + h * p.lse_sh;
+
+        const ME* mask_t = nullptr;
+        bool mask_on = false;
+        if (MASK_DT >= 0) {
+            const int w = b % p.n_windows;
+            mask_on = p.mask_live ? (p.mask_live[w] != 0) : true;
+            mask_t = reinterpret_cast<const ME*>(p.mask_t) + ((int64_t)w * NPk + key) * R;
+        }
+
+        __syncthreads();   // the previous unit's epilogue is done with LDS
+        // ---- load: one 8-element chunk of one row per thread ----
+        for (int r = tid >> 2; r < R; r += nthreads >> 2) {
+            const int dc = (tid & 3) * 8;
+            V8 q8 = zero8<V8>(), k8 = zero8<V8>(), do8 = zero8<V8>(), o8 = zero8<V8>();
+            if (r < N) {
+                q8 = ld8<V8>(qptr + (int64_t)r * p.q.sn + dc);
+                k8 = ld8<V8>(kptr + (int64_t)r * p.k.sn + dc);
+                do8 = ld8<V8>(doptr + (int64_t)r * p.d_o.sn + dc);
+                o8 = ld8<V8>(optr + (int64_t)r * p.o.sn + dc);
+            }
+            float xq[8], xk[8], xd[8], xo[8];
+            unpack8b(q8, xq); unpack8b(k8, xk); unpack8b(do8, xd); unpack8b(o8, xo);
+            float sq = 0.f, sk = 0.f, dl = 0.f;
+#pragma unroll
+            for (int j = 0; j < 8; j++) { sq += xq[j] * xq[j]; sk += xk[j] * xk[j]; dl += xo[j] * xd[j]; }
+            sq = quad_add(sq); sk = quad_add(sk); dl = quad_add(dl);
+            const float iq = inv_norm(sq) * scale2, ik = inv_norm(sk);
+            V8 qn, kn;
+#pragma unroll
+            for (int j = 0; j < 8; j++) { qn[j] = (E)(xq[j] * iq); kn[j] = (E)(xk[j] * ik); }
+            st8<V8>(Qs + r * kRow + dc, qn);
+            st8<V8>(Ks + r * kRow + dc, kn);
+            st8<V8>(dOs + r * kRow + dc, do8);
+            if ((tid & 3) == 0) deltas[r] = dl;
+            if ((tid & 3) == 1) {
+                float l2 = INFINITY;           // padded / fully masked rows: P = 0
+                if (r < N) { const float l = lseptr[r]; l2 = (l == -INFINITY) ? INFINITY : l * kLog2e; }
+                lse2s[r] = l2;
+            }
+#pragma unroll
+            for (int j = 0; j < 8; j++) dQacc[r * kAccRow + dc + j] = 0.f;
+        }
+        V8 bv = zero8<V8>();
+        if (key_ok) bv = ld8<V8>(vptr + (int64_t)key * p.v.sn + 8 * g);
+        __syncthreads();
+        const V8 bk = ld8<V8>(Ks + key * kRow + 8 * g);
+
+        f32x4 dvacc[2], dkacc[2];
+#pragma unroll
+        for (int dt = 0; dt < 2; dt++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) { dvacc[dt][i] = 0.f; dkacc[dt][i] = 0.f; }
+
+#pragma unroll
+        for (int qb = 0; qb < NQB; qb++) {
+            if (qb < nqb) {
+                E* dZbuf = dZs + (qb & 1) * R * kRow;
+                const int q8 = 32 * qb + 8 * g;          // first of this lane's 8 queries
+                // ---- phase A ----
+                f32x4 sacc[2], pacc[2];
+#pragma unroll
+                for (int t = 0; t < 2; t++) {
+                    const int rowq = 32 * qb + 8 * (l16 >> 2) + 4 * t + (l16 & 3);
+                    const V8 aq = ld8<V8>(Qs + rowq * kRow + 8 * g);
+                    const V8 ado = ld8<V8>(dOs + rowq * kRow + 8 * g);
+                    f32x4 z = {0.f, 0.f, 0.f, 0.f};
+                    sacc[t] = Elem<DT>::mfma16(aq, bk, z);
+                    pacc[t] = Elem<DT>::mfma16(ado, bv, z);
+                }
+                float zz[8];
+#pragma unroll
+                for (int j = 0; j < 8; j++) zz[j] = sacc[j >> 2][j & 3];
+                if (HAS_BIAS) {
+                    float x[8];
+                    unpack8b(ld8<V8>(bias_t + q8), x);
+#pragma unroll
+                    for (int j = 0; j < 8; j++) zz[j] = fmaf(x[j], kLog2e, zz[j]);
+                }
+                if (MASK_DT >= 0) {
+                    if (mask_on) {
+                        const MV8 mv = *reinterpret_cast<const MV8*>(mask_t + q8);
+#pragma unroll
+                        for (int j = 0; j < 8; j++) zz[j] = fmaf((float)mv[j], kLog2e, zz[j]);
+                    }
+                }
+                const f32x4 la = *reinterpret_cast<const f32x4*>(lse2s + q8);
+                const f32x4 lb = *reinterpret_cast<const f32x4*>(lse2s + q8 + 4);
+                const f32x4 da = *reinterpret_cast<const f32x4*>(deltas + q8);
+                const f32x4 db = *reinterpret_cast<const f32x4*>(deltas + q8 + 4);
+                V8 p8, z8;
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    const float l2 = j < 4 ? la[j & 3] : lb[j & 3];
+                    const float dl = j < 4 ? da[j & 3] : db[j & 3];
+                    const float zin = key_ok ? zz[j] : -INFINITY;
+                    const float pj = fast_exp2(zin - l2);
+                    const float dz = pj * (pacc[j >> 2][j & 3] - dl);
+                    if (HAS_BIAS) dbacc[qb][j] += dz;
+                    p8[j] = (E)pj;
+                    z8[j] = (E)dz;
+                }
+                st8<V8>(dZbuf + key * kRow + 8 * g, z8);
+#pragma unroll
+                for (int dt = 0; dt < 2; dt++) {
+                    const int off = (q8 + (l16 >> 2)) * kRow + 16 * dt + 4 * (l16 & 3);
+                    const V8 a_do = lds_tr8<DT>(dOs + off, dOs + off + 4 * kRow);
+                    dvacc[dt] = Elem<DT>::mfma16(a_do, p8, dvacc[dt]);
+                    const V8 a_q = lds_tr8<DT>(Qs + off, Qs + off + 4 * kRow);
+                    dkacc[dt] = Elem<DT>::mfma16(a_q, z8, dkacc[dt]);
+                }
+                __syncthreads();
+                // ---- phase B: dQ_hat^T tile (dt, qt), a share of the key steps ----
+                if (wave < 4 * ngroups) {
+                    const int dt = wave & 1, qt = (wave >> 1) & 1;
+                    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+                    for (int ks = wave >> 2; ks < nks; ks += ngroups) {
+                        const int rowk = (32 * ks + 8 * g + (l16 >> 2)) * kRow;
+                        const int ca = rowk + 16 * dt + 4 * (l16 & 3);
+                        const int cb = rowk + 16 * qt + 4 * (l16 & 3);
+                        const V8 a_k = lds_tr8<DT>(Ks + ca, Ks + ca + 4 * kRow);
+                        const V8 b_z = lds_tr8<DT>(dZbuf + cb, dZbuf + cb + 4 * kRow);
+                        acc = Elem<DT>::mfma16(a_k, b_z, acc);
+                    }
+                    float* dst = dQacc + (32 * qb + 16 * qt + l16) * kAccRow + 16 * dt + 4 * g;
+#pragma unroll
+                    for (int i = 0; i < 4; i++) atomicAdd(dst + i, acc[i]);
+                }
+            }
+        }
+        __syncthreads();
+        // ---- epilogue dq: back through q / max(|q|, eps) ----
+        for (int r = tid >> 2; r < N; r += nthreads >> 2) {
+            const int dc = (tid & 3) * 8;
+            float x[8], a[8];
+            unpack8b(ld8<V8>(qptr + (int64_t)r * p.q.sn + dc), x);
+            float ss = 0.f, dot = 0.f;
+#pragma unroll
+            for (int j = 0; j < 8; j++) { a[j] = dQacc[r * kAccRow + dc + j]; ss += x[j] * x[j]; }
+            ss = quad_add(ss);
+            const float nrm = sqrtf(ss);
+            const float inv = 1.0f / fmaxf(nrm, kNormEps);
+#pragma unroll
+            for (int j = 0; j < 8; j++) { x[j] *= inv; dot += a[j] * x[j]; }
+            dot = quad_add(dot);
+            const float proj = nrm > kNormEps ? dot : 0.f;
+            const float f = s_true * inv;
+            V8 out;
+#pragma unroll
+            for (int j = 0; j < 8; j++) out[j] = (E)(f * (a[j] - x[j] * proj));
+            st8<V8>(reinterpret_cast<E*>(const_cast<void*>(p.dq.ptr)) + b * p.dq.sb + h * p.dq.sh + (int64_t)r * p.dq.sn + dc, out);
+            if ((tid & 3) == 0) ds_part += dot;
+        }
+        // ---- epilogue dk, dv: lane (key, g) holds d = 16dt + 4g + i ----
+        if (key_ok) {
+            E* dvp = reinterpret_cast<E*>(const_cast<void*>(p.dv.ptr)) + b * p.dv.sb + h * p.dv.sh + (int64_t)key * p.dv.sn;
+#pragma unroll
+            for (int dt = 0; dt < 2; dt++) {
+                V4 o4;
+#pragma unroll
+                for (int i = 0; i < 4; i++) o4[i] = (E)dvacc[dt][i];
+                *reinterpret_cast<V4*>(dvp + 16 * dt + 4 * g) = o4;
+            }
+        }
+        {
+            float x[8], a[8];
+            float ss = 0.f, dot = 0.f;
+#pragma unroll
+            for (int dt = 0; dt < 2; dt++) {
+                V4 k4;
+#pragma unroll
+                for (int i = 0; i < 4; i++) k4[i] = 0;
+                if (key_ok) k4 = *reinterpret_cast<const V4*>(kptr + (int64_t)key * p.k.sn + 16 * dt + 4 * g);
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    x[4 * dt + i] = (float)k4[i];
+                    a[4 * dt + i] = dkacc[dt][i] * kLn2;      // undo the log2e folded into Q_hat
+                    ss += x[4 * dt + i] * x[4 * dt + i];
+                }
+            }
+            ss = xor32_add(xor16_add(ss));
+            const float nrm = sqrtf(ss);
+            const float inv = 1.0f / fmaxf(nrm, kNormEps);
+#pragma unroll
+            for (int j = 0; j < 8; j++) { x[j] *= inv; dot += a[j] * x[j]; }
+            dot = xor32_add(xor16_add(dot));
+            const float proj = nrm > kNormEps ? dot : 0.f;
+            if (key_ok) {
+                E* dkp = reinterpret_cast<E*>(const_cast<void*>(p.dk.ptr)) + b * p.dk.sb + h * p.dk.sh + (int64_t)key * p.dk.sn;
+#pragma unroll
+                for (int dt = 0; dt < 2; dt++) {
+                    V4 o4;
+#pragma unroll
+                    for (int i = 0; i < 4; i++) o4[i] = (E)(inv * (a[4 * dt + i] - x[4 * dt + i] * proj));
+                    *reinterpret_cast<V4*>(dkp + 16 * dt + 4 * g) = o4;
+                }
+            }
+        }
+    }
+
+    // ---- flush the per-workgroup partial sums ----
+    if (HAS_BIAS) {
+        float* dst = p.part_dbias + (((int64_t)h * p.groups + grp) * NPk + key) * R;
+#pragma unroll
+        for (int qb = 0; qb < NQB; qb++) {
+            if (qb < nqb) {
+                f32x4 a, c;
+#pragma unroll
+                for (int j = 0; j < 4; j++) { a[j] = dbacc[qb][j]; c[j] = dbacc[qb][4 + j]; }
+                *reinterpret_cast<f32x4*>(dst + 32 * qb + 8 * g) = a;
+                *reinterpret_cast<f32x4*>(dst + 32 * qb + 8 * g + 4) = c;
+            }
+        }
+    }
+    if (p.scale_kind == FWA2_SCALE_TENSOR) {
+        const float wsum = wave_sum(ds_part);
+        __syncthreads();
+        if (lane == 0) red[wave] = wsum;
+        __syncthreads();
+        if (tid == 0) {
+            float tot = 0.f;
+            for (int w = 0; w < p.waves; w++) tot += red[w];
+            p.part_dscale[h * p.groups + grp] = tot * s_true;
+        }
+    }
+}
+
+// bias [H,N,N] / mask [nW,N,N] (query-major) -> key-major, zero padded to [*, NPk, R].
+template <class T>
+__global__ void __launch_bounds__(256) transpose_pad_kernel(const T* src, int64_t sa, int64_t sn, int n, int npk, int r,
+                                                            const uint8_t* live, T* dst) {
+    __shared__ T tile[32][33];
+    const int a = blockIdx.z;
+    if (live && !live[a]) return;
+    const int q0 = blockIdx.x * 32, k0 = blockIdx.y * 32;
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+    for (int i = ty; i < 32; i += 8) {
+        const int q = q0 + i, k = k0 + tx;
+        tile[i][tx] = (q < n && k < n) ? src[a * sa + (int64_t)q * sn + k] : (T)0.f;
+    }
+    __syncthreads();
+    for (int i = ty; i < 32; i += 8) {
+        const int k = k0 + i, q = q0 + tx;
+        if (k < npk && q < r) dst[((int64_t)a * npk + k) * r + q] = tile[tx][i];
+    }
+}
+
+// dbias[h][q][k] = sum_g part[h][g][k][q]; dscale[h] = gate * sum_g part_dscale[h][g].
+template <int DT>
+__global__ void __launch_bounds__(256) reduce_kernel(const BwdParams p, int npk, int r, bool has_bias) {
+    typedef typename Elem<DT>::E E;
+    __shared__ float tile[8][33];
+    const int h = blockIdx.z;
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+    if (has_bias) {
+        const int q0 = blockIdx.x * 32, k0 = blockIdx.y * 8;
+        float acc = 0.f;
+        if (k0 + ty < npk) {
+            const float* src = p.part_dbias + (((int64_t)h * p.groups) * npk + k0 + ty) * r + q0 + tx;
+            const int64_t gs = (int64_t)npk * r;
+#pragma unroll 4
+            for (int gi = 0; gi < p.groups; gi++) acc += src[gi * gs];
+        }
+        tile[ty][tx] = acc;
+        __syncthreads();
+        // thread (ty, tx) -> query q0 + (4*ty + tx/8), key k0 + tx%8
+        const int qq = 4 * ty + (tx >> 3), kk = tx & 7;
+        const int q = q0 + qq, k = k0 + kk;
+        if (q < p.n && k < p.n) reinterpret_cast<E*>(p.dbias)[((int64_t)h * p.n + q) * p.n + k] = (E)tile[kk][qq];
+    }
+    if (p.scale_kind == FWA2_SCALE_TENSOR && blockIdx.x == 0 && blockIdx.y == 0) {
+        float v = 0.f;
+        for (int gi = threadIdx.x; gi < p.groups; gi += 256) v += p.part_dscale[h * p.groups + gi];
+        __shared__ float red[256];
+        red[threadIdx.x] = v;
+        __syncthreads();
+        for (int sft = 128; sft > 0; sft >>= 1) {
+            if (threadIdx.x < sft) red[threadIdx.x] += red[threadIdx.x + sft];
+            __syncthreads();
+        }
+        if (threadIdx.x == 0) {
+            const float ls = (float)reinterpret_cast<const E*>(p.logit_scale)[h];
+            reinterpret_cast<E*>(p.dscale)[h] = (E)(ls <= kLn100 ? red[0] : 0.f);
+        }
+    }
+}
+
+// ---- host side -----------------------------------------------------------------
+static size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
+
+int backward_supported(int n) { return n >= 1 && n <= 256; }
+
+struct BwdPlan {
+    int waves, groups, npk, r, nqb_t;
+    size_t off_dbias, off_dscale, off_bias_t, off_mask_t, total;
+    size_t smem;
+};
+
+static BwdPlan make_plan(int heads, int n, int bw, bool has_bias, bool has_mask, int n_windows, int cus) {
+    BwdPlan pl;
+    pl.waves = (n + 15) / 16;
+    pl.npk = pl.waves * 16;
+    pl.r = (n + 31) & ~31;
+    const int nqb = pl.r / 32;
+    pl.nqb_t = nqb <= 2 ? 2 : (nqb <= 4 ? 4 : 8);
+    // registers allow 16 wavefronts per CU: as many workgroups as fit
+    const int wg_per_cu = pl.waves <= 4 ? 4 : (pl.waves <= 8 ? 2 : 1);
+    int groups = (cus * wg_per_cu) / heads;
+    if (groups < 1) groups = 1;
+    if (groups > bw) groups = bw;
+    pl.groups = groups;
+    size_t off = 0;
+    pl.off_dbias = off;
+    if (has_bias) off += align256((size_t)heads * groups * pl.npk * pl.r * 4);
+    pl.off_dscale = off;
+    off += align256((size_t)heads * groups * 4);
+    pl.off_bias_t = off;
+    if (has_bias) off += align256((size_t)heads * pl.npk * pl.r * 2);
+    pl.off_mask_t = off;
+    if (has_mask) off += align256((size_t)n_windows * pl.npk * pl.r * 4);
+    pl.total = off;
+    pl.smem = (size_t)5 * pl.r * kRow * 2 + (size_t)pl.r * kAccRow * 4 + (size_t)2 * pl.r * 4 + 16 * 4;
+    return pl;
+}
+
+size_t backward_workspace_bytes(int heads, int n, int bw, bool has_bias, bool has_mask, int n_windows, int cus) {
+    if (!backward_supported(n)) return 0;
+    return make_plan(heads, n, bw, has_bias, has_mask, n_windows, cus).total;
+}
+
+template <int DT, bool HAS_BIAS, int MASK_DT, int NQB>
+static hipError_t launch_main(const BwdParams& p, const BwdPlan& pl, hipStream_t st) {
+    auto kern = bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB>;
+    if (pl.smem > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)pl.smem);
+        if (e != hipSuccess) return e;
+    }
+    hipLaunchKernelGGL(kern, dim3(p.heads * pl.groups), dim3(64 * pl.waves), pl.smem, st, p);
+    return hipGetLastError();
+}
+
+template <int DT, bool HAS_BIAS, int MASK_DT>
+static hipError_t launch_nqb(const BwdParams& p, const BwdPlan& pl, hipStream_t st) {
+    if (pl.nqb_t == 2) return launch_main<DT, HAS_BIAS, MASK_DT, 2>(p, pl, st);
+    if (pl.nqb_t == 4) return launch_main<DT, HAS_BIAS, MASK_DT, 4>(p, pl, st);
+    return launch_main<DT, HAS_BIAS, MASK_DT, 8>(p, pl, st);
+}
+
+template <int DT>
+static hipError_t launch_bwd_dt(BwdParams p, bool has_bias, int mask_dt, hipStream_t st) {
+    typedef typename Elem<DT>::E E;
+    const BwdPlan pl = make_plan(p.heads, p.n, p.bw, has_bias, mask_dt >= 0, p.n_windows, p.cus);
+    unsigned char* ws = reinterpret_cast<unsigned char*>(p.workspace);
+    p.waves = pl.waves;
+    p.groups = pl.groups;
+    p.part_dbias = reinterpret_cast<float*>(ws + pl.off_dbias);
+    p.part_dscale = reinterpret_cast<float*>(ws + pl.off_dscale);
+    p.bias_t = ws + pl.off_bias_t;
+    p.mask_t = ws + pl.off_mask_t;
+    const dim3 tgrid(pl.r / 32, (pl.npk + 31) / 32, 1);
+    if (has_bias) {
+        dim3 gr(tgrid.x, tgrid.y, p.heads);
+        hipLaunchKernelGGL(transpose_pad_kernel<E>, gr, dim3(256), 0, st, reinterpret_cast<const E*>(p.bias), p.bias_sh,
+                           p.bias_sn, p.n, pl.npk, pl.r, (const uint8_t*)nullptr,
+                           reinterpret_cast<E*>(const_cast<void*>(p.bias_t)));
+    }
+    if (mask_dt >= 0) {
+        dim3 gr(tgrid.x, tgrid.y, p.n_windows);
+        if (mask_dt == FWA2_F32)
+            hipLaunchKernelGGL(transpose_pad_kernel<float>, gr, dim3(256), 0, st, reinterpret_cast<const float*>(p.mask),
+                               p.mask_sw, p.mask_sn, p.n, pl.npk, pl.r, p.mask_live,
+                               reinterpret_cast<float*>(const_cast<void*>(p.mask_t)));
+        else
+            hipLaunchKernelGGL(transpose_pad_kernel<E>, gr, dim3(256), 0, st, reinterpret_cast<const E*>(p.mask),
+                               p.mask_sw, p.mask_sn, p.n, pl.npk, pl.r, p.mask_live,
+                               reinterpret_cast<E*>(const_cast<void*>(p.mask_t)));
+    }
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    if (has_bias) {
+        if (mask_dt < 0) e = launch_nqb<DT, true, -1>(p, pl, st);
+        else if (mask_dt == FWA2_F32) e = launch_nqb<DT, true, FWA2_F32>(p, pl, st);
+        else e = launch_nqb<DT, true, DT>(p, pl, st);
+    } else {
+        if (mask_dt < 0) e = launch_nqb<DT, false, -1>(p, pl, st);
+        else if (mask_dt == FWA2_F32) e = launch_nqb<DT, false, FWA2_F32>(p, pl, st);
+        else e = launch_nqb<DT, false, DT>(p, pl, st);
+    }
+    if (e != hipSuccess) return e;
+    if (has_bias || p.scale_kind == FWA2_SCALE_TENSOR) {
+        dim3 gr(has_bias ? pl.r / 32 : 1, has_bias ? (pl.npk + 7) / 8 : 1, p.heads);
+        hipLaunchKernelGGL(reduce_kernel<DT>, gr, dim3(256), 0, st, p, pl.npk, pl.r, has_bias);
+        e = hipGetLastError();
+    }
+    return e;
+}
+
+hipError_t launch_backward(const BwdParams& p, int dtype, bool has_bias, int mask_dt, hipStream_t st) {
+    if (dtype == FWA2_BF16) return launch_bwd_dt<FWA2_BF16>(p, has_bias, mask_dt, st);
+    return launch_bwd_dt<FWA2_F16>(p, has_bias, mask_dt, st);
+}
+
+}  // namespace fwa2

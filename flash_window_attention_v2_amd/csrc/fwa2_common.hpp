@@ -1,0 +1,174 @@
+// Shared device helpers for the gfx950 window-attention kernels: vector types,
+// MFMA wrappers for bf16 / fp16, cross-lane reductions on 64-wide wavefronts,
+// LDS transpose reads and the launch-side parameter block.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/fwa2.h"
+
+namespace fwa2 {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+constexpr float kLn100 = 4.605170185988092f;
+constexpr float kNormEps = 1e-12f;
+
+// Element-type traits: E = storage element, V8 / V4 = 8- and 4-wide vectors.
+template <int DT> struct Elem;
+template <> struct Elem<FWA2_BF16> {
+    typedef __bf16 E;
+    typedef bf16x8 V8;
+    typedef bf16x4 V4;
+    static __device__ __forceinline__ f32x16 mfma32(V8 a, V8 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ f32x4 mfma16(V8 a, V8 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ V4 lds_tr(const E* p) {
+        return __builtin_bit_cast(V4, __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                                          (__attribute__((address_space(3))) s16x4*)(p)));
+    }
+};
+template <> struct Elem<FWA2_F16> {
+    typedef _Float16 E;
+    typedef f16x8 V8;
+    typedef f16x4 V4;
+    static __device__ __forceinline__ f32x16 mfma32(V8 a, V8 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ f32x4 mfma16(V8 a, V8 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ V4 lds_tr(const E* p) {
+        return __builtin_bit_cast(V4, __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                                          (__attribute__((address_space(3))) s16x4*)(p)));
+    }
+};
+
+// 16-byte global / LDS accesses of 8 elements.
+template <class V8, class E>
+__device__ __forceinline__ V8 ld8(const E* p) { return *reinterpret_cast<const V8*>(p); }
+template <class V8, class E>
+__device__ __forceinline__ void st8(E* p, V8 v) { *reinterpret_cast<V8*>(p) = v; }
+
+template <class V8>
+__device__ __forceinline__ V8 zero8() {
+    V8 z;
+#pragma unroll
+    for (int j = 0; j < 8; j++) z[j] = 0;
+    return z;
+}
+
+// Two transposing LDS reads glued into one 8-element MFMA operand.
+template <int DT>
+__device__ __forceinline__ typename Elem<DT>::V8 lds_tr8(const typename Elem<DT>::E* lo,
+                                                         const typename Elem<DT>::E* hi) {
+    typename Elem<DT>::V4 a = Elem<DT>::lds_tr(lo);
+    typename Elem<DT>::V4 b = Elem<DT>::lds_tr(hi);
+    typename Elem<DT>::V8 r;
+#pragma unroll
+    for (int j = 0; j < 4; j++) { r[j] = a[j]; r[4 + j] = b[j]; }
+    return r;
+}
+
+// ---- cross-lane helpers (wave64) -------------------------------------------
+// Value held by the lane 32 away, combined with the own value by max / add.
+__device__ __forceinline__ float xor32_max(float x) {
+    u32x2 r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float xor32_add(float x) {
+    u32x2 r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float xor16_add(float x) {
+    u32x2 r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+// Sum over the 4 lanes of an aligned quad (DPP quad_perm, no LDS traffic).
+__device__ __forceinline__ float quad_add(float x) {
+    float y = __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(x), 0xB1, 0xF, 0xF, true));
+    x += y;   // lanes (0,1) (2,3) paired
+    y = __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(x), 0x4E, 0xF, 0xF, true));
+    return x + y;
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+__device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+
+// 1 / max(||x||, eps) from a sum of squares (torch.nn.functional.normalize).
+__device__ __forceinline__ float inv_norm(float sumsq) {
+    return 1.0f / fmaxf(sqrtf(sumsq), kNormEps);
+}
+
+// Row r of a 32-row MFMA A operand <-> position inside a 32-key tile such that
+// the 8 accumulator registers a lane feeds to the next MFMA as its k-slots are
+// 8 consecutive positions: swap bits 2 and 3 of r.
+__host__ __device__ constexpr int swap_bits23(int r) {
+    return (r & ~12) | ((r & 4) << 1) | ((r & 8) >> 1);
+}
+
+// ---- launch parameters -------------------------------------------------------
+struct T4 {
+    const void* ptr;
+    int64_t sb, sh, sn;
+};
+struct FwdParams {
+    T4 q, k, v, o;
+    const void* logit_scale;
+    const void* bias;
+    int64_t bias_sh, bias_sn;
+    const void* mask;
+    int64_t mask_sw, mask_sn;
+    const uint8_t* mask_live;  // [n_windows] 1 = window's mask has a non-zero entry; nullptr = assume all live
+    float* lse;
+    int64_t lse_sb, lse_sh;
+    int bw, heads, n, n_windows;
+    int scale_kind;
+    float default_scale;  // 1/sqrt(head_dim), used when no logit scale is given
+    bool bias_vec, mask_vec;  // rows of bias / mask may be read with 16-byte loads
+    int waves;        // wavefronts per workgroup
+    int q_chunks;     // workgroups per (bw, head)
+};
+
+struct BwdParams {
+    T4 q, k, v, o, d_o, dq, dk, dv;
+    const void* logit_scale;
+    const void* bias;
+    int64_t bias_sh, bias_sn;
+    const void* mask;
+    int64_t mask_sw, mask_sn;
+    const uint8_t* mask_live;
+    const float* lse;
+    int64_t lse_sb, lse_sh;
+    int bw, heads, n, n_windows;
+    int scale_kind;
+    float default_scale;
+    void* dbias;      // [H, N, N] in the input dtype
+    void* dscale;     // [H] in the input dtype
+    void* workspace;
+    int cus;          // compute units of the device
+    // filled in by the launcher
+    int waves;        // wavefronts per workgroup = key tiles of 16
+    int groups;       // workgroups per head (each walks bw = g, g + groups, ...)
+    float* part_dbias;   // [H, groups, NP, NQ] fp32, key-major
+    float* part_dscale;  // [H, groups] fp32
+    const void* bias_t;  // [H, NP, NQ] input dtype: bias transposed to key-major, zero padded
+    const void* mask_t;  // [nW, NP, NQ] mask dtype: mask transposed to key-major, zero padded
+};
+
+}  // namespace fwa2

@@ -1,0 +1,328 @@
+// Forward kernel: o, lse = softmax(s * q_hat k_hat^T + bias + mask) v  for gfx950.
+//
+// Replaces the Triton kernel _fwd_kernel of the reference
+// (flash_win_attn_v2/kernels/attn_kernel_forward.py:33-258).
+//
+// Work split.  One workgroup owns one (batch*window, head) pair and a chunk of
+// up to 32*waves query rows; each wavefront owns 32 query rows and walks over
+// all keys in blocks of 64.  K (L2-normalised, in the input dtype) and V are
+// staged once per workgroup in LDS, 256 keys at a time.
+//
+// Matrix shapes.  Scores are computed transposed, S^T = K_hat Q_hat^T, with
+// v_mfma_f32_32x32x16: rows = keys, columns = queries.  A lane then holds, for
+// ONE query (column lane%32), the scores of 16 keys of the tile in its
+// accumulator registers, so the softmax row reductions are in-lane plus one
+// exchange with the lane 32 away, and the exponentiated accumulators are
+// directly the B operand (k = keys) of the second MFMA O^T = V^T P^T.  The rows
+// of each 32-key tile are permuted (swap_bits23) so that the 8 registers fed
+// to one MFMA are 8 consecutive keys; V^T comes out of row-major V in LDS with
+// ds_read_b64_tr_b16.
+//
+// Numerics.  Scores live in the log2 domain: q_hat is multiplied by
+// s * log2(e) in fp32 before it is rounded to the input dtype, bias and mask
+// are multiplied by log2(e) in fp32, exp is v_exp_f32 (2^x).  Softmax state,
+// accumulators and the log-sum-exp are fp32; P is rounded to the input dtype
+// for the second MFMA (as the reference does, attn_kernel_forward.py:225-226).
+#include "fwa2_common.hpp"
+
+namespace fwa2 {
+
+constexpr int kKeyChunk = 256;   // keys staged in LDS at a time
+constexpr int kLdsStride = 40;   // elements per staged row (32 + 8 pad): 80-byte rows
+
+template <class V8>
+__device__ __forceinline__ void unpack8(V8 v, float* x) {
+#pragma unroll
+    for (int j = 0; j < 8; j++) x[j] = (float)v[j];
+}
+
+// 8 consecutive elements starting at column c0 of one row of bias / mask, as
+// floats; columns >= n read as `fill`.  `vec` says 16-byte loads are legal.
+template <class E>
+__device__ __forceinline__ void load_row8(const E* row, int c0, int n, bool vec, float fill, float* x) {
+    typedef E V8 __attribute__((ext_vector_type(8)));
+    if (vec && c0 + 8 <= n) {
+        V8 v = *reinterpret_cast<const V8*>(row + c0);
+#pragma unroll
+        for (int j = 0; j < 8; j++) x[j] = (float)v[j];
+    } else {
+#pragma unroll
+        for (int j = 0; j < 8; j++) x[j] = (c0 + j < n) ? (float)row[c0 + j] : fill;
+    }
+}
+
+// Element type of the mask: the input dtype, or float for an fp32 mask.
+template <int DT, int MASK_DT> struct MaskElem { typedef typename Elem<DT>::E E; };
+template <int DT> struct MaskElem<DT, FWA2_F32> { typedef float E; };
+
+template <int DT, bool HAS_BIAS, int MASK_DT>
+__global__ void __launch_bounds__(512) fwd_kernel(const FwdParams p) {
+    typedef typename Elem<DT>::E E;
+    typedef typename Elem<DT>::V8 V8;
+    typedef typename Elem<DT>::V4 V4;
+    typedef typename MaskElem<DT, MASK_DT>::E ME;
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    const int N = p.n;
+    const int chunk_rows = (min(N, kKeyChunk) + 63) & ~63;
+    E* Ks = reinterpret_cast<E*>(smem_raw);
+    E* Vs = Ks + chunk_rows * kLdsStride;
+
+    const int tid = threadIdx.x;
+    const int nthreads = blockDim.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int col = lane & 31;       // query column of this lane
+    const int hf = lane >> 5;        // which half of the k-slots / rows
+    const int li = lane & 15;        // lane inside its 16-lane block (transpose reads)
+    const int blk1 = (lane >> 4) & 1;
+
+    int idx = blockIdx.x;
+    const int qc = idx % p.q_chunks;
+    idx /= p.q_chunks;
+    const int h = idx % p.heads;
+    const int b = idx / p.heads;
+
+    const E* qptr = reinterpret_cast<const E*>(p.q.ptr) + b * p.q.sb + h * p.q.sh;
+    const E* kptr = reinterpret_cast<const E*>(p.k.ptr) + b * p.k.sb + h * p.k.sh;
+    const E* vptr = reinterpret_cast<const E*>(p.v.ptr) + b * p.v.sb + h * p.v.sh;
+    E* optr = reinterpret_cast<E*>(const_cast<void*>(p.o.ptr)) + b * p.o.sb + h * p.o.sh;
+
+    float scale2;
+    if (p.scale_kind == FWA2_SCALE_TENSOR) {
+        float ls = (float)reinterpret_cast<const E*>(p.logit_scale)[h];
+        scale2 = expf(fminf(ls, kLn100)) * kLog2e;
+    } else {
+        scale2 = p.default_scale * kLog2e;
+    }
+
+    const int q0 = (qc * p.waves + wave) * 32;
+    const int qi = q0 + col;
+    const bool qv = qi < N;
+    const bool wave_live = q0 < N;
+
+    // ---- Q operand: normalise, fold the scale, round to the input dtype ----
+    V8 bq0 = zero8<V8>(), bq1 = zero8<V8>();
+    if (wave_live) {
+        V8 a = zero8<V8>(), c = zero8<V8>();
+        if (qv) {
+            a = ld8<V8>(qptr + qi * p.q.sn + 8 * hf);
+            c = ld8<V8>(qptr + qi * p.q.sn + 16 + 8 * hf);
+        }
+        float xa[8], xc[8];
+        unpack8(a, xa);
+        unpack8(c, xc);
+        float ss = 0.f;
+#pragma unroll
+        for (int j = 0; j < 8; j++) ss += xa[j] * xa[j] + xc[j] * xc[j];
+        ss = xor32_add(ss);
+        const float sc = scale2 * inv_norm(ss);
+#pragma unroll
+        for (int j = 0; j < 8; j++) { bq0[j] = (E)(xa[j] * sc); bq1[j] = (E)(xc[j] * sc); }
+    }
+
+    const E* bias_row = nullptr;
+    if (HAS_BIAS) bias_row = reinterpret_cast<const E*>(p.bias) + h * p.bias_sh + (int64_t)min(qi, N - 1) * p.bias_sn;
+    const ME* mask_row = nullptr;
+    bool mask_on = false;
+    if (MASK_DT >= 0) {
+        const int w = b % p.n_windows;
+        mask_on = p.mask_live ? (p.mask_live[w] != 0) : true;
+        mask_row = reinterpret_cast<const ME*>(p.mask) + w * p.mask_sw + (int64_t)min(qi, N - 1) * p.mask_sn;
+    }
+
+    float m_run = -INFINITY;   // running row max (log2 domain)
+    float l_run = 0.f;         // this lane's share of the running row sum
+    f32x16 oacc;
+#pragma unroll
+    for (int i = 0; i < 16; i++) oacc[i] = 0.f;
+
+    for (int c0 = 0; c0 < N; c0 += kKeyChunk) {
+        const int rows = min(N - c0, kKeyChunk);
+        const int rows_pad = (rows + 63) & ~63;
+        if (c0 > 0) __syncthreads();
+        // ---- stage K_hat and V rows c0 .. c0+rows_pad of this (b, h) ----
+        for (int r = tid >> 2; r < rows_pad; r += nthreads >> 2) {
+            const int dch = (tid & 3) * 8;
+            V8 kk = zero8<V8>(), vv = zero8<V8>();
+            if (r < rows) {
+                kk = ld8<V8>(kptr + (int64_t)(c0 + r) * p.k.sn + dch);
+                vv = ld8<V8>(vptr + (int64_t)(c0 + r) * p.v.sn + dch);
+            }
+            float x[8];
+            unpack8(kk, x);
+            float ss = 0.f;
+#pragma unroll
+            for (int j = 0; j < 8; j++) ss += x[j] * x[j];
+            ss = quad_add(ss);
+            const float inv = inv_norm(ss);
+            V8 kn;
+#pragma unroll
+            for (int j = 0; j < 8; j++) kn[j] = (E)(x[j] * inv);
+            st8<V8>(Ks + r * kLdsStride + dch, kn);
+            st8<V8>(Vs + r * kLdsStride + dch, vv);
+        }
+        __syncthreads();
+        if (!wave_live) continue;
+
+        const int nblk = rows_pad >> 6;
+        for (int kb = 0; kb < nblk; kb++) {
+            // ---- S^T tiles: 2 x (32 keys x 32 queries) ----
+            f32x16 acc[2];
+#pragma unroll
+            for (int t = 0; t < 2; t++) {
+                const E* krow = Ks + (kb * 64 + 32 * t + swap_bits23(col)) * kLdsStride + 8 * hf;
+                V8 a0 = ld8<V8>(krow);
+                V8 a1 = ld8<V8>(krow + 16);
+                f32x16 z;
+#pragma unroll
+                for (int i = 0; i < 16; i++) z[i] = 0.f;
+                z = Elem<DT>::mfma32(a0, bq0, z);
+                acc[t] = Elem<DT>::mfma32(a1, bq1, z);
+            }
+            // register i of tile t <-> key kbase + 32t + 16(i/8) + 8hf + i%8
+            const int kbase = c0 + kb * 64;
+            if (HAS_BIAS) {
+#pragma unroll
+                for (int t = 0; t < 2; t++)
+#pragma unroll
+                    for (int u = 0; u < 2; u++) {
+                        float x[8];
+                        load_row8<E>(bias_row, kbase + 32 * t + 16 * u + 8 * hf, N, p.bias_vec, 0.f, x);
+#pragma unroll
+                        for (int j = 0; j < 8; j++) acc[t][8 * u + j] = fmaf(x[j], kLog2e, acc[t][8 * u + j]);
+                    }
+            }
+            if (MASK_DT >= 0) {
+                if (mask_on) {
+#pragma unroll
+                    for (int t = 0; t < 2; t++)
+#pragma unroll
+                        for (int u = 0; u < 2; u++) {
+                            float x[8];
+                            load_row8<ME>(mask_row, kbase + 32 * t + 16 * u + 8 * hf, N, p.mask_vec, 0.f, x);
+#pragma unroll
+                            for (int j = 0; j < 8; j++) acc[t][8 * u + j] = fmaf(x[j], kLog2e, acc[t][8 * u + j]);
+                        }
+                }
+            }
+            if (kbase + 64 > N) {   // padded key columns never take part
+#pragma unroll
+                for (int t = 0; t < 2; t++)
+#pragma unroll
+                    for (int i = 0; i < 16; i++) {
+                        const int key = kbase + 32 * t + 16 * (i >> 3) + 8 * hf + (i & 7);
+                        if (key >= N) acc[t][i] = -INFINITY;
+                    }
+            }
+            // ---- online softmax over this 64-key block ----
+            float bm = acc[0][0];
+#pragma unroll
+            for (int i = 1; i < 16; i++) bm = fmaxf(bm, acc[0][i]);
+#pragma unroll
+            for (int i = 0; i < 16; i++) bm = fmaxf(bm, acc[1][i]);
+            bm = xor32_max(bm);
+            const float m_new = fmaxf(m_run, bm);
+            const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+            const float alpha = fast_exp2(m_run - m_use);
+            m_run = m_new;
+            float psum = 0.f;
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    acc[t][i] = fast_exp2(acc[t][i] - m_use);
+                    psum += acc[t][i];
+                }
+            l_run = l_run * alpha + psum;
+#pragma unroll
+            for (int i = 0; i < 16; i++) oacc[i] *= alpha;
+            // ---- O^T += V^T P^T, 16 keys per MFMA ----
+#pragma unroll
+            for (int mm = 0; mm < 4; mm++) {
+                V8 bp;
+#pragma unroll
+                for (int j = 0; j < 8; j++) bp[j] = (E)acc[mm >> 1][8 * (mm & 1) + j];
+                const E* vlo = Vs + (kb * 64 + 16 * mm + 8 * hf + (li >> 2)) * kLdsStride + 16 * blk1 + 4 * (li & 3);
+                V8 av = lds_tr8<DT>(vlo, vlo + 4 * kLdsStride);
+                oacc = Elem<DT>::mfma32(av, bp, oacc);
+            }
+        }
+    }
+
+    if (!wave_live) return;
+    // ---- normalise, write o (input dtype) and lse (natural log, fp32) ----
+    const float l_tot = xor32_add(l_run);
+    const float inv_l = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+    if (qv) {
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            V4 ov;
+#pragma unroll
+            for (int j = 0; j < 4; j++) ov[j] = (E)(oacc[4 * c + j] * inv_l);
+            *reinterpret_cast<V4*>(optr + (int64_t)qi * p.o.sn + 8 * c + 4 * hf) = ov;
+        }
+        if (hf == 0) {
+            const float lse = l_tot > 0.f ? (m_run + fast_log2(l_tot)) * kLn2 : -INFINITY;
+            p.lse[b * p.lse_sb + h * p.lse_sh + qi] = lse;
+        }
+    }
+}
+
+// One byte per window: does the window's [N, N] mask hold any non-zero entry?
+template <class ME>
+__global__ void __launch_bounds__(256) mask_scan_kernel(const ME* mask, int64_t sw, int64_t sn, int n,
+                                                        uint8_t* live) {
+    const int w = blockIdx.x;
+    const ME* m = mask + w * sw;
+    int any = 0;
+    for (int i = threadIdx.x; i < n * n; i += blockDim.x) {
+        const int r = i / n, c = i - r * n;
+        any |= ((float)m[r * sn + c] != 0.f);
+    }
+    any = __syncthreads_or(any);
+    if (threadIdx.x == 0) live[w] = any ? 1 : 0;
+}
+
+template <int DT, bool HAS_BIAS, int MASK_DT>
+static hipError_t launch_one(const FwdParams& p, dim3 grid, dim3 block, size_t smem, hipStream_t st) {
+    hipLaunchKernelGGL((fwd_kernel<DT, HAS_BIAS, MASK_DT>), grid, block, smem, st, p);
+    return hipGetLastError();
+}
+
+template <int DT>
+static hipError_t launch_dt(const FwdParams& p, bool has_bias, int mask_dt, dim3 g, dim3 b, size_t s, hipStream_t st) {
+    if (has_bias) {
+        if (mask_dt < 0) return launch_one<DT, true, -1>(p, g, b, s, st);
+        if (mask_dt == FWA2_F32) return launch_one<DT, true, FWA2_F32>(p, g, b, s, st);
+        return launch_one<DT, true, DT>(p, g, b, s, st);
+    }
+    if (mask_dt < 0) return launch_one<DT, false, -1>(p, g, b, s, st);
+    if (mask_dt == FWA2_F32) return launch_one<DT, false, FWA2_F32>(p, g, b, s, st);
+    return launch_one<DT, false, DT>(p, g, b, s, st);
+}
+
+hipError_t launch_forward(FwdParams p, int dtype, bool has_bias, int mask_dt, hipStream_t st) {
+    const int q_tiles = (p.n + 31) / 32;
+    p.waves = q_tiles < 8 ? q_tiles : 8;
+    p.q_chunks = (q_tiles + p.waves - 1) / p.waves;
+    const int chunk_rows = ((p.n < kKeyChunk ? p.n : kKeyChunk) + 63) & ~63;
+    const size_t smem = (size_t)2 * chunk_rows * kLdsStride * 2;
+    dim3 grid((unsigned)((int64_t)p.bw * p.heads * p.q_chunks)), block(64 * p.waves);
+    if (dtype == FWA2_BF16) return launch_dt<FWA2_BF16>(p, has_bias, mask_dt, grid, block, smem, st);
+    return launch_dt<FWA2_F16>(p, has_bias, mask_dt, grid, block, smem, st);
+}
+
+hipError_t launch_mask_scan(const void* mask, int mask_dt, int64_t sw, int64_t sn, int n, int n_windows,
+                            uint8_t* live, hipStream_t st) {
+    dim3 grid(n_windows), block(256);
+    if (mask_dt == FWA2_F32)
+        hipLaunchKernelGGL(mask_scan_kernel<float>, grid, block, 0, st, (const float*)mask, sw, sn, n, live);
+    else if (mask_dt == FWA2_BF16)
+        hipLaunchKernelGGL(mask_scan_kernel<__bf16>, grid, block, 0, st, (const __bf16*)mask, sw, sn, n, live);
+    else
+        hipLaunchKernelGGL(mask_scan_kernel<_Float16>, grid, block, 0, st, (const _Float16*)mask, sw, sn, n, live);
+    return hipGetLastError();
+}
+
+}  // namespace fwa2

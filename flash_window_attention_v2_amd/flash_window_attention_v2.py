@@ -1,0 +1,161 @@
+"""`FlashWindowAttentionV2`: the autograd Function of the reference
+(flash_win_attn_v2/flash_window_attention_v2.py:5-57) with the same
+signature, saved tensors and six-value backward, whose body marshals raw
+device pointers and strides to the gfx950 kernels in libfwa2.so.
+
+Every buffer -- outputs, log-sum-exp, gradients and the backward workspace --
+is a torch tensor allocated here, so torch's allocator statistics stay honest
+and the C side allocates nothing.
+"""
+import math
+
+import torch
+
+from . import _abi
+
+_DTYPES = {torch.float16: _abi.F16, torch.bfloat16: _abi.BF16, torch.float32: _abi.F32}
+
+
+def _t4(t):
+    return _abi.Tensor4(t.data_ptr(), t.stride(0), t.stride(1), t.stride(2))
+
+
+def _rows_16b_aligned(t):
+    return t.stride(-1) == 1 and t.data_ptr() % 16 == 0 and all(s % 8 == 0 for s in t.stride()[:-1])
+
+
+def _kernel_ready(t):
+    """Unit inner stride is the reference's requirement (flash_window_attention_v2.py:20);
+    16-byte-aligned rows are this library's: copy only when either fails."""
+    return t if _rows_16b_aligned(t) else t.contiguous()
+
+
+def mask_window_flags(mask):
+    """uint8[nW]: 1 where a window's mask has a non-zero entry (device tensor).
+    Cached on the mask tensor object and refreshed if the tensor is modified in place."""
+    cached = getattr(mask, "_fwa2_live", None)
+    if cached is not None and cached[0] == mask._version and cached[1].device == mask.device:
+        return cached[1]
+    lib = _abi.load()
+    live = torch.empty(mask.shape[0], dtype=torch.uint8, device=mask.device)
+    with torch.cuda.device(mask.device):
+        st = lib.fwa2_mask_scan(mask.data_ptr(), _DTYPES[mask.dtype], mask.shape[0], mask.shape[1], mask.stride(0),
+                                mask.stride(1), live.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    _abi.check(st, "fwa2_mask_scan")
+    try:
+        mask._fwa2_live = (mask._version, live)
+    except Exception:
+        pass
+    return live
+
+
+def _describe(q, k, v, o, lse, logit_scale, bias, mask, mask_live, scale_type):
+    bw, heads, n, d = q.shape
+    p = _abi.new_problem()
+    p.dtype = _DTYPES[q.dtype]
+    p.scale_kind = _abi.SCALE_TENSOR if scale_type == "tensor" else _abi.SCALE_DEFAULT
+    p.bw, p.heads, p.n, p.head_dim = bw, heads, n, d
+    p.n_windows = mask.shape[0] if mask is not None else 1
+    p.q, p.k, p.v, p.o = _t4(q), _t4(k), _t4(v), _t4(o)
+    if scale_type == "tensor":
+        p.logit_scale = logit_scale.data_ptr()
+    if bias is not None:
+        p.bias = _abi.Tensor3(bias.data_ptr(), bias.stride(0), bias.stride(1))
+    if mask is not None:
+        p.mask = _abi.Tensor3(mask.data_ptr(), mask.stride(0), mask.stride(1))
+        p.mask_dtype = _DTYPES[mask.dtype]
+        if mask_live is not None:
+            p.mask_live = mask_live.data_ptr()
+    else:
+        p.mask_dtype = p.dtype
+    p.lse = lse.data_ptr()
+    p.lse_stride_bw, p.lse_stride_h = lse.stride(0), lse.stride(1)
+    return p
+
+
+def _check_inputs(q, k, v, logit_scale, bias, mask, scale_type):
+    """The reference launcher's assertions (attn_kernel_forward.py:263-292)."""
+    bw, heads, n, d = q.shape
+    assert k.shape == (bw, heads, k.shape[2], d) and v.shape == k.shape, "q, k, v shapes do not match"
+    assert k.shape[2] == n, "this build requires as many keys as queries (every caller of the reference does)"
+    assert d <= 128, "FlashAttention only support head dimensions up to 128"
+    assert q.dtype == k.dtype == v.dtype, "All tensors must have the same type"
+    assert q.dtype in (torch.float16, torch.bfloat16), "Only support fp16 and bf16"
+    assert q.is_cuda and k.is_cuda and v.is_cuda, "q, k, v must be on the GPU"
+    if scale_type == "tensor":
+        assert logit_scale.is_cuda
+        assert logit_scale.shape == (heads, 1, 1)
+        assert logit_scale.dtype == q.dtype
+    if bias is not None:
+        assert bias.dtype == q.dtype
+        assert bias.is_cuda
+        assert bias.shape == (heads, n, n)
+    if mask is not None:
+        assert mask.dtype in (q.dtype, torch.float32)
+        assert mask.is_cuda
+        assert mask.dim() == 3 and mask.shape[1:] == (n, n) and bw % mask.shape[0] == 0, "mask must be [nW, N, N] with BW % nW == 0"
+
+
+class FlashWindowAttentionV2(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q, k, v, logit_scale=None, bias=None, mask=None):
+        if logit_scale is not None:
+            assert isinstance(logit_scale, torch.Tensor), \
+                "Make sure logit_scale is a tensor if defined in the paramaters."
+            scale_type = "tensor"
+            logit_scale = logit_scale if logit_scale.stride(-1) == 1 else logit_scale.contiguous()
+        else:
+            scale_type = "scalar"
+            logit_scale = torch.tensor(1.0 / math.sqrt(q.shape[-1]), device=q.device)
+
+        _check_inputs(q, k, v, logit_scale, bias, mask, scale_type)
+        q, k, v = (_kernel_ready(x) for x in (q, k, v))
+        if scale_type == "tensor" and not logit_scale.is_contiguous():
+            logit_scale = logit_scale.contiguous()
+        if bias is not None and bias.stride(-1) != 1:
+            bias = bias.contiguous()
+        if mask is not None and mask.stride(-1) != 1:
+            mask = mask.contiguous()
+
+        bw, heads, n, _ = q.shape
+        lib = _abi.load()
+        lse = torch.empty((bw, heads, (n + 63) // 64 * 64), device=q.device, dtype=torch.float32)
+        o = torch.empty_like(q)
+        if not _rows_16b_aligned(o):
+            o = torch.empty(q.shape, device=q.device, dtype=q.dtype)
+        mask_live = mask_window_flags(mask) if mask is not None else None
+        p = _describe(q, k, v, o, lse, logit_scale, bias, mask, mask_live, scale_type)
+        with torch.cuda.device(q.device):
+            p.stream = torch.cuda.current_stream().cuda_stream
+            _abi.check(lib.fwa2_forward(p), "fwa2_forward")
+
+        ctx.save_for_backward(q, k, v, o, lse, logit_scale, bias, mask)
+        ctx.scale_type = scale_type
+        ctx.mask_live = mask_live
+        return o
+
+    @staticmethod
+    def backward(ctx, do):
+        q, k, v, o, lse, logit_scale, bias, mask = ctx.saved_tensors
+        scale_type = ctx.scale_type
+        do = _kernel_ready(do)
+        dq, dk, dv = (torch.empty_like(x) for x in (q, k, v))
+        if not all(_rows_16b_aligned(x) for x in (dq, dk, dv)):
+            dq, dk, dv = (torch.empty(x.shape, device=x.device, dtype=x.dtype) for x in (q, k, v))
+        dscale = torch.empty_like(logit_scale, memory_format=torch.contiguous_format) if scale_type == "tensor" else None
+        db = torch.empty_like(bias, memory_format=torch.contiguous_format) if bias is not None else None
+
+        lib = _abi.load()
+        p = _describe(q, k, v, o, lse, logit_scale, bias, mask, ctx.mask_live, scale_type)
+        p.d_o, p.dq, p.dk, p.dv = _t4(do), _t4(dq), _t4(dk), _t4(dv)
+        if db is not None:
+            p.dbias = db.data_ptr()
+        if dscale is not None:
+            p.dscale = dscale.data_ptr()
+        with torch.cuda.device(q.device):
+            need = lib.fwa2_backward_workspace_bytes(p)
+            ws = torch.empty(max(need, 1), dtype=torch.uint8, device=q.device)
+            p.workspace, p.workspace_bytes = ws.data_ptr(), need
+            p.stream = torch.cuda.current_stream().cuda_stream
+            _abi.check(lib.fwa2_backward(p), "fwa2_backward")
+        return dq, dk, dv, dscale, db, None

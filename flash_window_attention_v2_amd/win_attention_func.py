@@ -1,0 +1,37 @@
+"""Operator entry points, named as in the reference
+(flash_win_attn_v2/win_attention_func.py): the fused gfx950 path and the
+classic materialised path that `WindowAttention(is_flash=False)` uses."""
+import math
+
+import torch
+import torch.nn.functional as F
+
+from .flash_window_attention_v2 import FlashWindowAttentionV2
+
+#: fused forward/backward: (q, k, v, logit_scale=None, bias=None, mask=None) -> o
+flash_win_attn_v2_func = FlashWindowAttentionV2.apply
+
+
+def win_attention_torch(q, k, v, logit_scale=None, bias=None, mask=None):
+    """Classic window attention with explicit [BW, H, N, N] scores, in the dtype of
+    its inputs (the operator selected by `is_flash=False`; it is a different,
+    slower operator chosen by the caller, never a substitute for the fused one).
+
+    q, k, v: [BW, H, N, d]; logit_scale: [H, 1, 1] or None; bias: [H, N, N] or
+    None; mask: [nW, N, N] or None with window index bw % nW.
+    """
+    bw, heads, n_q, d = q.shape
+    n_k = k.shape[2]
+    scores = F.normalize(q, p=2, dim=-1) @ F.normalize(k, p=2, dim=-1).transpose(-2, -1)
+    if logit_scale is None:
+        scores = scores * (1.0 / math.sqrt(d))
+    else:
+        limit = torch.log(torch.tensor(100.0, dtype=logit_scale.dtype, device=logit_scale.device))
+        scores = scores * logit_scale.clamp(max=limit).exp()
+    if bias is not None:
+        scores = scores + bias.unsqueeze(0)
+    if mask is not None:
+        n_w = mask.shape[0]
+        scores = scores.view(bw // n_w, n_w, heads, n_q, n_k) + mask.unsqueeze(1).unsqueeze(0)
+        scores = scores.view(bw, heads, n_q, n_k)
+    return torch.softmax(scores, dim=-1) @ v

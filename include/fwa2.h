@@ -1,0 +1,165 @@
+/*
+ * fwa2.h -- C ABI of libfwa2: Swin V2 scaled-cosine window attention,
+ * forward and backward, as hand-written HIP kernels for gfx950 (MI355X).
+ *
+ * The library replaces the two host launchers of the reference
+ * implementation and the Triton kernels behind them:
+ *
+ *   fwa2_forward   <->  _flash_attn_forward
+ *                       flash_win_attn_v2/kernels/attn_kernel_forward.py:261-345
+ *                       (kernel _fwd_kernel, :33-258)
+ *   fwa2_backward  <->  _flash_attn_backward
+ *                       flash_win_attn_v2/kernels/attn_kernel_backward.py:567-711
+ *                       (kernels _bwd_preprocess_do_o_dot :6-51, _bwd_kernel :389-564)
+ *
+ * Conventions
+ *   - plain pointers and sizes only; no framework types cross this boundary.
+ *   - the library allocates nothing and keeps no pointer after a call returns;
+ *     every buffer, including workspaces, belongs to the caller.
+ *   - every call only enqueues work on `stream` (a hipStream_t, NULL = the
+ *     default stream) and never synchronises the device.
+ *   - strides are in ELEMENTS of the tensor's own type; the innermost (head
+ *     dim) stride of q, k, v, o, do, dq, dk, dv is 1 and is not passed.  The
+ *     other three strides are free, as in the reference
+ *     (flash_window_attention_v2.py:20, attn_kernel_forward.py:313-328).
+ *   - all functions are re-entrant; the error string is thread-local.
+ *   - return value 0 = FWA2_OK, otherwise an fwa2_status; fwa2_last_error()
+ *     then describes the failure.
+ */
+#ifndef FWA2_H
+#define FWA2_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FWA2_ABI_VERSION 1
+
+typedef enum fwa2_status {
+    FWA2_OK = 0,
+    FWA2_ERR_INVALID_ARGUMENT = 1, /* contract violation (the reference's AssertionError) */
+    FWA2_ERR_UNSUPPORTED = 2,      /* legal for the reference, not built here (e.g. head dim != 32) */
+    FWA2_ERR_HIP = 3,              /* a HIP runtime call failed */
+    FWA2_ERR_NO_DEVICE = 4         /* no gfx950 device available for the launch */
+} fwa2_status;
+
+typedef enum fwa2_dtype {
+    FWA2_F16 = 0,
+    FWA2_BF16 = 1,
+    FWA2_F32 = 2 /* only valid as mask_dtype (attn_kernel_forward.py:287) */
+} fwa2_dtype;
+
+typedef enum fwa2_scale_kind {
+    FWA2_SCALE_DEFAULT = 0, /* no logit scale given: scores * 1/sqrt(d)  (flash_window_attention_v2.py:14-17) */
+    FWA2_SCALE_TENSOR = 1   /* logit_scale[H] given: scores * exp(min(l_h, ln 100)) (attn_kernel_forward.py:118-121) */
+} fwa2_scale_kind;
+
+/* A [BW, H, N, d] tensor with unit innermost stride. */
+typedef struct fwa2_tensor4 {
+    void*   ptr;
+    int64_t stride_bw;
+    int64_t stride_h;
+    int64_t stride_n;
+} fwa2_tensor4;
+
+/* A [A, N, N] tensor (bias: A = H, mask: A = nW) with unit innermost stride. */
+typedef struct fwa2_tensor3 {
+    void*   ptr;       /* NULL = absent */
+    int64_t stride_a;
+    int64_t stride_n;
+} fwa2_tensor3;
+
+/*
+ * One operator call.  The same description serves forward and backward; the
+ * fields marked (bwd) are ignored by fwa2_forward.
+ */
+typedef struct fwa2_problem {
+    uint32_t struct_bytes;   /* sizeof(fwa2_problem) as the caller compiled it */
+    uint32_t abi_version;    /* FWA2_ABI_VERSION */
+
+    int32_t dtype;           /* fwa2_dtype of q,k,v,o,do,dq,dk,dv,bias,logit_scale,dbias,dscale: F16 or BF16 */
+    int32_t mask_dtype;      /* fwa2_dtype of mask: == dtype or F32 */
+    int32_t scale_kind;      /* fwa2_scale_kind */
+    int32_t bw;              /* batch * windows-per-image */
+    int32_t heads;
+    int32_t n;               /* tokens per window (queries == keys) */
+    int32_t head_dim;
+    int32_t n_windows;       /* leading extent of mask; window of row b is b % n_windows; 1 if no mask */
+
+    fwa2_tensor4 q, k, v;    /* inputs */
+    fwa2_tensor4 o;          /* forward: output.  backward: the saved forward output */
+    const void*  logit_scale;/* [H] elements of `dtype`, stride 1; NULL unless FWA2_SCALE_TENSOR */
+    fwa2_tensor3 bias;       /* [H, N, N] of `dtype`, or ptr NULL */
+    fwa2_tensor3 mask;       /* [nW, N, N] of `mask_dtype`, or ptr NULL */
+    const uint8_t* mask_live;/* optional [nW] bytes from fwa2_mask_scan: 0 = that window's mask is all
+                                zero and is skipped; NULL = every window's mask is read */
+
+    float*  lse;             /* [BW, H, lse_stride_h] fp32 natural-log log-sum-exp per query row;
+                                written by forward, read by backward (attn_kernel_forward.py:294-295) */
+    int64_t lse_stride_bw;
+    int64_t lse_stride_h;    /* >= n; the reference rounds N up to a multiple of 64 */
+
+    /* (bwd) */
+    fwa2_tensor4 d_o;        /* upstream gradient of o */
+    fwa2_tensor4 dq, dk, dv; /* outputs, `dtype` */
+    void*   dbias;           /* [H, N, N] contiguous, `dtype`; NULL when bias is absent */
+    void*   dscale;          /* [H] contiguous, `dtype`; NULL unless FWA2_SCALE_TENSOR.  Already
+                                multiplied by [l_h <= ln 100] (attn_kernel_backward.py:706-711) */
+    void*   workspace;       /* device scratch of at least fwa2_backward_workspace_bytes() bytes,
+                                256-byte aligned; contents need not be initialised */
+    size_t  workspace_bytes;
+
+    void*   stream;          /* hipStream_t */
+} fwa2_problem;
+
+/* Library / ABI identification.  Returns FWA2_ABI_VERSION. */
+int fwa2_abi_version(void);
+
+/* Thread-local description of the last failure on the calling thread ("" if none). */
+const char* fwa2_last_error(void);
+
+/*
+ * Checks a problem description against the contract without touching the
+ * device (shapes, dtypes, strides, NULL-ness, supported sizes).  `backward`
+ * non-zero also checks the (bwd) fields.  Mirrors the assertions at
+ * attn_kernel_forward.py:263-292 and attn_kernel_backward.py:571-579, 616-633.
+ */
+int fwa2_validate(const fwa2_problem* p, int backward);
+
+/*
+ * live[w] = 1 if mask[w] holds any non-zero entry, else 0 (device bytes, one
+ * per window).  Shifted-window masks are all zero for most windows; passing
+ * the result as fwa2_problem.mask_live lets the kernels skip those reads.
+ * Has no counterpart in the reference, which always reads the mask.
+ */
+int fwa2_mask_scan(const void* mask, int mask_dtype, int n_windows, int n, int64_t stride_w, int64_t stride_n,
+                   uint8_t* live, void* stream);
+
+/*
+ * Bytes of device scratch fwa2_backward needs for this problem (fp32
+ * accumulators for dbias and dscale; the reference allocates these as
+ * db_accum / dscale_accum, attn_kernel_backward.py:609-626).  0 if none.
+ */
+size_t fwa2_backward_workspace_bytes(const fwa2_problem* p);
+
+/*
+ * o, lse = attention(q, k, v, logit_scale, bias, mask).
+ * Replaces _flash_attn_forward (attn_kernel_forward.py:261-345).
+ */
+int fwa2_forward(const fwa2_problem* p);
+
+/*
+ * dq, dk, dv, dbias, dscale from d_o and the saved q, k, v, o, lse.
+ * Replaces _flash_attn_backward (attn_kernel_backward.py:567-711), including
+ * its delta = rowsum(o * do) pre-pass (:6-51), accumulator zero-fill, down-cast
+ * copies and the clamp gate on dscale.
+ */
+int fwa2_backward(const fwa2_problem* p);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FWA2_H */
