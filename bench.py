@@ -1,0 +1,243 @@
+#!/usr/bin/env python3
+"""Benchmark of the hot path: Swin V2 scaled-cosine window attention, forward +
+backward, on one MI355X.
+
+A "step" is one forward + backward of the operator on the benchmark's
+synthetic batch (BASELINE config 3: B=64 images x 64 windows of N=256 tokens,
+3 heads, head dim 32, bf16, shifted-window mask, bias = 16*sigmoid(N(0,1)),
+logit_scale = ln 10), inputs already resident in HBM.  One JSON line goes to
+stdout; progress goes to stderr.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extras]
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+METRIC = "fwd+bwd ms & TFLOPS (% MFMA peak), B64 nW64 H3 d32 N256 bf16, 1 GPU"
+MFMA_BF16_PEAK_TFLOPS = 2500.0     # MI355X dense bf16
+HBM_PEAK_GBS = 8000.0              # MI355X HBM3E
+# HBM bytes per launch of the backward kernel at the benchmark shape, from
+# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a copy kernel of known size
+# (profiles/bwd_kernel_C3_pmc.txt); None until measured.
+BWD_KERNEL_TRAFFIC_BYTES = None
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def flops_matmul(bw, heads, n, d, fwd=True, bwd=True):
+    """Algorithmic matmul flops: 4 N^2 d forward (QK^T, PV), 10 N^2 d backward."""
+    per = (4 if fwd else 0) + (10 if bwd else 0)
+    return per * n * n * d * bw * heads
+
+
+def bytes_min(bw, heads, n, d, n_windows, fwd=True, bwd=True, e=2):
+    """Algorithmic HBM bytes: q,k,v,o (+lse) forward; q,k,v,o,do,dq,dk,dv (+lse, dbias) backward;
+    bias and mask once per pass."""
+    unit = bw * heads
+    side = heads * n * n * e + n_windows * n * n * e
+    tot = 0
+    if fwd:
+        tot += unit * (4 * n * d * e + 4 * n) + side
+    if bwd:
+        tot += unit * (8 * n * d * e + 4 * n) + side + heads * n * n * e
+    return tot
+
+
+class HipEvents:
+    """Raw hipEvent pairs (torch.cuda.Event would only see torch's current stream; these are
+    recorded by the library on the stream the kernel is launched on)."""
+
+    def __init__(self, count):
+        self.hip = ctypes.CDLL("libamdhip64.so")
+        self.hip.hipEventElapsedTime.argtypes = [ctypes.POINTER(ctypes.c_float), ctypes.c_void_p, ctypes.c_void_p]
+        self.hip.hipEventCreate.argtypes = [ctypes.POINTER(ctypes.c_void_p)]
+        self.hip.hipEventSynchronize.argtypes = [ctypes.c_void_p]
+        self.pairs = []
+        for _ in range(count):
+            a, b = ctypes.c_void_p(), ctypes.c_void_p()
+            assert self.hip.hipEventCreate(ctypes.byref(a)) == 0 and self.hip.hipEventCreate(ctypes.byref(b)) == 0
+            self.pairs.append((a, b))
+
+    def elapsed_ms(self):
+        out = []
+        for a, b in self.pairs:
+            assert self.hip.hipEventSynchronize(b) == 0
+            ms = ctypes.c_float()
+            assert self.hip.hipEventElapsedTime(ctypes.byref(ms), a, b) == 0
+            out.append(ms.value)
+        return out
+
+
+def time_steps(fn, steps, warmup, torch):
+    for _ in range(warmup):
+        fn(-1)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        fn(i)
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
+def cpu_baseline(cfg, torch):
+    """The oracle's classic fp32 path (forward + autograd backward) on the host cores, on a
+    bounded batch slice of the same workload."""
+    from oracle.classic_torch import classic_fwd_bwd
+    from oracle.swin_inputs import make_inputs
+
+    cores = len(os.sched_getaffinity(0))
+    torch.set_num_threads(cores)
+    sample_batch = 1
+    small = dict(cfg, batch=sample_batch)
+    inp = make_inputs(**small, dtype=torch.bfloat16, seed=0)
+    args = (inp["q"], inp["k"], inp["v"], inp["logit_scale"], inp["bias"], inp["mask"], inp["do"])
+    classic_fwd_bwd(*args)                       # warm-up
+    times = []
+    t_end = time.perf_counter() + 20.0
+    while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 10):
+        t0 = time.perf_counter()
+        classic_fwd_bwd(*args)
+        times.append(time.perf_counter() - t0)
+    sec = sorted(times)[len(times) // 2]
+    fl = flops_matmul(sample_batch * cfg["n_windows"], cfg["heads"], cfg["n"], cfg["d"])
+    return {
+        "value": round(fl / sec * 1e-12, 5), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+        "sample": f"classic fp32 torch forward+backward on batch {sample_batch} of {cfg['batch']} "
+                  f"(BW={sample_batch * cfg['n_windows']}), median of {len(times)} runs, {sec * 1e3:.1f} ms each; "
+                  f"scaled to the full batch: {sec * 1e3 * cfg['batch'] / sample_batch:.0f} ms per step",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extras", action="store_true", help="skip forward-only, N=64 and memory figures")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU only (the hot path has no cross-GPU step); use --gpus 1")
+
+    import torch
+
+    from flash_window_attention_v2_amd import _abi, flash_win_attn_v2_func
+    from oracle.swin_inputs import CONFIGS, make_inputs
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    lib = _abi.load()
+    torch.cuda.set_device(0)
+
+    def setup(cfg):
+        inp = make_inputs(**cfg, dtype=torch.bfloat16, seed=0)
+        dev = {k: (None if v is None else v.cuda()) for k, v in inp.items()}
+        for name in ("q", "k", "v", "bias", "logit_scale"):
+            dev[name].requires_grad_(True)
+        return dev
+
+    def make_step(dev, events=None):
+        leaves = [dev[n] for n in ("q", "k", "v", "bias", "logit_scale")]
+
+        def step(i):
+            if events is not None and i >= 0:
+                lib.fwa2_set_kernel_events(*events.pairs[i])
+            o = flash_win_attn_v2_func(dev["q"], dev["k"], dev["v"], dev["logit_scale"], dev["bias"], dev["mask"])
+            o.backward(dev["do"])
+            if events is not None:
+                lib.fwa2_set_kernel_events(None, None)
+            for t in leaves:
+                t.grad = None
+        return step
+
+    cfg = CONFIGS["C3"]
+    bw = cfg["batch"] * cfg["n_windows"]
+    log(f"[bench] building inputs {cfg}")
+    dev = setup(cfg)
+    events = HipEvents(args.steps)
+    log("[bench] timing forward+backward")
+    ms = time_steps(make_step(dev, events), args.steps, args.warmup, torch)
+    kern_ms = events.elapsed_ms()
+    kern_avg = sum(kern_ms) / len(kern_ms)
+    fl_all = flops_matmul(bw, cfg["heads"], cfg["n"], cfg["d"])
+    fl_bwd = flops_matmul(bw, cfg["heads"], cfg["n"], cfg["d"], fwd=False)
+    tflops = fl_all / (ms * 1e-3) * 1e-12
+    achieved = fl_bwd / (kern_avg * 1e-3) * 1e-12
+
+    result = {
+        "metric": METRIC, "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "C3: B64 x 64 windows, H3, N256, d32, bf16, shift-8 mask, fwd+bwd", "bw": bw,
+                   "heads": cfg["heads"], "n": cfg["n"], "head_dim": cfg["d"]},
+        "pct_mfma_peak": round(100 * tflops / MFMA_BF16_PEAK_TFLOPS, 2),
+        "roofline": {"bound": "mfma", "kernel": "bwd_kernel", "achieved": round(achieved, 2),
+                     "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": BWD_KERNEL_TRAFFIC_BYTES,
+                     "kernel_ms": round(kern_avg, 4),
+                     "hbm_frac_of_8TBs": round(bytes_min(bw, cfg["heads"], cfg["n"], cfg["d"], cfg["n_windows"], fwd=False)
+                                               / (kern_avg * 1e-3) / (HBM_PEAK_GBS * 1e9), 4)},
+    }
+
+    if not args.no_extras:
+        extras = {}
+        log("[bench] forward only")
+        with torch.no_grad():
+            f_ms = time_steps(lambda i: flash_win_attn_v2_func(dev["q"], dev["k"], dev["v"], dev["logit_scale"],
+                                                               dev["bias"], dev["mask"]), args.steps, args.warmup, torch)
+        extras["fwd_ms"] = round(f_ms, 4)
+        extras["fwd_tflops"] = round(flops_matmul(bw, cfg["heads"], cfg["n"], cfg["d"], bwd=False) / f_ms * 1e-9, 2)
+        extras["fwd_hbm_gbs"] = round(bytes_min(bw, cfg["heads"], cfg["n"], cfg["d"], cfg["n_windows"], bwd=False) / f_ms * 1e-6, 1)
+        extras["fwd_bwd_hbm_gbs"] = round(bytes_min(bw, cfg["heads"], cfg["n"], cfg["d"], cfg["n_windows"]) / ms * 1e-6, 1)
+        # peak memory of the op against the classic path in the same dtype on the GPU
+        step = make_step(dev)
+        torch.cuda.synchronize(); torch.cuda.empty_cache(); torch.cuda.reset_peak_memory_stats()
+        base = torch.cuda.memory_allocated()
+        step(-1); torch.cuda.synchronize()
+        extras["peak_mem_mb_new"] = round((torch.cuda.max_memory_allocated() - base) / 2**20, 1)
+        from flash_window_attention_v2_amd import win_attention_torch
+        torch.cuda.empty_cache(); torch.cuda.reset_peak_memory_stats()
+        base = torch.cuda.memory_allocated()
+        o = win_attention_torch(dev["q"], dev["k"], dev["v"], dev["logit_scale"], dev["bias"], dev["mask"])
+        o.backward(dev["do"]); torch.cuda.synchronize()
+        extras["peak_mem_mb_classic_bf16"] = round((torch.cuda.max_memory_allocated() - base) / 2**20, 1)
+        del o
+        for n_ in ("q", "k", "v", "bias", "logit_scale"):
+            dev[n_].grad = None
+        extras["peak_mem_ratio"] = round(extras["peak_mem_mb_new"] / extras["peak_mem_mb_classic_bf16"], 4)
+        del dev
+        torch.cuda.empty_cache()
+        # N = 64 (config 2) is bandwidth-bound: report achieved HBM GB/s
+        log("[bench] config 2 (N=64)")
+        c2 = CONFIGS["C2"]
+        dev2 = setup(c2)
+        ms2 = time_steps(make_step(dev2), args.steps, args.warmup, torch)
+        bw2 = c2["batch"] * c2["n_windows"]
+        extras["c2_fwd_bwd_ms"] = round(ms2, 4)
+        extras["c2_hbm_gbs"] = round(bytes_min(bw2, c2["heads"], c2["n"], c2["d"], c2["n_windows"]) / ms2 * 1e-6, 1)
+        extras["c2_hbm_frac"] = round(extras["c2_hbm_gbs"] / HBM_PEAK_GBS, 4)
+        extras["c2_tflops"] = round(flops_matmul(bw2, c2["heads"], c2["n"], c2["d"]) / ms2 * 1e-9, 2)
+        del dev2
+        result["extras"] = extras
+
+    if not args.no_cpu:
+        log("[bench] CPU baseline (classic fp32 on host cores)")
+        result["cpu_baseline"] = cpu_baseline(cfg, torch)
+    else:
+        result["cpu_baseline"] = None
+
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

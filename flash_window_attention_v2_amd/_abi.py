@@ -25,6 +25,7 @@ EXPORTS = (
     "fwa2_backward_workspace_bytes",
     "fwa2_forward",
     "fwa2_backward",
+    "fwa2_set_kernel_events",
 )
 
 
@@ -93,6 +94,8 @@ def load():
         lib.fwa2_forward.restype = ctypes.c_int
         lib.fwa2_backward.argtypes = [ctypes.POINTER(Problem)]
         lib.fwa2_backward.restype = ctypes.c_int
+        lib.fwa2_set_kernel_events.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
+        lib.fwa2_set_kernel_events.restype = None
         if lib.fwa2_abi_version() != ABI_VERSION:
             raise Fwa2Error(f"libfwa2 ABI {lib.fwa2_abi_version()} != binding ABI {ABI_VERSION}")
         _lib = lib

@@ -1,6 +1,7 @@
 // extern "C" surface of libfwa2 (declared in include/fwa2.h): argument
 // validation, workspace sizing and dispatch to the gfx950 kernels.  Nothing
 // here allocates device memory or synchronises.
+#include <atomic>
 #include <stdarg.h>
 #include <stdio.h>
 #include <string.h>
@@ -19,6 +20,8 @@ int backward_supported(int n);
 namespace {
 
 thread_local char g_err[512] = "";
+// measurement hook: process-wide, because autograd runs backward on its own thread
+std::atomic<void*> g_ev_start{nullptr}, g_ev_stop{nullptr};
 
 int fail(int code, const char* fmt, ...) {
     va_list ap;
@@ -140,6 +143,11 @@ int fwa2_mask_scan(const void* mask, int mask_dtype, int n_windows, int n, int64
     return FWA2_OK;
 }
 
+void fwa2_set_kernel_events(void* start, void* stop) {
+    g_ev_start.store(start);
+    g_ev_stop.store(stop);
+}
+
 int fwa2_forward(const fwa2_problem* p) {
     g_err[0] = 0;
     int rc = validate(p, 0);
@@ -182,6 +190,8 @@ int fwa2_backward(const fwa2_problem* p) {
     k.dbias = p->dbias; k.dscale = p->dscale;
     k.workspace = p->workspace;
     k.cus = cu_count();
+    k.ev_start = (hipEvent_t)g_ev_start.load();
+    k.ev_stop = (hipEvent_t)g_ev_stop.load();
     hipError_t e = fwa2::launch_backward(k, p->dtype, p->bias.ptr != nullptr, p->mask.ptr ? p->mask_dtype : -1,
                                          (hipStream_t)p->stream);
     if (e != hipSuccess) return fail(FWA2_ERR_HIP, "backward launch: %s", hipGetErrorString(e));

@@ -35,7 +35,6 @@
 namespace fwa2 {
 
 constexpr int kRow = 40;    // LDS row stride of 16-bit tiles, in elements (80 bytes)
-constexpr int kAccRow = 33; // LDS row stride of the fp32 dQ accumulator, in floats
 
 template <int DT, int MASK_DT> struct MaskElemB { typedef typename Elem<DT>::E E; };
 template <int DT> struct MaskElemB<DT, FWA2_F32> { typedef float E; };
@@ -52,8 +51,9 @@ __device__ __forceinline__ float wave_sum(float x) {
     return x;
 }
 
-template <int DT, bool HAS_BIAS, int MASK_DT, int NQB>
-__global__ void __launch_bounds__(NQB * 128) bwd_kernel(const BwdParams p) {
+// KT = key tiles of 16 owned by one wavefront, NQB = compile-time bound on query blocks of 32.
+template <int DT, bool HAS_BIAS, int MASK_DT, int NQB, int KT>
+__global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) {
     typedef typename Elem<DT>::E E;
     typedef typename Elem<DT>::V8 V8;
     typedef typename Elem<DT>::V4 V4;
@@ -62,18 +62,16 @@ __global__ void __launch_bounds__(NQB * 128) bwd_kernel(const BwdParams p) {
 
     const int N = p.n;
     const int R = (N + 31) & ~31;          // padded query rows (and LDS rows)
-    const int NPk = p.waves * 16;          // padded key rows
+    const int NPk = p.waves * 16 * KT;     // padded key rows
     const int nqb = R >> 5;                // query blocks of 32
     const int nks = R >> 5;                // key steps of 32 in phase B
-    const int ngroups = p.waves >= 4 ? (p.waves >> 2) : 1;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     E* Qs = reinterpret_cast<E*>(smem_raw);
     E* Ks = Qs + R * kRow;
     E* dOs = Ks + R * kRow;
     E* dZs = dOs + R * kRow;               // 2 buffers
-    float* dQacc = reinterpret_cast<float*>(dZs + 2 * R * kRow);
-    float* lse2s = dQacc + R * kAccRow;
+    float* lse2s = reinterpret_cast<float*>(dZs + 2 * R * kRow);
     float* deltas = lse2s + R;
     float* red = deltas + R;               // [16]
 
@@ -96,21 +94,22 @@ __global__ void __launch_bounds__(NQB * 128) bwd_kernel(const BwdParams p) {
     }
     const float scale2 = s_true * kLog2e;
 
-    const int key = wave * 16 + l16;       // the key this lane owns in the score tiles
-    const bool key_ok = key < N;
+    const int key0 = wave * 16 * KT + l16;  // this lane's key in key tile 0 (tile kt: + 16 kt)
 
-    float dbacc[NQB][8];
+    float dbacc[NQB][KT][8];
 #pragma unroll
     for (int a = 0; a < NQB; a++)
 #pragma unroll
-        for (int j = 0; j < 8; j++) dbacc[a][j] = 0.f;
+        for (int kt = 0; kt < KT; kt++)
+#pragma unroll
+            for (int j = 0; j < 8; j++) dbacc[a][kt][j] = 0.f;
     float ds_part = 0.f;
 
     // dZ staging rows that no wavefront writes must read as zeros in phase B
     for (int i = tid; i < 2 * R * kRow / 8; i += nthreads) st8<V8>(dZs + i * 8, zero8<V8>());
 
     const E* bias_t = nullptr;
-    if (HAS_BIAS) bias_t = reinterpret_cast<const E*>(p.bias_t) + ((int64_t)h * NPk + key) * R;
+    if (HAS_BIAS) bias_t = reinterpret_cast<const E*>(p.bias_t) + ((int64_t)h * NPk + key0) * R;
 
     for (int b = grp; b < p.bw; b += p.groups) {
         const E* qptr = reinterpret_cast<const E*>(p.q.ptr) + b * p.q.sb + h * p.q.sh;
@@ -118,6 +117,7 @@ __global__ void __launch_bounds__(NQB * 128) bwd_kernel(const BwdParams p) {
         const E* vptr = reinterpret_cast<const E*>(p.v.ptr) + b * p.v.sb + h * p.v.sh;
         const E* optr = reinterpret_cast<const E*>(p.o.ptr) + b * p.o.sb + h * p.o.sh;
         const E* doptr = reinterpret_cast<const E*>(p.d_o.ptr) + b * p.d_o.sb + h * p.d_o.sh;
+        E* dqptr = reinterpret_cast<E*>(const_cast<void*>(p.dq.ptr)) + b * p.dq.sb + h * p.dq.sh;
         const float* lseptr = p.lse + b * p.lse_sb + h * p.lse_sh;
 
         const ME* mask_t = nullptr;
@@ -125,11 +125,11 @@ __global__ void __launch_bounds__(NQB * 128) bwd_kernel(const BwdParams p) {
         if (MASK_DT >= 0) {
             const int w = b % p.n_windows;
             mask_on = p.mask_live ? (p.mask_live[w] != 0) : true;
-            mask_t = reinterpret_cast<const ME*>(p.mask_t) + ((int64_t)w * NPk + key) * R;
+            mask_t = reinterpret_cast<const ME*>(p.mask_t) + ((int64_t)w * NPk + key0) * R;
         }
 
-        __syncthreads();   // the previous unit's epilogue is done with LDS
-        // ---- load: one 8-element chunk of one row per thread ----
+        __syncthreads();   // the previous unit is done with LDS
+        // ---- load: one 8-element chunk of one row per thread and pass ----
         for (int r = tid >> 2; r < R; r += nthreads >> 2) {
             const int dc = (tid & 3) * 8;
             V8 q8 = zero8<V8>(), k8 = zero8<V8>(), do8 = zero8<V8>(), o8 = zero8<V8>();
@@ -158,131 +158,157 @@ __global__ void __launch_bounds__(NQB * 128) bwd_kernel(const BwdParams p) {
                 if (r < N) { const float l = lseptr[r]; l2 = (l == -INFINITY) ? INFINITY : l * kLog2e; }
                 lse2s[r] = l2;
             }
-#pragma unroll
-            for (int j = 0; j < 8; j++) dQacc[r * kAccRow + dc + j] = 0.f;
         }
-        V8 bv = zero8<V8>();
-        if (key_ok) bv = ld8<V8>(vptr + (int64_t)key * p.v.sn + 8 * g);
+        V8 bv[KT], bk[KT];
+#pragma unroll
+        for (int kt = 0; kt < KT; kt++) {
+            bv[kt] = zero8<V8>();
+            if (key0 + 16 * kt < N) bv[kt] = ld8<V8>(vptr + (int64_t)(key0 + 16 * kt) * p.v.sn + 8 * g);
+        }
         __syncthreads();
-        const V8 bk = ld8<V8>(Ks + key * kRow + 8 * g);
+#pragma unroll
+        for (int kt = 0; kt < KT; kt++) bk[kt] = ld8<V8>(Ks + (key0 + 16 * kt) * kRow + 8 * g);
 
-        f32x4 dvacc[2], dkacc[2];
+        f32x4 dvacc[KT][2], dkacc[KT][2];
 #pragma unroll
-        for (int dt = 0; dt < 2; dt++)
+        for (int kt = 0; kt < KT; kt++)
 #pragma unroll
-            for (int i = 0; i < 4; i++) { dvacc[dt][i] = 0.f; dkacc[dt][i] = 0.f; }
+            for (int dt = 0; dt < 2; dt++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) { dvacc[kt][dt][i] = 0.f; dkacc[kt][dt][i] = 0.f; }
 
 #pragma unroll
         for (int qb = 0; qb < NQB; qb++) {
             if (qb < nqb) {
+                __builtin_amdgcn_sched_barrier(0);   // keep the unrolled blocks apart: register pressure
                 E* dZbuf = dZs + (qb & 1) * R * kRow;
                 const int q8 = 32 * qb + 8 * g;          // first of this lane's 8 queries
                 // ---- phase A ----
-                f32x4 sacc[2], pacc[2];
+                V8 aq[2], ado[2];
 #pragma unroll
                 for (int t = 0; t < 2; t++) {
                     const int rowq = 32 * qb + 8 * (l16 >> 2) + 4 * t + (l16 & 3);
-                    const V8 aq = ld8<V8>(Qs + rowq * kRow + 8 * g);
-                    const V8 ado = ld8<V8>(dOs + rowq * kRow + 8 * g);
-                    f32x4 z = {0.f, 0.f, 0.f, 0.f};
-                    sacc[t] = Elem<DT>::mfma16(aq, bk, z);
-                    pacc[t] = Elem<DT>::mfma16(ado, bv, z);
-                }
-                float zz[8];
-#pragma unroll
-                for (int j = 0; j < 8; j++) zz[j] = sacc[j >> 2][j & 3];
-                if (HAS_BIAS) {
-                    float x[8];
-                    unpack8b(ld8<V8>(bias_t + q8), x);
-#pragma unroll
-                    for (int j = 0; j < 8; j++) zz[j] = fmaf(x[j], kLog2e, zz[j]);
-                }
-                if (MASK_DT >= 0) {
-                    if (mask_on) {
-                        const MV8 mv = *reinterpret_cast<const MV8*>(mask_t + q8);
-#pragma unroll
-                        for (int j = 0; j < 8; j++) zz[j] = fmaf((float)mv[j], kLog2e, zz[j]);
-                    }
+                    aq[t] = ld8<V8>(Qs + rowq * kRow + 8 * g);
+                    ado[t] = ld8<V8>(dOs + rowq * kRow + 8 * g);
                 }
                 const f32x4 la = *reinterpret_cast<const f32x4*>(lse2s + q8);
                 const f32x4 lb = *reinterpret_cast<const f32x4*>(lse2s + q8 + 4);
                 const f32x4 da = *reinterpret_cast<const f32x4*>(deltas + q8);
                 const f32x4 db = *reinterpret_cast<const f32x4*>(deltas + q8 + 4);
-                V8 p8, z8;
+                V8 p8[KT], z8[KT];
 #pragma unroll
-                for (int j = 0; j < 8; j++) {
-                    const float l2 = j < 4 ? la[j & 3] : lb[j & 3];
-                    const float dl = j < 4 ? da[j & 3] : db[j & 3];
-                    const float zin = key_ok ? zz[j] : -INFINITY;
-                    const float pj = fast_exp2(zin - l2);
-                    const float dz = pj * (pacc[j >> 2][j & 3] - dl);
-                    if (HAS_BIAS) dbacc[qb][j] += dz;
-                    p8[j] = (E)pj;
-                    z8[j] = (E)dz;
+                for (int kt = 0; kt < KT; kt++) {
+                    const bool key_ok = key0 + 16 * kt < N;
+                    f32x4 sacc[2], pacc[2];
+#pragma unroll
+                    for (int t = 0; t < 2; t++) {
+                        const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+                        sacc[t] = Elem<DT>::mfma16(aq[t], bk[kt], z);
+                        pacc[t] = Elem<DT>::mfma16(ado[t], bv[kt], z);
+                    }
+                    float zz[8];
+#pragma unroll
+                    for (int j = 0; j < 8; j++) zz[j] = sacc[j >> 2][j & 3];
+                    if (HAS_BIAS) {
+                        float x[8];
+                        unpack8b(ld8<V8>(bias_t + (int64_t)16 * kt * R + q8), x);
+#pragma unroll
+                        for (int j = 0; j < 8; j++) zz[j] = fmaf(x[j], kLog2e, zz[j]);
+                    }
+                    if (MASK_DT >= 0) {
+                        if (mask_on) {
+                            const MV8 mv = *reinterpret_cast<const MV8*>(mask_t + (int64_t)16 * kt * R + q8);
+#pragma unroll
+                            for (int j = 0; j < 8; j++) zz[j] = fmaf((float)mv[j], kLog2e, zz[j]);
+                        }
+                    }
+#pragma unroll
+                    for (int j = 0; j < 8; j++) {
+                        const float l2 = j < 4 ? la[j & 3] : lb[j & 3];
+                        const float dl = j < 4 ? da[j & 3] : db[j & 3];
+                        const float zin = key_ok ? zz[j] : -INFINITY;
+                        const float pj = fast_exp2(zin - l2);
+                        const float dz = pj * (pacc[j >> 2][j & 3] - dl);
+                        if (HAS_BIAS) dbacc[qb][kt][j] += dz;
+                        p8[kt][j] = (E)pj;
+                        z8[kt][j] = (E)dz;
+                    }
+                    st8<V8>(dZbuf + (key0 + 16 * kt) * kRow + 8 * g, z8[kt]);
                 }
-                st8<V8>(dZbuf + key * kRow + 8 * g, z8);
 #pragma unroll
                 for (int dt = 0; dt < 2; dt++) {
                     const int off = (q8 + (l16 >> 2)) * kRow + 16 * dt + 4 * (l16 & 3);
                     const V8 a_do = lds_tr8<DT>(dOs + off, dOs + off + 4 * kRow);
-                    dvacc[dt] = Elem<DT>::mfma16(a_do, p8, dvacc[dt]);
                     const V8 a_q = lds_tr8<DT>(Qs + off, Qs + off + 4 * kRow);
-                    dkacc[dt] = Elem<DT>::mfma16(a_q, z8, dkacc[dt]);
+#pragma unroll
+                    for (int kt = 0; kt < KT; kt++) {
+                        dvacc[kt][dt] = Elem<DT>::mfma16(a_do, p8[kt], dvacc[kt][dt]);
+                        dkacc[kt][dt] = Elem<DT>::mfma16(a_q, z8[kt], dkacc[kt][dt]);
+                    }
                 }
                 __syncthreads();
-                // ---- phase B: dQ_hat^T tile (dt, qt), a share of the key steps ----
-                if (wave < 4 * ngroups) {
-                    const int dt = wave & 1, qt = (wave >> 1) & 1;
-                    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-                    for (int ks = wave >> 2; ks < nks; ks += ngroups) {
-                        const int rowk = (32 * ks + 8 * g + (l16 >> 2)) * kRow;
-                        const int ca = rowk + 16 * dt + 4 * (l16 & 3);
-                        const int cb = rowk + 16 * qt + 4 * (l16 & 3);
-                        const V8 a_k = lds_tr8<DT>(Ks + ca, Ks + ca + 4 * kRow);
-                        const V8 b_z = lds_tr8<DT>(dZbuf + cb, dZbuf + cb + 4 * kRow);
-                        acc = Elem<DT>::mfma16(a_k, b_z, acc);
-                    }
-                    float* dst = dQacc + (32 * qb + 16 * qt + l16) * kAccRow + 16 * dt + 4 * g;
+                // ---- phase B: dQ_hat^T for 16 queries (all d, all keys), one wavefront per job,
+                //      then straight through the normalisation Jacobian to global memory ----
 #pragma unroll
-                    for (int i = 0; i < 4; i++) atomicAdd(dst + i, acc[i]);
+                for (int qt = 0; qt < 2; qt++) {
+                    if ((2 * qb + qt) % p.waves == wave) {
+                        f32x4 acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+                        for (int ks = 0; ks < nks; ks++) {
+                            const int rowk = (32 * ks + 8 * g + (l16 >> 2)) * kRow;
+                            const int cb = rowk + 16 * qt + 4 * (l16 & 3);
+                            const V8 b_z = lds_tr8<DT>(dZbuf + cb, dZbuf + cb + 4 * kRow);
+#pragma unroll
+                            for (int dt = 0; dt < 2; dt++) {
+                                const int ca = rowk + 16 * dt + 4 * (l16 & 3);
+                                const V8 a_k = lds_tr8<DT>(Ks + ca, Ks + ca + 4 * kRow);
+                                acc[dt] = Elem<DT>::mfma16(a_k, b_z, acc[dt]);
+                            }
+                        }
+                        // lane (query, g) holds d = 16dt + 4g + i
+                        const int query = 32 * qb + 16 * qt + l16;
+                        const bool q_ok = query < N;
+                        float x[8], a[8];
+                        float ss = 0.f, dot = 0.f;
+#pragma unroll
+                        for (int dt = 0; dt < 2; dt++) {
+                            V4 q4;
+#pragma unroll
+                            for (int i = 0; i < 4; i++) q4[i] = 0;
+                            if (q_ok) q4 = *reinterpret_cast<const V4*>(qptr + (int64_t)query * p.q.sn + 16 * dt + 4 * g);
+#pragma unroll
+                            for (int i = 0; i < 4; i++) {
+                                x[4 * dt + i] = (float)q4[i];
+                                a[4 * dt + i] = acc[dt][i];
+                                ss += x[4 * dt + i] * x[4 * dt + i];
+                            }
+                        }
+                        ss = xor32_add(xor16_add(ss));
+                        const float nrm = sqrtf(ss);
+                        const float inv = 1.0f / fmaxf(nrm, kNormEps);
+#pragma unroll
+                        for (int j = 0; j < 8; j++) { x[j] *= inv; dot += a[j] * x[j]; }
+                        dot = xor32_add(xor16_add(dot));
+                        const float proj = nrm > kNormEps ? dot : 0.f;
+                        const float f = s_true * inv;
+                        if (q_ok) {
+#pragma unroll
+                            for (int dt = 0; dt < 2; dt++) {
+                                V4 o4;
+#pragma unroll
+                                for (int i = 0; i < 4; i++) o4[i] = (E)(f * (a[4 * dt + i] - x[4 * dt + i] * proj));
+                                *reinterpret_cast<V4*>(dqptr + (int64_t)query * p.dq.sn + 16 * dt + 4 * g) = o4;
+                            }
+                            if (g == 0) ds_part += dot;
+                        }
+                    }
                 }
             }
         }
-        __syncthreads();
-        // ---- epilogue dq: back through q / max(|q|, eps) ----
-        for (int r = tid >> 2; r < N; r += nthreads >> 2) {
-            const int dc = (tid & 3) * 8;
-            float x[8], a[8];
-            unpack8b(ld8<V8>(qptr + (int64_t)r * p.q.sn + dc), x);
-            float ss = 0.f, dot = 0.f;
-#pragma unroll
-            for (int j = 0; j < 8; j++) { a[j] = dQacc[r * kAccRow + dc + j]; ss += x[j] * x[j]; }
-            ss = quad_add(ss);
-            const float nrm = sqrtf(ss);
-            const float inv = 1.0f / fmaxf(nrm, kNormEps);
-#pragma unroll
-            for (int j = 0; j < 8; j++) { x[j] *= inv; dot += a[j] * x[j]; }
-            dot = quad_add(dot);
-            const float proj = nrm > kNormEps ? dot : 0.f;
-            const float f = s_true * inv;
-            V8 out;
-#pragma unroll
-            for (int j = 0; j < 8; j++) out[j] = (E)(f * (a[j] - x[j] * proj));
-            st8<V8>(reinterpret_cast<E*>(const_cast<void*>(p.dq.ptr)) + b * p.dq.sb + h * p.dq.sh + (int64_t)r * p.dq.sn + dc, out);
-            if ((tid & 3) == 0) ds_part += dot;
-        }
         // ---- epilogue dk, dv: lane (key, g) holds d = 16dt + 4g + i ----
-        if (key_ok) {
-            E* dvp = reinterpret_cast<E*>(const_cast<void*>(p.dv.ptr)) + b * p.dv.sb + h * p.dv.sh + (int64_t)key * p.dv.sn;
 #pragma unroll
-            for (int dt = 0; dt < 2; dt++) {
-                V4 o4;
-#pragma unroll
-                for (int i = 0; i < 4; i++) o4[i] = (E)dvacc[dt][i];
-                *reinterpret_cast<V4*>(dvp + 16 * dt + 4 * g) = o4;
-            }
-        }
-        {
+        for (int kt = 0; kt < KT; kt++) {
+            const int key = key0 + 16 * kt;
+            const bool key_ok = key < N;
             float x[8], a[8];
             float ss = 0.f, dot = 0.f;
 #pragma unroll
@@ -294,7 +320,7 @@ __global__ void __launch_bounds__(NQB * 128) bwd_kernel(const BwdParams p) {
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     x[4 * dt + i] = (float)k4[i];
-                    a[4 * dt + i] = dkacc[dt][i] * kLn2;      // undo the log2e folded into Q_hat
+                    a[4 * dt + i] = dkacc[kt][dt][i] * kLn2;      // undo the log2e folded into Q_hat
                     ss += x[4 * dt + i] * x[4 * dt + i];
                 }
             }
@@ -307,12 +333,17 @@ __global__ void __launch_bounds__(NQB * 128) bwd_kernel(const BwdParams p) {
             const float proj = nrm > kNormEps ? dot : 0.f;
             if (key_ok) {
                 E* dkp = reinterpret_cast<E*>(const_cast<void*>(p.dk.ptr)) + b * p.dk.sb + h * p.dk.sh + (int64_t)key * p.dk.sn;
+                E* dvp = reinterpret_cast<E*>(const_cast<void*>(p.dv.ptr)) + b * p.dv.sb + h * p.dv.sh + (int64_t)key * p.dv.sn;
 #pragma unroll
                 for (int dt = 0; dt < 2; dt++) {
-                    V4 o4;
+                    V4 o4, v4;
 #pragma unroll
-                    for (int i = 0; i < 4; i++) o4[i] = (E)(inv * (a[4 * dt + i] - x[4 * dt + i] * proj));
+                    for (int i = 0; i < 4; i++) {
+                        o4[i] = (E)(inv * (a[4 * dt + i] - x[4 * dt + i] * proj));
+                        v4[i] = (E)dvacc[kt][dt][i];
+                    }
                     *reinterpret_cast<V4*>(dkp + 16 * dt + 4 * g) = o4;
+                    *reinterpret_cast<V4*>(dvp + 16 * dt + 4 * g) = v4;
                 }
             }
         }
@@ -320,15 +351,18 @@ __global__ void __launch_bounds__(NQB * 128) bwd_kernel(const BwdParams p) {
 
     // ---- flush the per-workgroup partial sums ----
     if (HAS_BIAS) {
-        float* dst = p.part_dbias + (((int64_t)h * p.groups + grp) * NPk + key) * R;
 #pragma unroll
-        for (int qb = 0; qb < NQB; qb++) {
-            if (qb < nqb) {
-                f32x4 a, c;
+        for (int kt = 0; kt < KT; kt++) {
+            float* dst = p.part_dbias + (((int64_t)h * p.groups + grp) * NPk + key0 + 16 * kt) * R;
 #pragma unroll
-                for (int j = 0; j < 4; j++) { a[j] = dbacc[qb][j]; c[j] = dbacc[qb][4 + j]; }
-                *reinterpret_cast<f32x4*>(dst + 32 * qb + 8 * g) = a;
-                *reinterpret_cast<f32x4*>(dst + 32 * qb + 8 * g + 4) = c;
+            for (int qb = 0; qb < NQB; qb++) {
+                if (qb < nqb) {
+                    f32x4 a, c;
+#pragma unroll
+                    for (int j = 0; j < 4; j++) { a[j] = dbacc[qb][kt][j]; c[j] = dbacc[qb][kt][4 + j]; }
+                    *reinterpret_cast<f32x4*>(dst + 32 * qb + 8 * g) = a;
+                    *reinterpret_cast<f32x4*>(dst + 32 * qb + 8 * g + 4) = c;
+                }
             }
         }
     }
@@ -411,20 +445,22 @@ static size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 int backward_supported(int n) { return n >= 1 && n <= 256; }
 
 struct BwdPlan {
-    int waves, groups, npk, r, nqb_t;
+    int waves, groups, npk, r, nqb_t, kt;
     size_t off_dbias, off_dscale, off_bias_t, off_mask_t, total;
     size_t smem;
 };
 
 static BwdPlan make_plan(int heads, int n, int bw, bool has_bias, bool has_mask, int n_windows, int cus) {
     BwdPlan pl;
-    pl.waves = (n + 15) / 16;
-    pl.npk = pl.waves * 16;
     pl.r = (n + 31) & ~31;
     const int nqb = pl.r / 32;
     pl.nqb_t = nqb <= 2 ? 2 : (nqb <= 4 ? 4 : 8);
-    // registers allow 16 wavefronts per CU: as many workgroups as fit
-    const int wg_per_cu = pl.waves <= 4 ? 4 : (pl.waves <= 8 ? 2 : 1);
+    // up to 128 queries a wavefront owns one 16-key tile (<= 128 registers, several workgroups
+    // per CU); above that two tiles (<= 256 registers, one workgroup of 8 wavefronts per CU)
+    pl.kt = nqb <= 4 ? 1 : 2;
+    pl.waves = (n + 16 * pl.kt - 1) / (16 * pl.kt);
+    pl.npk = pl.waves * 16 * pl.kt;
+    const int wg_per_cu = pl.nqb_t == 2 ? 4 : (pl.nqb_t == 4 ? 2 : 1);
     int groups = (cus * wg_per_cu) / heads;
     if (groups < 1) groups = 1;
     if (groups > bw) groups = bw;
@@ -439,7 +475,7 @@ static BwdPlan make_plan(int heads, int n, int bw, bool has_bias, bool has_mask,
     pl.off_mask_t = off;
     if (has_mask) off += align256((size_t)n_windows * pl.npk * pl.r * 4);
     pl.total = off;
-    pl.smem = (size_t)5 * pl.r * kRow * 2 + (size_t)pl.r * kAccRow * 4 + (size_t)2 * pl.r * 4 + 16 * 4;
+    pl.smem = (size_t)5 * pl.r * kRow * 2 + (size_t)2 * pl.r * 4 + 16 * 4;
     return pl;
 }
 
@@ -448,23 +484,25 @@ size_t backward_workspace_bytes(int heads, int n, int bw, bool has_bias, bool ha
     return make_plan(heads, n, bw, has_bias, has_mask, n_windows, cus).total;
 }
 
-template <int DT, bool HAS_BIAS, int MASK_DT, int NQB>
+template <int DT, bool HAS_BIAS, int MASK_DT, int NQB, int KT>
 static hipError_t launch_main(const BwdParams& p, const BwdPlan& pl, hipStream_t st) {
-    auto kern = bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB>;
+    auto kern = bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT>;
     if (pl.smem > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)pl.smem);
         if (e != hipSuccess) return e;
     }
+    if (p.ev_start) (void)hipEventRecord(p.ev_start, st);
     hipLaunchKernelGGL(kern, dim3(p.heads * pl.groups), dim3(64 * pl.waves), pl.smem, st, p);
+    if (p.ev_stop) (void)hipEventRecord(p.ev_stop, st);
     return hipGetLastError();
 }
 
 template <int DT, bool HAS_BIAS, int MASK_DT>
 static hipError_t launch_nqb(const BwdParams& p, const BwdPlan& pl, hipStream_t st) {
-    if (pl.nqb_t == 2) return launch_main<DT, HAS_BIAS, MASK_DT, 2>(p, pl, st);
-    if (pl.nqb_t == 4) return launch_main<DT, HAS_BIAS, MASK_DT, 4>(p, pl, st);
-    return launch_main<DT, HAS_BIAS, MASK_DT, 8>(p, pl, st);
+    if (pl.nqb_t == 2) return launch_main<DT, HAS_BIAS, MASK_DT, 2, 1>(p, pl, st);
+    if (pl.nqb_t == 4) return launch_main<DT, HAS_BIAS, MASK_DT, 4, 1>(p, pl, st);
+    return launch_main<DT, HAS_BIAS, MASK_DT, 8, 2>(p, pl, st);
 }
 
 template <int DT>

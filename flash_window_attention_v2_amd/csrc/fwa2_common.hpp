@@ -162,6 +162,7 @@ struct BwdParams {
     void* dscale;     // [H] in the input dtype
     void* workspace;
     int cus;          // compute units of the device
+    hipEvent_t ev_start, ev_stop;  // optional: recorded right around the main backward kernel
     // filled in by the launcher
     int waves;        // wavefronts per workgroup = key tiles of 16
     int groups;       // workgroups per head (each walks bw = g, g + groups, ...)

@@ -159,6 +159,16 @@ int fwa2_forward(const fwa2_problem* p);
  */
 int fwa2_backward(const fwa2_problem* p);
 
+/*
+ * Measurement hook, no counterpart in the reference: when both are non-NULL the
+ * next fwa2_backward calls (from any thread of the process) record the two hipEvent_t on the
+ * problem's stream immediately before and after the main backward kernel (the
+ * transposing pre-pass and the partial-sum reduction stay outside), so a
+ * benchmark can time that kernel alone without a profiler.  Pass NULLs to
+ * switch it off.
+ */
+void fwa2_set_kernel_events(void* start_event, void* stop_event);
+
 #ifdef __cplusplus
 }
 #endif

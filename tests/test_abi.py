@@ -1,0 +1,128 @@
+"""The C-ABI library loads without a GPU, exports every symbol include/fwa2.h
+declares, and rejects contract violations before touching a device."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from flash_window_attention_v2_amd import _abi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    if not os.path.exists(_abi.lib_path()):
+        import __graft_entry__
+
+        __graft_entry__.build()
+    return _abi.load()
+
+
+def test_header_symbols_are_exported(lib):
+    header = open(os.path.join(ROOT, "include", "fwa2.h")).read()
+    declared = set(re.findall(r"^\s*(?:int|size_t|void|const char\*)\s+(fwa2_\w+)\s*\(", header, flags=re.M))
+    assert declared == set(_abi.EXPORTS)
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert lib.fwa2_abi_version() == _abi.ABI_VERSION
+
+
+def test_struct_layout_matches(lib):
+    # a problem of the wrong size is refused, one of the right size gets past the layout check
+    p = _abi.new_problem()
+    p.struct_bytes -= 8
+    assert lib.fwa2_validate(p, 0) == _abi.ERR_INVALID_ARGUMENT
+    assert b"layout mismatch" in lib.fwa2_last_error()
+    p = _abi.new_problem()
+    assert lib.fwa2_validate(p, 0) == _abi.ERR_INVALID_ARGUMENT
+    assert b"layout" not in lib.fwa2_last_error()
+
+
+def _good_problem(n=64, bw=8, heads=2, backward=False):
+    p = _abi.new_problem()
+    p.dtype, p.mask_dtype, p.scale_kind = _abi.BF16, _abi.BF16, _abi.SCALE_DEFAULT
+    p.bw, p.heads, p.n, p.head_dim, p.n_windows = bw, heads, n, 32, 1
+    fake = 0x10000  # never dereferenced by fwa2_validate
+    t4 = lambda: _abi.Tensor4(fake, heads * n * 32, n * 32, 32)
+    p.q, p.k, p.v, p.o = t4(), t4(), t4(), t4()
+    p.lse, p.lse_stride_bw, p.lse_stride_h = fake, heads * n, n
+    if backward:
+        p.d_o, p.dq, p.dk, p.dv = t4(), t4(), t4(), t4()
+        p.workspace, p.workspace_bytes = 0x100000, 1 << 30
+    return p
+
+
+def test_validate_accepts_and_rejects(lib):
+    assert lib.fwa2_validate(_good_problem(), 0) == _abi.OK
+    assert lib.fwa2_validate(_good_problem(backward=True), 1) == _abi.OK
+
+    p = _good_problem()
+    p.dtype = _abi.F32
+    assert lib.fwa2_validate(p, 0) == _abi.ERR_INVALID_ARGUMENT and b"fp16 and bf16" in lib.fwa2_last_error()
+
+    p = _good_problem()
+    p.head_dim = 256
+    assert lib.fwa2_validate(p, 0) == _abi.ERR_INVALID_ARGUMENT and b"up to 128" in lib.fwa2_last_error()
+
+    p = _good_problem()
+    p.head_dim = 64
+    assert lib.fwa2_validate(p, 0) == _abi.ERR_UNSUPPORTED
+
+    p = _good_problem()
+    p.q = _abi.Tensor4(0x10002, 4096, 2048, 32)  # rows not 16-byte aligned
+    assert lib.fwa2_validate(p, 0) == _abi.ERR_UNSUPPORTED
+
+    p = _good_problem()
+    p.scale_kind = _abi.SCALE_TENSOR  # without a pointer
+    assert lib.fwa2_validate(p, 0) == _abi.ERR_INVALID_ARGUMENT
+
+    p = _good_problem(bw=9)
+    p.mask = _abi.Tensor3(0x10000, 64 * 64, 64)
+    p.n_windows = 4  # 9 % 4 != 0
+    assert lib.fwa2_validate(p, 0) == _abi.ERR_INVALID_ARGUMENT and b"multiple of n_windows" in lib.fwa2_last_error()
+
+    p = _good_problem(backward=True)
+    p.bias = _abi.Tensor3(0x10000, 64 * 64, 64)  # bias without dbias / workspace
+    assert lib.fwa2_validate(p, 1) == _abi.ERR_INVALID_ARGUMENT
+
+
+def test_workspace_size_is_reported(lib):
+    p = _good_problem(n=256, bw=4096, heads=3, backward=True)
+    p.bias = _abi.Tensor3(0x10000, 65536, 256)
+    need = lib.fwa2_backward_workspace_bytes(p)
+    # one fp32 [256, 256] partial per persistent workgroup plus the transposed bias
+    assert 3 * 256 * 256 * 4 < need < 512 * 1024 * 1024
+    p.workspace, p.workspace_bytes, p.dbias = 0x100000, need - 1, 0x20000
+    assert lib.fwa2_validate(p, 1) == _abi.ERR_INVALID_ARGUMENT and b"workspace" in lib.fwa2_last_error()
+    p.workspace_bytes = need
+    assert lib.fwa2_validate(p, 1) == _abi.OK
+
+
+def test_status_to_exception(lib):
+    p = _good_problem()
+    p.head_dim = 64
+    with pytest.raises(NotImplementedError):
+        _abi.check(lib.fwa2_validate(p, 0), "validate")
+    p.head_dim = 200
+    with pytest.raises(AssertionError):
+        _abi.check(lib.fwa2_validate(p, 0), "validate")
+
+
+def test_function_rejects_bad_arguments_on_cpu():
+    """The reference asserts before launching (attn_kernel_forward.py:265-292);
+    so does this Function, which lets the checks run without a GPU."""
+    import torch
+
+    from flash_window_attention_v2_amd import flash_win_attn_v2_func
+
+    q = torch.randn(4, 2, 64, 32, dtype=torch.bfloat16)
+    with pytest.raises(AssertionError):            # CPU tensors
+        flash_win_attn_v2_func(q, q, q)
+    with pytest.raises(AssertionError):            # fp32 inputs
+        flash_win_attn_v2_func(q.float(), q.float(), q.float())
+    with pytest.raises(AssertionError):            # mixed dtypes
+        flash_win_attn_v2_func(q, q.half(), q)
+    with pytest.raises(AssertionError):            # logit_scale must be a tensor
+        flash_win_attn_v2_func(q, q, q, 1.0)

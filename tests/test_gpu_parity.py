@@ -1,0 +1,265 @@
+"""Parity of the gfx950 kernels (through the C ABI) with the classic fp32 oracle.
+
+Tolerances (stated by the task): bf16 -- max abs error <= 2e-2 on the output,
+<= 5e-2 relative (max |x - ref| / max |ref|) on dq, dk, dv, dbias, dlogit_scale;
+fp16 -- 5e-3 and 2e-2.  The oracle consumes the already-rounded low-precision
+inputs upcast to fp32, so input quantisation is not charged to the kernels.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import window_attention_np as wa
+from oracle.classic_torch import classic_fwd_bwd, win_attention_classic
+from oracle.swin_inputs import CONFIGS, make_inputs, shifted_window_mask
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.bfloat16: (2e-2, 5e-2), torch.float16: (5e-3, 2e-2)}
+GRADS = (("dq", "q"), ("dk", "k"), ("dv", "v"), ("dbias", "bias"), ("dscale", "logit_scale"))
+
+
+def _func():
+    from flash_window_attention_v2_amd import flash_win_attn_v2_func
+
+    return flash_win_attn_v2_func
+
+
+def _to_dev(inp, grad=True):
+    dev = {k: (None if v is None else v.cuda()) for k, v in inp.items()}
+    if grad:
+        for name in ("q", "k", "v", "bias", "logit_scale"):
+            if dev[name] is not None:
+                dev[name].requires_grad_(True)
+    return dev
+
+
+def _rel(got, ref):
+    ref = ref.float().cpu()
+    return float((got.float().cpu() - ref).abs().max() / ref.abs().max().clamp_min(1e-20))
+
+
+def _run_and_check(inp, dtype, backward=True, tag=""):
+    tol_o, tol_g = TOL[dtype]
+    ref = classic_fwd_bwd(inp["q"], inp["k"], inp["v"], inp["logit_scale"], inp["bias"], inp["mask"], inp["do"])
+    dev = _to_dev(inp, grad=backward)
+    o = _func()(dev["q"], dev["k"], dev["v"], dev["logit_scale"], dev["bias"], dev["mask"])
+    assert o.shape == dev["q"].shape and o.dtype == dtype
+    err = float((o.detach().float().cpu() - ref["o"]).abs().max())
+    assert err <= tol_o, f"{tag} forward max abs err {err}"
+    if not backward:
+        return
+    o.backward(dev["do"])
+    torch.cuda.synchronize()
+    for gname, tname in GRADS:
+        if dev[tname] is None:
+            continue
+        g = dev[tname].grad
+        assert g is not None and g.shape == dev[tname].shape and g.dtype == dtype
+        r = _rel(g, ref[gname])
+        assert r <= tol_g, f"{tag} {gname} relative err {r}"
+    assert dev["mask"] is None or dev["mask"].grad is None
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_config1_shape(dtype):
+    """BASELINE config 1 (B2, 16 windows of 8x8, H4, d32, shift 4) on the GPU in low precision."""
+    _run_and_check(make_inputs(**CONFIGS["C1"], dtype=dtype, seed=1), dtype, tag="C1")
+
+
+@pytest.mark.parametrize("n,res,win,shift", [(64, 16, 8, 4), (256, 32, 16, 8), (144, 24, 12, 6), (49, 14, 7, 3),
+                                             (16, 8, 4, 2)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_window_sizes_with_shift_mask(n, res, win, shift, dtype):
+    nw = (res // win) ** 2
+    inp = make_inputs(batch=2, n_windows=nw, heads=3, n=n, dtype=dtype, seed=n, resolution=res, window=win, shift=shift)
+    _run_and_check(inp, dtype, tag=f"N{n}")
+
+
+@pytest.mark.parametrize("with_scale,with_bias,with_mask", [(0, 1, 1), (1, 0, 1), (1, 1, 0), (0, 0, 0), (0, 0, 1)])
+def test_optional_arguments(with_scale, with_bias, with_mask):
+    inp = make_inputs(batch=2, n_windows=4, heads=2, n=64, dtype=torch.bfloat16, seed=5, resolution=16, window=8, shift=4,
+                      with_scale=bool(with_scale), with_bias=bool(with_bias), with_mask=bool(with_mask))
+    _run_and_check(inp, torch.bfloat16, tag=f"opt{with_scale}{with_bias}{with_mask}")
+
+
+def test_fp32_mask_and_odd_group_counts():
+    """mask may be fp32 with low-precision q/k/v (attn_kernel_forward.py:287); BW=5 is not a
+    multiple of the number of persistent workgroups."""
+    inp = make_inputs(batch=5, n_windows=1, heads=3, n=64, dtype=torch.bfloat16, seed=6, with_mask=False)
+    g = torch.Generator().manual_seed(9)
+    inp["mask"] = torch.where(torch.rand(1, 64, 64, generator=g) < 0.3, -100.0, 0.0)  # fp32
+    _run_and_check(inp, torch.bfloat16, tag="fp32mask")
+
+
+def test_random_inf_mask_and_random_scale():
+    """The reference's own check protocol: randn bias and logit_scale, ~half the mask entries -inf
+    (benchmark/check.py:23-33), here with every row keeping at least one open key."""
+    dtype = torch.float16
+    g = torch.Generator().manual_seed(3)
+    bw, nw, h, n, d = 8, 4, 3, 64, 32
+    rnd = lambda *s: torch.randn(*s, generator=g)
+    mask = torch.zeros(nw, n, n).masked_fill(rnd(nw, n, n) < 0, -float("inf"))
+    mask[:, torch.arange(n), torch.arange(n)] = 0.0
+    inp = {"q": rnd(bw, h, n, d).to(dtype), "k": rnd(bw, h, n, d).to(dtype), "v": rnd(bw, h, n, d).to(dtype),
+           "do": -torch.ones(bw, h, n, d).to(dtype), "bias": rnd(h, n, n).to(dtype),
+           "logit_scale": rnd(h, 1, 1).to(dtype), "mask": mask.to(dtype)}
+    _run_and_check(inp, dtype, tag="check.py protocol")
+
+
+def test_fully_masked_rows_and_clamped_scale():
+    dtype = torch.bfloat16
+    inp = make_inputs(batch=2, n_windows=2, heads=2, n=64, dtype=dtype, seed=8, with_mask=False)
+    mask = torch.zeros(2, 64, 64)
+    mask[1, 5, :] = -float("inf")
+    inp["mask"] = mask.to(dtype)
+    inp["logit_scale"] = torch.tensor([5.0, math.log(50.0)]).view(2, 1, 1).to(dtype)  # head 0 above ln 100
+    dev = _to_dev(inp)
+    o = _func()(dev["q"], dev["k"], dev["v"], dev["logit_scale"], dev["bias"], dev["mask"])
+    o.backward(dev["do"])
+    torch.cuda.synchronize()
+    assert torch.all(o[1::2, :, 5] == 0), "fully masked rows give zeros (attn_kernel_forward.py:233)"
+    for t in ("q", "k", "v", "bias", "logit_scale"):
+        assert torch.isfinite(dev[t].grad).all(), t
+    assert float(dev["logit_scale"].grad[0]) == 0.0 and float(dev["logit_scale"].grad[1]) != 0.0
+    # against the float64 oracle, which shares the zero-row convention
+    f64 = lambda x: None if x is None else x.double().numpy()
+    oo, lse = wa.forward(f64(inp["q"]), f64(inp["k"]), f64(inp["v"]), f64(inp["logit_scale"]), f64(inp["bias"]),
+                         f64(inp["mask"]))
+    assert float(np.abs(o.detach().float().cpu().numpy() - oo).max()) <= 2e-2
+    gr = wa.backward(f64(inp["q"]), f64(inp["k"]), f64(inp["v"]), f64(inp["do"]), f64(inp["logit_scale"]),
+                     f64(inp["bias"]), f64(inp["mask"]))
+    for gname, tname in GRADS:
+        ref = torch.from_numpy(gr[gname])
+        assert _rel(dev[tname].grad, ref) <= 5e-2, gname
+
+
+def test_lse_matches_oracle():
+    from flash_window_attention_v2_amd.flash_window_attention_v2 import FlashWindowAttentionV2
+
+    inp = make_inputs(batch=2, n_windows=4, heads=2, n=144, dtype=torch.bfloat16, seed=2, with_mask=False)
+    dev = _to_dev(inp, grad=False)
+
+    class Ctx:
+        def save_for_backward(self, *t):
+            self.saved = t
+
+    ctx = Ctx()
+    FlashWindowAttentionV2.forward(ctx, dev["q"], dev["k"], dev["v"], dev["logit_scale"], dev["bias"], None)
+    lse = ctx.saved[4]
+    assert lse.shape == (8, 2, 192) and lse.dtype == torch.float32      # N rounded up to 64
+    f64 = lambda x: x.double().numpy()
+    _, ref = wa.forward(f64(inp["q"]), f64(inp["k"]), f64(inp["v"]), f64(inp["logit_scale"]), f64(inp["bias"]))
+    assert float(np.abs(lse[:, :, :144].cpu().numpy() - ref).max()) <= 2e-2
+
+
+def test_strided_qkv_views_like_swin():
+    """q, k, v as non-contiguous views of one [B_, N, 3, H, d] buffer (swin_transformer_v2.py:279-281);
+    the output keeps q's stride order so the caller's transpose+reshape is free."""
+    dtype = torch.bfloat16
+    bw, n, h, d = 8, 64, 3, 32
+    g = torch.Generator().manual_seed(4)
+    qkv = torch.randn(bw, n, 3, h, d, generator=g).to(dtype)
+    inp = make_inputs(batch=2, n_windows=4, heads=h, n=n, dtype=dtype, seed=4, resolution=16, window=8, shift=4)
+    q, k, v = qkv.permute(2, 0, 3, 1, 4)
+    ref = classic_fwd_bwd(q, k, v, inp["logit_scale"], inp["bias"], inp["mask"], inp["do"])
+    dqkv = qkv.cuda().requires_grad_(True)
+    dq_, dk_, dv_ = dqkv.permute(2, 0, 3, 1, 4)
+    assert not dq_.is_contiguous()
+    dev = _to_dev(inp)
+    o = _func()(dq_, dk_, dv_, dev["logit_scale"], dev["bias"], dev["mask"])
+    assert o.stride() == (n * h * d, d, h * d, 1)
+    assert o.transpose(1, 2).reshape(bw, n, h * d).data_ptr() == o.data_ptr()
+    o.backward(dev["do"])
+    assert float((o.detach().float().cpu() - ref["o"]).abs().max()) <= 2e-2
+    got = dqkv.grad.permute(2, 0, 3, 1, 4)
+    for i, name in enumerate(("dq", "dk", "dv")):
+        assert _rel(got[i], ref[name]) <= 5e-2, name
+
+
+def test_backward_is_deterministic_and_reentrant():
+    inp = make_inputs(batch=4, n_windows=4, heads=3, n=256, dtype=torch.bfloat16, seed=7, resolution=32, window=16, shift=8)
+    outs = []
+    for _ in range(2):
+        dev = _to_dev(inp)
+        o = _func()(dev["q"], dev["k"], dev["v"], dev["logit_scale"], dev["bias"], dev["mask"])
+        o.backward(dev["do"])
+        outs.append([o.detach()] + [dev[t].grad for t in ("q", "k", "v", "bias", "logit_scale")])
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)          # no atomics on global memory: bit-identical reruns
+
+
+def test_recompute_under_checkpoint():
+    """use_checkpoint re-runs forward during backward (swin_transformer_v2.py:593-594)."""
+    from torch.utils.checkpoint import checkpoint
+
+    inp = make_inputs(batch=2, n_windows=4, heads=2, n=64, dtype=torch.bfloat16, seed=12, resolution=16, window=8, shift=4)
+    dev = _to_dev(inp)
+    o = checkpoint(_func(), dev["q"], dev["k"], dev["v"], dev["logit_scale"], dev["bias"], dev["mask"], use_reentrant=False)
+    o.backward(dev["do"])
+    ref = classic_fwd_bwd(inp["q"], inp["k"], inp["v"], inp["logit_scale"], inp["bias"], inp["mask"], inp["do"])
+    assert _rel(dev["q"].grad, ref["dq"]) <= 5e-2 and _rel(dev["bias"].grad, ref["dbias"]) <= 5e-2
+
+
+def test_large_windows_forward():
+    """N = 576 and 1024 (window 24 and 32 of the sweep): several LDS key chunks per workgroup."""
+    for n in (576, 1024):
+        inp = make_inputs(batch=1, n_windows=2, heads=2, n=n, dtype=torch.bfloat16, seed=n, with_mask=False)
+        _run_and_check(inp, torch.bfloat16, backward=False, tag=f"N{n}")
+
+
+def _classic_on_gpu_fp32(dev, chunk):
+    """The oracle's classic path in fp32 run on the device, over batch chunks (same code as the
+    CPU oracle; the device only makes the full benchmark sizes finish in seconds)."""
+    nw = dev["mask"].shape[0] if dev["mask"] is not None else 1
+    assert chunk % nw == 0
+    bw = dev["q"].shape[0]
+    out = {"o": [], "dq": [], "dk": [], "dv": [], "dbias": 0, "dscale": 0}
+    for s in range(0, bw, chunk):
+        sl = slice(s, s + chunk)
+        r = classic_fwd_bwd(dev["q"][sl], dev["k"][sl], dev["v"][sl], dev["logit_scale"], dev["bias"], dev["mask"],
+                            dev["do"][sl])
+        for name in ("o", "dq", "dk", "dv"):
+            out[name].append(r[name])
+        out["dbias"] = out["dbias"] + r["dbias"]
+        out["dscale"] = out["dscale"] + r["dscale"]
+    for name in ("o", "dq", "dk", "dv"):
+        out[name] = torch.cat(out[name])
+    return out
+
+
+@pytest.mark.parametrize("cfg", ["C2", "C3"])
+def test_full_benchmark_shapes(cfg):
+    """BASELINE configs 2 and 3 at full size (BW = 4096, H = 3, N = 64 / 256, bf16, shift mask)."""
+    dtype = torch.bfloat16
+    inp = make_inputs(**CONFIGS[cfg], dtype=dtype, seed=0)
+    dev = _to_dev(inp)
+    o = _func()(dev["q"], dev["k"], dev["v"], dev["logit_scale"], dev["bias"], dev["mask"])
+    o.backward(dev["do"])
+    torch.cuda.synchronize()
+    with torch.no_grad():
+        plain = {k: (None if v is None else v.detach()) for k, v in dev.items()}
+    ref = _classic_on_gpu_fp32(plain, chunk=256 if cfg == "C3" else 1024)
+    err = float((o.detach().float() - ref["o"]).abs().max())
+    assert err <= 2e-2, f"{cfg} forward max abs err {err}"
+    for gname, tname in GRADS:
+        r = float((dev[tname].grad.float() - ref[gname]).abs().max() / ref[gname].abs().max())
+        assert r <= 5e-2, f"{cfg} {gname} rel err {r}"
+    # size-independent properties at full size: gradients orthogonal to q and k, dbias rows sum to 0
+    qf, kf = dev["q"].detach().float(), dev["k"].detach().float()
+    dq, dk = dev["q"].grad.float(), dev["k"].grad.float()
+    cosq = (dq * qf).sum(-1).abs() / (dq.norm(dim=-1) * qf.norm(dim=-1) + 1e-20)
+    cosk = (dk * kf).sum(-1).abs() / (dk.norm(dim=-1) * kf.norm(dim=-1) + 1e-20)
+    assert float(cosq.max()) < 2e-2 and float(cosk.max()) < 2e-2
+    db = dev["bias"].grad.float()
+    assert float(db.sum(-1).abs().max()) <= 2e-2 * float(db.abs().max()) * math.sqrt(db.shape[-1])
+    # no worse than the eager classic path run in the same low precision (proxy for the reference's claim)
+    with torch.no_grad():
+        sl = slice(0, 256)
+        low = win_attention_classic(plain["q"][sl], plain["k"][sl], plain["v"][sl], plain["logit_scale"], plain["bias"],
+                                    plain["mask"])
+        err_low = float((low.float() - ref["o"][sl]).abs().max())
+        err_hip = float((o.detach()[sl].float() - ref["o"][sl]).abs().max())
+    assert err_hip <= max(err_low, 2e-2)
