@@ -15,8 +15,8 @@
 //   load     q, k (L2-normalised, q additionally times s*log2e), dO -> LDS in
 //            the input dtype; delta = rowsum(o*dO) and lse*log2e -> LDS.
 //   phase A  S = Q_hat K_hat^T and dP = dO V^T with v_mfma_f32_16x16x32
-//            (rows = queries, columns = this wave's keys), P = 2^(S+bias+mask-lse),
-//            dZ = P (dP - delta); dbias registers += dZ; the accumulators,
+//            (rows = queries, columns = this wave's keys; -lse and -delta ride in as
+//            the accumulator inits), P = 2^(S+bias+mask-lse), dZ = P (dP - delta); dbias registers += dZ; the accumulators,
 //            rounded to the input dtype, are directly the B operands (k =
 //            queries) of dV^T += dO^T P and dK_hat^T += Q_hat^T dZ, whose A
 //            operands come out of the row-major LDS tiles with
@@ -58,29 +58,30 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
     typedef typename Elem<DT>::V8 V8;
     typedef typename Elem<DT>::V4 V4;
     typedef typename MaskElemB<DT, MASK_DT>::E ME;
-    typedef ME MV8 __attribute__((ext_vector_type(8)));
+    typedef ME MV4 __attribute__((ext_vector_type(4)));
 
     const int N = p.n;
-    const int R = (N + 31) & ~31;          // padded query rows (and LDS rows)
+    constexpr int R = 32 * NQB;            // padded rows of every LDS tile and of the key-major side tables
     const int NPk = p.waves * 16 * KT;     // padded key rows
-    const int nqb = R >> 5;                // query blocks of 32
-    const int nks = R >> 5;                // key steps of 32 in phase B
+    const int nqb = (N + 31) >> 5;         // query blocks of 32 that hold real rows
+    const int nks = nqb;                   // key steps of 32 in phase B
 
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-    E* Qs = reinterpret_cast<E*>(smem_raw);
-    E* Ks = Qs + R * kRow;
-    E* dOs = Ks + R * kRow;
-    E* dZs = dOs + R * kRow;               // 2 buffers
-    float* lse2s = reinterpret_cast<float*>(dZs + 2 * R * kRow);
-    float* deltas = lse2s + R;
-    float* red = deltas + R;               // [16]
+    // compile-time LDS layout: every tile address is a lane offset plus an immediate
+    __shared__ __attribute__((aligned(16))) E Qs[R * kRow];
+    __shared__ __attribute__((aligned(16))) E Ks[R * kRow];
+    __shared__ __attribute__((aligned(16))) E dOs[R * kRow];
+    __shared__ __attribute__((aligned(16))) E dZs[2 * R * kRow];
+    __shared__ __attribute__((aligned(16))) float lse2s[R];
+    __shared__ __attribute__((aligned(16))) float deltas[R];
+    __shared__ float red[16];
 
     const int tid = threadIdx.x;
     const int nthreads = blockDim.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
-    const int l16 = lane & 15;
-    const int g = lane >> 4;
+    const int l16_0 = lane & 15;
+    const int g_0 = lane >> 4;
+    int l16 = l16_0, g = g_0;
 
     const int h = blockIdx.x / p.groups;
     const int grp = blockIdx.x - h * p.groups;
@@ -95,6 +96,7 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
     const float scale2 = s_true * kLog2e;
 
     const int key0 = wave * 16 * KT + l16;  // this lane's key in key tile 0 (tile kt: + 16 kt)
+    const bool tail_keys = NPk > N;         // some key columns are padding
 
     float dbacc[NQB][KT][8];
 #pragma unroll
@@ -104,6 +106,9 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
 #pragma unroll
             for (int j = 0; j < 8; j++) dbacc[a][kt][j] = 0.f;
     float ds_part = 0.f;
+    // bit (2 qb + qt) set: this wavefront finishes dq for queries 32 qb + 16 qt .. + 16
+    uint32_t my_jobs = 0;
+    for (int j = wave; j < 2 * NQB; j += p.waves) my_jobs |= 1u << j;
 
     // dZ staging rows that no wavefront writes must read as zeros in phase B
     for (int i = tid; i < 2 * R * kRow / 8; i += nthreads) st8<V8>(dZs + i * 8, zero8<V8>());
@@ -128,6 +133,10 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
             mask_t = reinterpret_cast<const ME*>(p.mask_t) + ((int64_t)w * NPk + key0) * R;
         }
 
+        // lane-derived values are re-materialised per unit so that the compiler does not keep
+        // dozens of per-block addresses alive (and spilled) across the whole unit loop
+        l16 = l16_0; g = g_0;
+        asm volatile("" : "+v"(l16), "+v"(g));
         __syncthreads();   // the previous unit is done with LDS
         // ---- load: one 8-element chunk of one row per thread and pass ----
         for (int r = tid >> 2; r < R; r += nthreads >> 2) {
@@ -152,10 +161,10 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
             st8<V8>(Qs + r * kRow + dc, qn);
             st8<V8>(Ks + r * kRow + dc, kn);
             st8<V8>(dOs + r * kRow + dc, do8);
-            if ((tid & 3) == 0) deltas[r] = dl;
+            if ((tid & 3) == 0) deltas[r] = -dl;
             if ((tid & 3) == 1) {
-                float l2 = INFINITY;           // padded / fully masked rows: P = 0
-                if (r < N) { const float l = lseptr[r]; l2 = (l == -INFINITY) ? INFINITY : l * kLog2e; }
+                float l2 = -INFINITY;          // padded / fully masked rows: P = 0
+                if (r < N) { const float l = lseptr[r]; l2 = (l == -INFINITY) ? -INFINITY : -l * kLog2e; }
                 lse2s[r] = l2;
             }
         }
@@ -184,74 +193,65 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
                 E* dZbuf = dZs + (qb & 1) * R * kRow;
                 const int q8 = 32 * qb + 8 * g;          // first of this lane's 8 queries
                 // ---- phase A ----
-                V8 aq[2], ado[2];
+                V8 p8[KT], z8[KT];
 #pragma unroll
                 for (int t = 0; t < 2; t++) {
                     const int rowq = 32 * qb + 8 * (l16 >> 2) + 4 * t + (l16 & 3);
-                    aq[t] = ld8<V8>(Qs + rowq * kRow + 8 * g);
-                    ado[t] = ld8<V8>(dOs + rowq * kRow + 8 * g);
-                }
-                const f32x4 la = *reinterpret_cast<const f32x4*>(lse2s + q8);
-                const f32x4 lb = *reinterpret_cast<const f32x4*>(lse2s + q8 + 4);
-                const f32x4 da = *reinterpret_cast<const f32x4*>(deltas + q8);
-                const f32x4 db = *reinterpret_cast<const f32x4*>(deltas + q8 + 4);
-                V8 p8[KT], z8[KT];
+                    const V8 aq = ld8<V8>(Qs + rowq * kRow + 8 * g);
+                    const V8 ado = ld8<V8>(dOs + rowq * kRow + 8 * g);
+                    // accumulator inits: -lse*log2e and -delta of this lane's 4 queries
+                    const f32x4 nl = *reinterpret_cast<const f32x4*>(lse2s + q8 + 4 * t);
+                    const f32x4 nd = *reinterpret_cast<const f32x4*>(deltas + q8 + 4 * t);
 #pragma unroll
-                for (int kt = 0; kt < KT; kt++) {
-                    const bool key_ok = key0 + 16 * kt < N;
-                    f32x4 sacc[2], pacc[2];
+                    for (int kt = 0; kt < KT; kt++) {
+                        f32x4 sacc = Elem<DT>::mfma16(aq, bk[kt], nl);     // S*log2e - lse*log2e
+                        const f32x4 pacc = Elem<DT>::mfma16(ado, bv[kt], nd);  // dP - delta
+                        if (HAS_BIAS) {
+                            const V4 b4 = *reinterpret_cast<const V4*>(bias_t + (int64_t)16 * kt * R + q8 + 4 * t);
 #pragma unroll
-                    for (int t = 0; t < 2; t++) {
-                        const f32x4 z = {0.f, 0.f, 0.f, 0.f};
-                        sacc[t] = Elem<DT>::mfma16(aq[t], bk[kt], z);
-                        pacc[t] = Elem<DT>::mfma16(ado[t], bv[kt], z);
-                    }
-                    float zz[8];
+                            for (int i = 0; i < 4; i++) sacc[i] = fmaf((float)b4[i], kLog2e, sacc[i]);
+                        }
+                        if (MASK_DT >= 0) {
+                            if (mask_on) {
+                                const MV4 m4 = *reinterpret_cast<const MV4*>(mask_t + (int64_t)16 * kt * R + q8 + 4 * t);
 #pragma unroll
-                    for (int j = 0; j < 8; j++) zz[j] = sacc[j >> 2][j & 3];
-                    if (HAS_BIAS) {
-                        float x[8];
-                        unpack8b(ld8<V8>(bias_t + (int64_t)16 * kt * R + q8), x);
+                                for (int i = 0; i < 4; i++) sacc[i] = fmaf((float)m4[i], kLog2e, sacc[i]);
+                            }
+                        }
+                        if (tail_keys) {
+                            if (key0 + 16 * kt >= N) {
 #pragma unroll
-                        for (int j = 0; j < 8; j++) zz[j] = fmaf(x[j], kLog2e, zz[j]);
-                    }
-                    if (MASK_DT >= 0) {
-                        if (mask_on) {
-                            const MV8 mv = *reinterpret_cast<const MV8*>(mask_t + (int64_t)16 * kt * R + q8);
+                                for (int i = 0; i < 4; i++) sacc[i] = -INFINITY;
+                            }
+                        }
 #pragma unroll
-                            for (int j = 0; j < 8; j++) zz[j] = fmaf((float)mv[j], kLog2e, zz[j]);
+                        for (int i = 0; i < 4; i++) {
+                            const float pj = fast_exp2(sacc[i]);
+                            const float dz = pj * pacc[i];
+                            if (HAS_BIAS) dbacc[qb][kt][4 * t + i] += dz;
+                            p8[kt][4 * t + i] = (E)pj;
+                            z8[kt][4 * t + i] = (E)dz;
                         }
                     }
-#pragma unroll
-                    for (int j = 0; j < 8; j++) {
-                        const float l2 = j < 4 ? la[j & 3] : lb[j & 3];
-                        const float dl = j < 4 ? da[j & 3] : db[j & 3];
-                        const float zin = key_ok ? zz[j] : -INFINITY;
-                        const float pj = fast_exp2(zin - l2);
-                        const float dz = pj * (pacc[j >> 2][j & 3] - dl);
-                        if (HAS_BIAS) dbacc[qb][kt][j] += dz;
-                        p8[kt][j] = (E)pj;
-                        z8[kt][j] = (E)dz;
-                    }
-                    st8<V8>(dZbuf + (key0 + 16 * kt) * kRow + 8 * g, z8[kt]);
                 }
+#pragma unroll
+                for (int kt = 0; kt < KT; kt++) st8<V8>(dZbuf + (key0 + 16 * kt) * kRow + 8 * g, z8[kt]);
 #pragma unroll
                 for (int dt = 0; dt < 2; dt++) {
                     const int off = (q8 + (l16 >> 2)) * kRow + 16 * dt + 4 * (l16 & 3);
                     const V8 a_do = lds_tr8<DT>(dOs + off, dOs + off + 4 * kRow);
+#pragma unroll
+                    for (int kt = 0; kt < KT; kt++) dvacc[kt][dt] = Elem<DT>::mfma16(a_do, p8[kt], dvacc[kt][dt]);
                     const V8 a_q = lds_tr8<DT>(Qs + off, Qs + off + 4 * kRow);
 #pragma unroll
-                    for (int kt = 0; kt < KT; kt++) {
-                        dvacc[kt][dt] = Elem<DT>::mfma16(a_do, p8[kt], dvacc[kt][dt]);
-                        dkacc[kt][dt] = Elem<DT>::mfma16(a_q, z8[kt], dkacc[kt][dt]);
-                    }
+                    for (int kt = 0; kt < KT; kt++) dkacc[kt][dt] = Elem<DT>::mfma16(a_q, z8[kt], dkacc[kt][dt]);
                 }
                 __syncthreads();
                 // ---- phase B: dQ_hat^T for 16 queries (all d, all keys), one wavefront per job,
                 //      then straight through the normalisation Jacobian to global memory ----
 #pragma unroll
                 for (int qt = 0; qt < 2; qt++) {
-                    if ((2 * qb + qt) % p.waves == wave) {
+                    if ((my_jobs >> (2 * qb + qt)) & 1u) {
                         f32x4 acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
                         for (int ks = 0; ks < nks; ks++) {
                             const int rowk = (32 * ks + 8 * g + (l16 >> 2)) * kRow;
@@ -452,9 +452,9 @@ struct BwdPlan {
 
 static BwdPlan make_plan(int heads, int n, int bw, bool has_bias, bool has_mask, int n_windows, int cus) {
     BwdPlan pl;
-    pl.r = (n + 31) & ~31;
-    const int nqb = pl.r / 32;
+    const int nqb = (n + 31) / 32;
     pl.nqb_t = nqb <= 2 ? 2 : (nqb <= 4 ? 4 : 8);
+    pl.r = 32 * pl.nqb_t;
     // up to 128 queries a wavefront owns one 16-key tile (<= 128 registers, several workgroups
     // per CU); above that two tiles (<= 256 registers, one workgroup of 8 wavefronts per CU)
     pl.kt = nqb <= 4 ? 1 : 2;
@@ -475,7 +475,7 @@ static BwdPlan make_plan(int heads, int n, int bw, bool has_bias, bool has_mask,
     pl.off_mask_t = off;
     if (has_mask) off += align256((size_t)n_windows * pl.npk * pl.r * 4);
     pl.total = off;
-    pl.smem = (size_t)5 * pl.r * kRow * 2 + (size_t)2 * pl.r * 4 + 16 * 4;
+    pl.smem = 0;   // the kernels use static LDS
     return pl;
 }
 
@@ -487,11 +487,6 @@ size_t backward_workspace_bytes(int heads, int n, int bw, bool has_bias, bool ha
 template <int DT, bool HAS_BIAS, int MASK_DT, int NQB, int KT>
 static hipError_t launch_main(const BwdParams& p, const BwdPlan& pl, hipStream_t st) {
     auto kern = bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT>;
-    if (pl.smem > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)pl.smem);
-        if (e != hipSuccess) return e;
-    }
     if (p.ev_start) (void)hipEventRecord(p.ev_start, st);
     hipLaunchKernelGGL(kern, dim3(p.heads * pl.groups), dim3(64 * pl.waves), pl.smem, st, p);
     if (p.ev_stop) (void)hipEventRecord(p.ev_stop, st);
