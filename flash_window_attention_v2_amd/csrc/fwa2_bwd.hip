@@ -30,6 +30,8 @@
 //
 // bias and mask are read key-major (transposed once per call by a small
 // pre-pass into the workspace) so that a lane's 8 scores are one 16-byte load.
+#include <type_traits>
+
 #include "fwa2_common.hpp"
 
 namespace fwa2 {
@@ -51,6 +53,195 @@ __device__ __forceinline__ float wave_sum(float x) {
     return x;
 }
 
+// Per-wavefront state that lives in registers across the query blocks of one unit (dvacc,
+// dkacc, bk, bv) or across all units of the workgroup (dbacc).
+template <int DT, int NQB, int KT>
+struct WaveRegs {
+    float dbacc[NQB][KT][8];
+    f32x4 dvacc[KT][2], dkacc[KT][2];
+    typename Elem<DT>::V8 bk[KT], bv[KT];
+};
+
+// LDS of one workgroup; all sizes are compile-time so tile addresses are lane offset + immediate.
+template <int DT, int NQB>
+struct BwdLds {
+    typedef typename Elem<DT>::E E;
+    static constexpr int R = 32 * NQB;
+    E Qs[R * kRow];          // q_hat * s * log2e, row-major [query][d]
+    E Ks[R * kRow];          // k_hat, [key][d]
+    E dOs[R * kRow];         // dO, [query][d]
+    E dZs[2][R * kRow];      // dZ of one query block, [key][32 queries], double buffered
+    f32x4 parts[2][2][4][64];// partial dQ_hat^T tiles: [buffer][key split][dt + 2 qt][lane]
+    float nlse2[R];          // -lse * log2e   (-inf for padded / fully masked rows)
+    float ndelta[R];         // -rowsum(o * dO)
+    float red[16];
+};
+
+struct UnitPtrs {
+    const void *q, *k;       // this unit's q and k rows (for the normalisation Jacobians)
+    void* dq;
+    int64_t q_sn, dq_sn;
+};
+
+// dq rows of 16 queries: sum the partial dQ_hat^T tiles, go back through q / max(|q|, eps).
+template <int DT, int NQB>
+__device__ __forceinline__ void finish_dq(BwdLds<DT, NQB>& L, const UnitPtrs& u, int qbr, int qt, int kh_count, int lane,
+                                          int l16, int g, int n, float s_true, float& ds_part) {
+    typedef typename Elem<DT>::E E;
+    typedef typename Elem<DT>::V4 V4;
+    const int query = 32 * qbr + 16 * qt + l16;
+    const bool q_ok = query < n;
+    float x[8], a[8];
+    float ss = 0.f, dot = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < 2; dt++) {
+        V4 q4;
+#pragma unroll
+        for (int i = 0; i < 4; i++) q4[i] = 0;
+        if (q_ok) q4 = *reinterpret_cast<const V4*>(reinterpret_cast<const E*>(u.q) + (int64_t)query * u.q_sn + 16 * dt + 4 * g);
+        f32x4 acc = L.parts[qbr & 1][0][dt + 2 * qt][lane];
+        if (kh_count > 1) acc += L.parts[qbr & 1][1][dt + 2 * qt][lane];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            x[4 * dt + i] = (float)q4[i];
+            a[4 * dt + i] = acc[i];
+            ss += x[4 * dt + i] * x[4 * dt + i];
+        }
+    }
+    ss = xor32_add(xor16_add(ss));
+    const float nrm = sqrtf(ss);
+    const float inv = 1.0f / fmaxf(nrm, kNormEps);
+#pragma unroll
+    for (int j = 0; j < 8; j++) { x[j] *= inv; dot += a[j] * x[j]; }
+    dot = xor32_add(xor16_add(dot));
+    const float proj = nrm > kNormEps ? dot : 0.f;
+    const float f = s_true * inv;
+    if (q_ok) {
+#pragma unroll
+        for (int dt = 0; dt < 2; dt++) {
+            V4 o4;
+#pragma unroll
+            for (int i = 0; i < 4; i++) o4[i] = (E)(f * (a[4 * dt + i] - x[4 * dt + i] * proj));
+            *reinterpret_cast<V4*>(reinterpret_cast<E*>(u.dq) + (int64_t)query * u.dq_sn + 16 * dt + 4 * g) = o4;
+        }
+        if (g == 0) ds_part += dot;   // sum_j dC_ij c_ij = q_hat_i . dq_hat_i  (dlogit_scale)
+    }
+}
+
+// All query blocks of one unit.  MASKED is uniform per unit (the window's mask is live or not),
+// so the whole block sequence exists twice instead of branching inside every block.
+template <int DT, bool HAS_BIAS, class ME, int NQB, int KT, bool MASKED>
+__device__ __forceinline__ void unit_blocks(BwdLds<DT, NQB>& L, WaveRegs<DT, NQB, KT>& w, const UnitPtrs& u,
+                                            const typename Elem<DT>::E* bias_t, const ME* mask_t, int n, int nqb,
+                                            int waves, int wave, int lane, int l16, int g, int key0, bool tail_keys,
+                                            uint32_t my_jobs, float s_true, float& ds_part) {
+    typedef typename Elem<DT>::E E;
+    typedef typename Elem<DT>::V8 V8;
+    typedef typename Elem<DT>::V4 V4;
+    typedef ME MV4 __attribute__((ext_vector_type(4)));
+    constexpr int R = 32 * NQB;
+    const int kh_count = waves >= 8 ? 2 : 1;          // key splits of the dQ product
+    const int nks = nqb;
+
+    // bias (and mask) values of the coming block travel in registers: they are fetched one block
+    // ahead so that the L2 round trip overlaps the rest of the block instead of stalling it
+    V4 bcur[KT][2];
+    MV4 mcur[KT][2];
+    auto fetch_side = [&](int qbn) __attribute__((always_inline)) {
+        const int q8n = 32 * qbn + 8 * g;
+#pragma unroll
+        for (int kt = 0; kt < KT; kt++)
+#pragma unroll
+            for (int t = 0; t < 2; t++) {
+                if (HAS_BIAS) bcur[kt][t] = *reinterpret_cast<const V4*>(bias_t + (int64_t)16 * kt * R + q8n + 4 * t);
+                if (MASKED) mcur[kt][t] = *reinterpret_cast<const MV4*>(mask_t + (int64_t)16 * kt * R + q8n + 4 * t);
+            }
+    };
+    fetch_side(0);
+
+#pragma unroll
+    for (int qb = 0; qb < NQB; qb++) {
+        if (qb < nqb) {
+            E* dZbuf = L.dZs[qb & 1];
+            const int q8 = 32 * qb + 8 * g;          // first of this lane's 8 queries
+            // ---- phase A, one key tile at a time ----
+#pragma unroll
+            for (int kt = 0; kt < KT; kt++) {
+                V8 p8, z8;
+#pragma unroll
+                for (int t = 0; t < 2; t++) {
+                    const int rowq = 32 * qb + 8 * (l16 >> 2) + 4 * t + (l16 & 3);
+                    const V8 aq = ld8<V8>(L.Qs + rowq * kRow + 8 * g);
+                    const V8 ado = ld8<V8>(L.dOs + rowq * kRow + 8 * g);
+                    // accumulator inits: -lse*log2e and -delta of this lane's 4 queries
+                    const f32x4 nl = *reinterpret_cast<const f32x4*>(L.nlse2 + q8 + 4 * t);
+                    const f32x4 nd = *reinterpret_cast<const f32x4*>(L.ndelta + q8 + 4 * t);
+                    f32x4 sacc = Elem<DT>::mfma16(aq, w.bk[kt], nl);          // (S - lse) * log2e
+                    const f32x4 pacc = Elem<DT>::mfma16(ado, w.bv[kt], nd);   // dP - delta
+                    if (HAS_BIAS) {   // padded key rows of bias_t hold -inf
+#pragma unroll
+                        for (int i = 0; i < 4; i++) sacc[i] = fmaf((float)bcur[kt][t][i], kLog2e, sacc[i]);
+                    }
+                    if (MASKED) {
+#pragma unroll
+                        for (int i = 0; i < 4; i++) sacc[i] = fmaf((float)mcur[kt][t][i], kLog2e, sacc[i]);
+                    }
+                    if (!HAS_BIAS) {
+                        if (tail_keys) {
+#pragma unroll
+                            for (int i = 0; i < 4; i++) sacc[i] = (key0 + 16 * kt < n) ? sacc[i] : -INFINITY;
+                        }
+                    }
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const float pj = fast_exp2(sacc[i]);
+                        const float dz = pj * pacc[i];
+                        if (HAS_BIAS) w.dbacc[qb][kt][4 * t + i] += dz;
+                        p8[4 * t + i] = (E)pj;
+                        z8[4 * t + i] = (E)dz;
+                    }
+                }
+                st8<V8>(dZbuf + (key0 + 16 * kt) * kRow + 8 * g, z8);
+#pragma unroll
+                for (int dt = 0; dt < 2; dt++) {
+                    const int off = (q8 + (l16 >> 2)) * kRow + 16 * dt + 4 * (l16 & 3);
+                    const V8 a_do = lds_tr8<DT>(L.dOs + off, L.dOs + off + 4 * kRow);
+                    w.dvacc[kt][dt] = Elem<DT>::mfma16(a_do, p8, w.dvacc[kt][dt]);
+                    const V8 a_q = lds_tr8<DT>(L.Qs + off, L.Qs + off + 4 * kRow);
+                    w.dkacc[kt][dt] = Elem<DT>::mfma16(a_q, z8, w.dkacc[kt][dt]);
+                }
+            }
+            fetch_side(qb + 1 < nqb ? qb + 1 : 0);
+            __syncthreads();
+            // ---- phase B, spread over the wavefronts: dQ_hat^T tile (dt, qt) over a share of the keys ----
+            for (int job = wave; job < 4 * kh_count; job += waves) {
+                const int tile = job & 3, kh = job >> 2;
+                const int dt = tile & 1, qt = tile >> 1;
+                f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+                for (int ks = kh; ks < nks; ks += kh_count) {
+                    const int rowk = (32 * ks + 8 * g + (l16 >> 2)) * kRow + 4 * (l16 & 3);
+                    const V8 a_k = lds_tr8<DT>(L.Ks + rowk + 16 * dt, L.Ks + rowk + 16 * dt + 4 * kRow);
+                    const V8 b_z = lds_tr8<DT>(dZbuf + rowk + 16 * qt, dZbuf + rowk + 16 * qt + 4 * kRow);
+                    acc = Elem<DT>::mfma16(a_k, b_z, acc);
+                }
+                L.parts[qb & 1][kh][tile][lane] = acc;
+            }
+            // ---- the previous block's partial tiles are complete: finish its dq rows ----
+            if (qb > 0) {
+#pragma unroll
+                for (int qt = 0; qt < 2; qt++)
+                    if ((my_jobs >> (2 * (qb - 1) + qt)) & 1u)
+                        finish_dq<DT, NQB>(L, u, qb - 1, qt, kh_count, lane, l16, g, n, s_true, ds_part);
+            }
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int qt = 0; qt < 2; qt++)
+        if ((my_jobs >> (2 * (nqb - 1) + qt)) & 1u)
+            finish_dq<DT, NQB>(L, u, nqb - 1, qt, kh_count, lane, l16, g, n, s_true, ds_part);
+}
+
 // KT = key tiles of 16 owned by one wavefront, NQB = compile-time bound on query blocks of 32.
 template <int DT, bool HAS_BIAS, int MASK_DT, int NQB, int KT>
 __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) {
@@ -58,22 +249,13 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
     typedef typename Elem<DT>::V8 V8;
     typedef typename Elem<DT>::V4 V4;
     typedef typename MaskElemB<DT, MASK_DT>::E ME;
-    typedef ME MV4 __attribute__((ext_vector_type(4)));
 
     const int N = p.n;
     constexpr int R = 32 * NQB;            // padded rows of every LDS tile and of the key-major side tables
     const int NPk = p.waves * 16 * KT;     // padded key rows
     const int nqb = (N + 31) >> 5;         // query blocks of 32 that hold real rows
-    const int nks = nqb;                   // key steps of 32 in phase B
 
-    // compile-time LDS layout: every tile address is a lane offset plus an immediate
-    __shared__ __attribute__((aligned(16))) E Qs[R * kRow];
-    __shared__ __attribute__((aligned(16))) E Ks[R * kRow];
-    __shared__ __attribute__((aligned(16))) E dOs[R * kRow];
-    __shared__ __attribute__((aligned(16))) E dZs[2 * R * kRow];
-    __shared__ __attribute__((aligned(16))) float lse2s[R];
-    __shared__ __attribute__((aligned(16))) float deltas[R];
-    __shared__ float red[16];
+    __shared__ __attribute__((aligned(16))) BwdLds<DT, NQB> L;
 
     const int tid = threadIdx.x;
     const int nthreads = blockDim.x;
@@ -98,39 +280,40 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
     const int key0 = wave * 16 * KT + l16;  // this lane's key in key tile 0 (tile kt: + 16 kt)
     const bool tail_keys = NPk > N;         // some key columns are padding
 
-    float dbacc[NQB][KT][8];
+    WaveRegs<DT, NQB, KT> w;
 #pragma unroll
     for (int a = 0; a < NQB; a++)
 #pragma unroll
         for (int kt = 0; kt < KT; kt++)
 #pragma unroll
-            for (int j = 0; j < 8; j++) dbacc[a][kt][j] = 0.f;
+            for (int j = 0; j < 8; j++) w.dbacc[a][kt][j] = 0.f;
     float ds_part = 0.f;
     // bit (2 qb + qt) set: this wavefront finishes dq for queries 32 qb + 16 qt .. + 16
     uint32_t my_jobs = 0;
     for (int j = wave; j < 2 * NQB; j += p.waves) my_jobs |= 1u << j;
 
     // dZ staging rows that no wavefront writes must read as zeros in phase B
-    for (int i = tid; i < 2 * R * kRow / 8; i += nthreads) st8<V8>(dZs + i * 8, zero8<V8>());
+    for (int i = tid; i < 2 * R * kRow / 8; i += nthreads) st8<V8>(&L.dZs[0][0] + i * 8, zero8<V8>());
 
     const E* bias_t = nullptr;
     if (HAS_BIAS) bias_t = reinterpret_cast<const E*>(p.bias_t) + ((int64_t)h * NPk + key0) * R;
 
-    for (int b = grp; b < p.bw; b += p.groups) {
+    auto process_unit = [&](auto masked_tag, int b) __attribute__((always_inline)) {
+        constexpr bool MASKED = decltype(masked_tag)::value;
         const E* qptr = reinterpret_cast<const E*>(p.q.ptr) + b * p.q.sb + h * p.q.sh;
         const E* kptr = reinterpret_cast<const E*>(p.k.ptr) + b * p.k.sb + h * p.k.sh;
         const E* vptr = reinterpret_cast<const E*>(p.v.ptr) + b * p.v.sb + h * p.v.sh;
         const E* optr = reinterpret_cast<const E*>(p.o.ptr) + b * p.o.sb + h * p.o.sh;
         const E* doptr = reinterpret_cast<const E*>(p.d_o.ptr) + b * p.d_o.sb + h * p.d_o.sh;
-        E* dqptr = reinterpret_cast<E*>(const_cast<void*>(p.dq.ptr)) + b * p.dq.sb + h * p.dq.sh;
         const float* lseptr = p.lse + b * p.lse_sb + h * p.lse_sh;
+        UnitPtrs u;
+        u.q = qptr; u.k = kptr; u.q_sn = p.q.sn; u.dq_sn = p.dq.sn;
+        u.dq = reinterpret_cast<E*>(const_cast<void*>(p.dq.ptr)) + b * p.dq.sb + h * p.dq.sh;
 
         const ME* mask_t = nullptr;
-        bool mask_on = false;
         if (MASK_DT >= 0) {
-            const int w = b % p.n_windows;
-            mask_on = p.mask_live ? (p.mask_live[w] != 0) : true;
-            mask_t = reinterpret_cast<const ME*>(p.mask_t) + ((int64_t)w * NPk + key0) * R;
+            const int wnd = b % p.n_windows;
+            mask_t = reinterpret_cast<const ME*>(p.mask_t) + ((int64_t)wnd * NPk + key0) * R;
         }
 
         // lane-derived values are re-materialised per unit so that the compiler does not keep
@@ -158,152 +341,34 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
             V8 qn, kn;
 #pragma unroll
             for (int j = 0; j < 8; j++) { qn[j] = (E)(xq[j] * iq); kn[j] = (E)(xk[j] * ik); }
-            st8<V8>(Qs + r * kRow + dc, qn);
-            st8<V8>(Ks + r * kRow + dc, kn);
-            st8<V8>(dOs + r * kRow + dc, do8);
-            if ((tid & 3) == 0) deltas[r] = -dl;
+            st8<V8>(L.Qs + r * kRow + dc, qn);
+            st8<V8>(L.Ks + r * kRow + dc, kn);
+            st8<V8>(L.dOs + r * kRow + dc, do8);
+            if ((tid & 3) == 0) L.ndelta[r] = -dl;
             if ((tid & 3) == 1) {
                 float l2 = -INFINITY;          // padded / fully masked rows: P = 0
                 if (r < N) { const float l = lseptr[r]; l2 = (l == -INFINITY) ? -INFINITY : -l * kLog2e; }
-                lse2s[r] = l2;
+                L.nlse2[r] = l2;
             }
         }
-        V8 bv[KT], bk[KT];
 #pragma unroll
         for (int kt = 0; kt < KT; kt++) {
-            bv[kt] = zero8<V8>();
-            if (key0 + 16 * kt < N) bv[kt] = ld8<V8>(vptr + (int64_t)(key0 + 16 * kt) * p.v.sn + 8 * g);
+            w.bv[kt] = zero8<V8>();
+            if (key0 + 16 * kt < N) w.bv[kt] = ld8<V8>(vptr + (int64_t)(key0 + 16 * kt) * p.v.sn + 8 * g);
         }
         __syncthreads();
 #pragma unroll
-        for (int kt = 0; kt < KT; kt++) bk[kt] = ld8<V8>(Ks + (key0 + 16 * kt) * kRow + 8 * g);
-
-        f32x4 dvacc[KT][2], dkacc[KT][2];
+        for (int kt = 0; kt < KT; kt++) w.bk[kt] = ld8<V8>(L.Ks + (key0 + 16 * kt) * kRow + 8 * g);
 #pragma unroll
         for (int kt = 0; kt < KT; kt++)
 #pragma unroll
             for (int dt = 0; dt < 2; dt++)
 #pragma unroll
-                for (int i = 0; i < 4; i++) { dvacc[kt][dt][i] = 0.f; dkacc[kt][dt][i] = 0.f; }
+                for (int i = 0; i < 4; i++) { w.dvacc[kt][dt][i] = 0.f; w.dkacc[kt][dt][i] = 0.f; }
 
-#pragma unroll
-        for (int qb = 0; qb < NQB; qb++) {
-            if (qb < nqb) {
-                __builtin_amdgcn_sched_barrier(0);   // keep the unrolled blocks apart: register pressure
-                E* dZbuf = dZs + (qb & 1) * R * kRow;
-                const int q8 = 32 * qb + 8 * g;          // first of this lane's 8 queries
-                // ---- phase A ----
-                V8 p8[KT], z8[KT];
-#pragma unroll
-                for (int t = 0; t < 2; t++) {
-                    const int rowq = 32 * qb + 8 * (l16 >> 2) + 4 * t + (l16 & 3);
-                    const V8 aq = ld8<V8>(Qs + rowq * kRow + 8 * g);
-                    const V8 ado = ld8<V8>(dOs + rowq * kRow + 8 * g);
-                    // accumulator inits: -lse*log2e and -delta of this lane's 4 queries
-                    const f32x4 nl = *reinterpret_cast<const f32x4*>(lse2s + q8 + 4 * t);
-                    const f32x4 nd = *reinterpret_cast<const f32x4*>(deltas + q8 + 4 * t);
-#pragma unroll
-                    for (int kt = 0; kt < KT; kt++) {
-                        f32x4 sacc = Elem<DT>::mfma16(aq, bk[kt], nl);     // S*log2e - lse*log2e
-                        const f32x4 pacc = Elem<DT>::mfma16(ado, bv[kt], nd);  // dP - delta
-                        if (HAS_BIAS) {
-                            const V4 b4 = *reinterpret_cast<const V4*>(bias_t + (int64_t)16 * kt * R + q8 + 4 * t);
-#pragma unroll
-                            for (int i = 0; i < 4; i++) sacc[i] = fmaf((float)b4[i], kLog2e, sacc[i]);
-                        }
-                        if (MASK_DT >= 0) {
-                            if (mask_on) {
-                                const MV4 m4 = *reinterpret_cast<const MV4*>(mask_t + (int64_t)16 * kt * R + q8 + 4 * t);
-#pragma unroll
-                                for (int i = 0; i < 4; i++) sacc[i] = fmaf((float)m4[i], kLog2e, sacc[i]);
-                            }
-                        }
-                        if (tail_keys) {
-                            if (key0 + 16 * kt >= N) {
-#pragma unroll
-                                for (int i = 0; i < 4; i++) sacc[i] = -INFINITY;
-                            }
-                        }
-#pragma unroll
-                        for (int i = 0; i < 4; i++) {
-                            const float pj = fast_exp2(sacc[i]);
-                            const float dz = pj * pacc[i];
-                            if (HAS_BIAS) dbacc[qb][kt][4 * t + i] += dz;
-                            p8[kt][4 * t + i] = (E)pj;
-                            z8[kt][4 * t + i] = (E)dz;
-                        }
-                    }
-                }
-#pragma unroll
-                for (int kt = 0; kt < KT; kt++) st8<V8>(dZbuf + (key0 + 16 * kt) * kRow + 8 * g, z8[kt]);
-#pragma unroll
-                for (int dt = 0; dt < 2; dt++) {
-                    const int off = (q8 + (l16 >> 2)) * kRow + 16 * dt + 4 * (l16 & 3);
-                    const V8 a_do = lds_tr8<DT>(dOs + off, dOs + off + 4 * kRow);
-#pragma unroll
-                    for (int kt = 0; kt < KT; kt++) dvacc[kt][dt] = Elem<DT>::mfma16(a_do, p8[kt], dvacc[kt][dt]);
-                    const V8 a_q = lds_tr8<DT>(Qs + off, Qs + off + 4 * kRow);
-#pragma unroll
-                    for (int kt = 0; kt < KT; kt++) dkacc[kt][dt] = Elem<DT>::mfma16(a_q, z8[kt], dkacc[kt][dt]);
-                }
-                __syncthreads();
-                // ---- phase B: dQ_hat^T for 16 queries (all d, all keys), one wavefront per job,
-                //      then straight through the normalisation Jacobian to global memory ----
-#pragma unroll
-                for (int qt = 0; qt < 2; qt++) {
-                    if ((my_jobs >> (2 * qb + qt)) & 1u) {
-                        f32x4 acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
-                        for (int ks = 0; ks < nks; ks++) {
-                            const int rowk = (32 * ks + 8 * g + (l16 >> 2)) * kRow;
-                            const int cb = rowk + 16 * qt + 4 * (l16 & 3);
-                            const V8 b_z = lds_tr8<DT>(dZbuf + cb, dZbuf + cb + 4 * kRow);
-#pragma unroll
-                            for (int dt = 0; dt < 2; dt++) {
-                                const int ca = rowk + 16 * dt + 4 * (l16 & 3);
-                                const V8 a_k = lds_tr8<DT>(Ks + ca, Ks + ca + 4 * kRow);
-                                acc[dt] = Elem<DT>::mfma16(a_k, b_z, acc[dt]);
-                            }
-                        }
-                        // lane (query, g) holds d = 16dt + 4g + i
-                        const int query = 32 * qb + 16 * qt + l16;
-                        const bool q_ok = query < N;
-                        float x[8], a[8];
-                        float ss = 0.f, dot = 0.f;
-#pragma unroll
-                        for (int dt = 0; dt < 2; dt++) {
-                            V4 q4;
-#pragma unroll
-                            for (int i = 0; i < 4; i++) q4[i] = 0;
-                            if (q_ok) q4 = *reinterpret_cast<const V4*>(qptr + (int64_t)query * p.q.sn + 16 * dt + 4 * g);
-#pragma unroll
-                            for (int i = 0; i < 4; i++) {
-                                x[4 * dt + i] = (float)q4[i];
-                                a[4 * dt + i] = acc[dt][i];
-                                ss += x[4 * dt + i] * x[4 * dt + i];
-                            }
-                        }
-                        ss = xor32_add(xor16_add(ss));
-                        const float nrm = sqrtf(ss);
-                        const float inv = 1.0f / fmaxf(nrm, kNormEps);
-#pragma unroll
-                        for (int j = 0; j < 8; j++) { x[j] *= inv; dot += a[j] * x[j]; }
-                        dot = xor32_add(xor16_add(dot));
-                        const float proj = nrm > kNormEps ? dot : 0.f;
-                        const float f = s_true * inv;
-                        if (q_ok) {
-#pragma unroll
-                            for (int dt = 0; dt < 2; dt++) {
-                                V4 o4;
-#pragma unroll
-                                for (int i = 0; i < 4; i++) o4[i] = (E)(f * (a[4 * dt + i] - x[4 * dt + i] * proj));
-                                *reinterpret_cast<V4*>(dqptr + (int64_t)query * p.dq.sn + 16 * dt + 4 * g) = o4;
-                            }
-                            if (g == 0) ds_part += dot;
-                        }
-                    }
-                }
-            }
-        }
+        unit_blocks<DT, HAS_BIAS, ME, NQB, KT, MASKED>(L, w, u, bias_t, mask_t, N, nqb, p.waves, wave, lane, l16, g, key0,
+                                                       tail_keys, my_jobs, s_true, ds_part);
+
         // ---- epilogue dk, dv: lane (key, g) holds d = 16dt + 4g + i ----
 #pragma unroll
         for (int kt = 0; kt < KT; kt++) {
@@ -320,7 +385,7 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     x[4 * dt + i] = (float)k4[i];
-                    a[4 * dt + i] = dkacc[kt][dt][i] * kLn2;      // undo the log2e folded into Q_hat
+                    a[4 * dt + i] = w.dkacc[kt][dt][i] * kLn2;      // undo the log2e folded into Q_hat
                     ss += x[4 * dt + i] * x[4 * dt + i];
                 }
             }
@@ -340,13 +405,23 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
 #pragma unroll
                     for (int i = 0; i < 4; i++) {
                         o4[i] = (E)(inv * (a[4 * dt + i] - x[4 * dt + i] * proj));
-                        v4[i] = (E)dvacc[kt][dt][i];
+                        v4[i] = (E)w.dvacc[kt][dt][i];
                     }
                     *reinterpret_cast<V4*>(dkp + 16 * dt + 4 * g) = o4;
                     *reinterpret_cast<V4*>(dvp + 16 * dt + 4 * g) = v4;
                 }
             }
         }
+    };
+    // units whose window mask is all zero first, then the masked ones: two straight loops, each with
+    // its own copy of the block sequence, instead of a branch inside every block
+    if (MASK_DT >= 0) {
+        for (int b = grp; b < p.bw; b += p.groups)
+            if (p.mask_live && !p.mask_live[b % p.n_windows]) process_unit(std::false_type{}, b);
+        for (int b = grp; b < p.bw; b += p.groups)
+            if (!p.mask_live || p.mask_live[b % p.n_windows]) process_unit(std::true_type{}, b);
+    } else {
+        for (int b = grp; b < p.bw; b += p.groups) process_unit(std::false_type{}, b);
     }
 
     // ---- flush the per-workgroup partial sums ----
@@ -359,7 +434,7 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
                 if (qb < nqb) {
                     f32x4 a, c;
 #pragma unroll
-                    for (int j = 0; j < 4; j++) { a[j] = dbacc[qb][kt][j]; c[j] = dbacc[qb][kt][4 + j]; }
+                    for (int j = 0; j < 4; j++) { a[j] = w.dbacc[qb][kt][j]; c[j] = w.dbacc[qb][kt][4 + j]; }
                     *reinterpret_cast<f32x4*>(dst + 32 * qb + 8 * g) = a;
                     *reinterpret_cast<f32x4*>(dst + 32 * qb + 8 * g + 4) = c;
                 }
@@ -369,20 +444,21 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
     if (p.scale_kind == FWA2_SCALE_TENSOR) {
         const float wsum = wave_sum(ds_part);
         __syncthreads();
-        if (lane == 0) red[wave] = wsum;
+        if (lane == 0) L.red[wave] = wsum;
         __syncthreads();
         if (tid == 0) {
             float tot = 0.f;
-            for (int w = 0; w < p.waves; w++) tot += red[w];
+            for (int i = 0; i < p.waves; i++) tot += L.red[i];
             p.part_dscale[h * p.groups + grp] = tot * s_true;
         }
     }
 }
 
 // bias [H,N,N] / mask [nW,N,N] (query-major) -> key-major, zero padded to [*, NPk, R].
+// Key rows >= n read as `key_pad` (-inf for the bias, so padded keys drop out of the softmax).
 template <class T>
 __global__ void __launch_bounds__(256) transpose_pad_kernel(const T* src, int64_t sa, int64_t sn, int n, int npk, int r,
-                                                            const uint8_t* live, T* dst) {
+                                                            const uint8_t* live, T* dst, float key_pad) {
     __shared__ T tile[32][33];
     const int a = blockIdx.z;
     if (live && !live[a]) return;
@@ -390,7 +466,7 @@ __global__ void __launch_bounds__(256) transpose_pad_kernel(const T* src, int64_
     const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
     for (int i = ty; i < 32; i += 8) {
         const int q = q0 + i, k = k0 + tx;
-        tile[i][tx] = (q < n && k < n) ? src[a * sa + (int64_t)q * sn + k] : (T)0.f;
+        tile[i][tx] = (q < n && k < n) ? src[a * sa + (int64_t)q * sn + k] : (T)(k >= n ? key_pad : 0.f);
     }
     __syncthreads();
     for (int i = ty; i < 32; i += 8) {
@@ -493,6 +569,7 @@ static hipError_t launch_main(const BwdParams& p, const BwdPlan& pl, hipStream_t
     return hipGetLastError();
 }
 
+
 template <int DT, bool HAS_BIAS, int MASK_DT>
 static hipError_t launch_nqb(const BwdParams& p, const BwdPlan& pl, hipStream_t st) {
     if (pl.nqb_t == 2) return launch_main<DT, HAS_BIAS, MASK_DT, 2, 1>(p, pl, st);
@@ -516,18 +593,18 @@ static hipError_t launch_bwd_dt(BwdParams p, bool has_bias, int mask_dt, hipStre
         dim3 gr(tgrid.x, tgrid.y, p.heads);
         hipLaunchKernelGGL(transpose_pad_kernel<E>, gr, dim3(256), 0, st, reinterpret_cast<const E*>(p.bias), p.bias_sh,
                            p.bias_sn, p.n, pl.npk, pl.r, (const uint8_t*)nullptr,
-                           reinterpret_cast<E*>(const_cast<void*>(p.bias_t)));
+                           reinterpret_cast<E*>(const_cast<void*>(p.bias_t)), -INFINITY);
     }
     if (mask_dt >= 0) {
         dim3 gr(tgrid.x, tgrid.y, p.n_windows);
         if (mask_dt == FWA2_F32)
             hipLaunchKernelGGL(transpose_pad_kernel<float>, gr, dim3(256), 0, st, reinterpret_cast<const float*>(p.mask),
                                p.mask_sw, p.mask_sn, p.n, pl.npk, pl.r, p.mask_live,
-                               reinterpret_cast<float*>(const_cast<void*>(p.mask_t)));
+                               reinterpret_cast<float*>(const_cast<void*>(p.mask_t)), 0.f);
         else
             hipLaunchKernelGGL(transpose_pad_kernel<E>, gr, dim3(256), 0, st, reinterpret_cast<const E*>(p.mask),
                                p.mask_sw, p.mask_sn, p.n, pl.npk, pl.r, p.mask_live,
-                               reinterpret_cast<E*>(const_cast<void*>(p.mask_t)));
+                               reinterpret_cast<E*>(const_cast<void*>(p.mask_t)), 0.f);
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
