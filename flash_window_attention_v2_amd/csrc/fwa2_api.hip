@@ -164,8 +164,8 @@ int fwa2_forward(const fwa2_problem* p) {
     k.bw = p->bw; k.heads = p->heads; k.n = p->n; k.n_windows = p->mask.ptr ? p->n_windows : 1;
     k.scale_kind = p->scale_kind;
     k.default_scale = 1.0f / sqrtf((float)p->head_dim);
-    k.bias_vec = p->bias.ptr && row_vec_ok(p->bias.ptr, p->bias.stride_a, p->bias.stride_n, p->n);
-    k.mask_vec = p->mask.ptr && row_vec_ok(p->mask.ptr, p->mask.stride_a, p->mask.stride_n, p->n);
+    k.side_vec = (!p->bias.ptr || row_vec_ok(p->bias.ptr, p->bias.stride_a, p->bias.stride_n, p->n)) &&
+                 (!p->mask.ptr || row_vec_ok(p->mask.ptr, p->mask.stride_a, p->mask.stride_n, p->n));
     hipError_t e = fwa2::launch_forward(k, p->dtype, p->bias.ptr != nullptr, p->mask.ptr ? p->mask_dtype : -1,
                                         (hipStream_t)p->stream);
     if (e != hipSuccess) return fail(FWA2_ERR_HIP, "forward launch: %s", hipGetErrorString(e));
@@ -189,6 +189,8 @@ int fwa2_backward(const fwa2_problem* p) {
     k.scale_kind = p->scale_kind;
     k.default_scale = 1.0f / sqrtf((float)p->head_dim);
     k.dbias = p->dbias; k.dscale = p->dscale;
+    k.side_vec = (!p->bias.ptr || row_vec_ok(p->bias.ptr, p->bias.stride_a, p->bias.stride_n, p->n)) &&
+                 (!p->mask.ptr || row_vec_ok(p->mask.ptr, p->mask.stride_a, p->mask.stride_n, p->n));
     k.workspace = p->workspace;
     k.cus = cu_count();
     k.ev_start = (hipEvent_t)g_ev_start.load();

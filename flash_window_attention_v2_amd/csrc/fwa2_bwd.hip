@@ -1,35 +1,33 @@
-// Backward kernels: dq, dk, dv, dbias, dlogit_scale for gfx950.
+// Backward, key side: dk, dv and dbias for gfx950 (dq lives in fwa2_bwd_dq.hip).
 //
-// Replaces _bwd_preprocess_do_o_dot, _bwd_kernel and the host epilogue of the
-// reference (flash_win_attn_v2/kernels/attn_kernel_backward.py:6-51, 84-564,
-// 703-711).
+// Replaces _bwd_preprocess_do_o_dot, the dK/dV/dbias half of _bwd_kernel and
+// the host epilogue of the reference
+// (flash_win_attn_v2/kernels/attn_kernel_backward.py:6-51, 84-564, 703-711).
 //
 // Work split.  A workgroup is PERSISTENT for one head: it walks over many
 // (batch*window) units of that head and keeps the bias-gradient tile in
 // registers for the whole walk, so dbias costs one register add per score and
-// one plain store per workgroup instead of one global atomic per score.
-// Inside a workgroup every wavefront owns 16 keys (16 wavefronts at N = 256)
-// and streams all queries of the unit past them, 32 at a time.
+// one plain store per workgroup instead of one global atomic per score
+// (attn_kernel_backward.py:273).  Inside a workgroup every wavefront owns 16 or
+// 32 keys and streams all queries of the unit past them, 32 at a time; the
+// wavefronts only meet at the two barriers around the per-unit load.
 //
 // Per unit:
-//   load     q, k (L2-normalised, q additionally times s*log2e), dO -> LDS in
-//            the input dtype; delta = rowsum(o*dO) and lse*log2e -> LDS.
-//   phase A  S = Q_hat K_hat^T and dP = dO V^T with v_mfma_f32_16x16x32
-//            (rows = queries, columns = this wave's keys; -lse and -delta ride in as
-//            the accumulator inits), P = 2^(S+bias+mask-lse), dZ = P (dP - delta); dbias registers += dZ; the accumulators,
-//            rounded to the input dtype, are directly the B operands (k =
-//            queries) of dV^T += dO^T P and dK_hat^T += Q_hat^T dZ, whose A
-//            operands come out of the row-major LDS tiles with
-//            ds_read_b64_tr_b16.  dZ is also written to LDS, key-major.
-//   phase B  dQ_hat^T = K_hat^T dZ^T, the one product that contracts over keys:
-//            both operands are transposing LDS reads; the 4 partial sums per
-//            output tile meet in an fp32 LDS accumulator (ds_add_f32).
-//   epilogue back through the normalisation: dx = (dx_hat - x_hat (dx_hat.x_hat)) / |x|;
-//            dlogit_scale falls out of the same dot product because
-//            sum_j dC_ij c_ij = q_hat_i . dq_hat_i.
+//   load     q (L2-normalised, times s*log2e) and dO -> LDS in the input dtype;
+//            k_hat -> LDS (each wavefront then takes its own rows as an MFMA
+//            operand); -delta = -rowsum(o*dO) and -lse*log2e -> LDS.
+//   blocks   S = Q_hat K_hat^T and dP = dO V^T with v_mfma_f32_16x16x32 (rows =
+//            queries, columns = this wave's keys; -lse and -delta ride in as the
+//            accumulator inits), P = 2^(S+bias+mask-lse), dZ = P (dP - delta);
+//            dbias registers += dZ; the accumulators, rounded to the input dtype,
+//            are directly the B operands (k = queries) of dV^T += dO^T P and
+//            dK_hat^T += Q_hat^T dZ, whose A operands come out of the row-major
+//            LDS tiles with ds_read_b64_tr_b16.
+//   epilogue dk = (dk_hat - k_hat (dk_hat.k_hat)) / |k| in registers, dv as is.
 //
 // bias and mask are read key-major (transposed once per call by a small
-// pre-pass into the workspace) so that a lane's 8 scores are one 16-byte load.
+// pre-pass into the workspace) so that a lane's scores are one vector load,
+// and are fetched one block ahead of their use.
 #include <type_traits>
 
 #include "fwa2_common.hpp"
@@ -38,20 +36,6 @@ namespace fwa2 {
 
 constexpr int kRow = 40;    // LDS row stride of 16-bit tiles, in elements (80 bytes)
 
-template <int DT, int MASK_DT> struct MaskElemB { typedef typename Elem<DT>::E E; };
-template <int DT> struct MaskElemB<DT, FWA2_F32> { typedef float E; };
-
-template <class V8>
-__device__ __forceinline__ void unpack8b(V8 v, float* x) {
-#pragma unroll
-    for (int j = 0; j < 8; j++) x[j] = (float)v[j];
-}
-
-__device__ __forceinline__ float wave_sum(float x) {
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) x += __shfl_xor(x, off);
-    return x;
-}
 
 // Per-wavefront state that lives in registers across the query blocks of one unit (dvacc,
 // dkacc, bk, bv) or across all units of the workgroup (dbacc).
@@ -70,78 +54,21 @@ struct BwdLds {
     E Qs[R * kRow];          // q_hat * s * log2e, row-major [query][d]
     E Ks[R * kRow];          // k_hat, [key][d]
     E dOs[R * kRow];         // dO, [query][d]
-    E dZs[2][R * kRow];      // dZ of one query block, [key][32 queries], double buffered
-    f32x4 parts[2][2][4][64];// partial dQ_hat^T tiles: [buffer][key split][dt + 2 qt][lane]
     float nlse2[R];          // -lse * log2e   (-inf for padded / fully masked rows)
     float ndelta[R];         // -rowsum(o * dO)
-    float red[16];
 };
-
-struct UnitPtrs {
-    const void *q, *k;       // this unit's q and k rows (for the normalisation Jacobians)
-    void* dq;
-    int64_t q_sn, dq_sn;
-};
-
-// dq rows of 16 queries: sum the partial dQ_hat^T tiles, go back through q / max(|q|, eps).
-template <int DT, int NQB>
-__device__ __forceinline__ void finish_dq(BwdLds<DT, NQB>& L, const UnitPtrs& u, int qbr, int qt, int kh_count, int lane,
-                                          int l16, int g, int n, float s_true, float& ds_part) {
-    typedef typename Elem<DT>::E E;
-    typedef typename Elem<DT>::V4 V4;
-    const int query = 32 * qbr + 16 * qt + l16;
-    const bool q_ok = query < n;
-    float x[8], a[8];
-    float ss = 0.f, dot = 0.f;
-#pragma unroll
-    for (int dt = 0; dt < 2; dt++) {
-        V4 q4;
-#pragma unroll
-        for (int i = 0; i < 4; i++) q4[i] = 0;
-        if (q_ok) q4 = *reinterpret_cast<const V4*>(reinterpret_cast<const E*>(u.q) + (int64_t)query * u.q_sn + 16 * dt + 4 * g);
-        f32x4 acc = L.parts[qbr & 1][0][dt + 2 * qt][lane];
-        if (kh_count > 1) acc += L.parts[qbr & 1][1][dt + 2 * qt][lane];
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            x[4 * dt + i] = (float)q4[i];
-            a[4 * dt + i] = acc[i];
-            ss += x[4 * dt + i] * x[4 * dt + i];
-        }
-    }
-    ss = xor32_add(xor16_add(ss));
-    const float nrm = sqrtf(ss);
-    const float inv = 1.0f / fmaxf(nrm, kNormEps);
-#pragma unroll
-    for (int j = 0; j < 8; j++) { x[j] *= inv; dot += a[j] * x[j]; }
-    dot = xor32_add(xor16_add(dot));
-    const float proj = nrm > kNormEps ? dot : 0.f;
-    const float f = s_true * inv;
-    if (q_ok) {
-#pragma unroll
-        for (int dt = 0; dt < 2; dt++) {
-            V4 o4;
-#pragma unroll
-            for (int i = 0; i < 4; i++) o4[i] = (E)(f * (a[4 * dt + i] - x[4 * dt + i] * proj));
-            *reinterpret_cast<V4*>(reinterpret_cast<E*>(u.dq) + (int64_t)query * u.dq_sn + 16 * dt + 4 * g) = o4;
-        }
-        if (g == 0) ds_part += dot;   // sum_j dC_ij c_ij = q_hat_i . dq_hat_i  (dlogit_scale)
-    }
-}
 
 // All query blocks of one unit.  MASKED is uniform per unit (the window's mask is live or not),
 // so the whole block sequence exists twice instead of branching inside every block.
 template <int DT, bool HAS_BIAS, class ME, int NQB, int KT, bool MASKED>
-__device__ __forceinline__ void unit_blocks(BwdLds<DT, NQB>& L, WaveRegs<DT, NQB, KT>& w, const UnitPtrs& u,
+__device__ __forceinline__ void unit_blocks(BwdLds<DT, NQB>& L, WaveRegs<DT, NQB, KT>& w,
                                             const typename Elem<DT>::E* bias_t, const ME* mask_t, int n, int nqb,
-                                            int waves, int wave, int lane, int l16, int g, int key0, bool tail_keys,
-                                            uint32_t my_jobs, float s_true, float& ds_part) {
+                                            int l16, int g, int key0, bool tail_keys) {
     typedef typename Elem<DT>::E E;
     typedef typename Elem<DT>::V8 V8;
     typedef typename Elem<DT>::V4 V4;
     typedef ME MV4 __attribute__((ext_vector_type(4)));
     constexpr int R = 32 * NQB;
-    const int kh_count = waves >= 8 ? 2 : 1;          // key splits of the dQ product
-    const int nks = nqb;
 
     // bias (and mask) values of the coming block travel in registers: they are fetched one block
     // ahead so that the L2 round trip overlaps the rest of the block instead of stalling it
@@ -162,7 +89,6 @@ __device__ __forceinline__ void unit_blocks(BwdLds<DT, NQB>& L, WaveRegs<DT, NQB
 #pragma unroll
     for (int qb = 0; qb < NQB; qb++) {
         if (qb < nqb) {
-            E* dZbuf = L.dZs[qb & 1];
             const int q8 = 32 * qb + 8 * g;          // first of this lane's 8 queries
             // ---- phase A, one key tile at a time ----
 #pragma unroll
@@ -201,7 +127,6 @@ __device__ __forceinline__ void unit_blocks(BwdLds<DT, NQB>& L, WaveRegs<DT, NQB
                         z8[4 * t + i] = (E)dz;
                     }
                 }
-                st8<V8>(dZbuf + (key0 + 16 * kt) * kRow + 8 * g, z8);
 #pragma unroll
                 for (int dt = 0; dt < 2; dt++) {
                     const int off = (q8 + (l16 >> 2)) * kRow + 16 * dt + 4 * (l16 & 3);
@@ -212,34 +137,8 @@ __device__ __forceinline__ void unit_blocks(BwdLds<DT, NQB>& L, WaveRegs<DT, NQB
                 }
             }
             fetch_side(qb + 1 < nqb ? qb + 1 : 0);
-            __syncthreads();
-            // ---- phase B, spread over the wavefronts: dQ_hat^T tile (dt, qt) over a share of the keys ----
-            for (int job = wave; job < 4 * kh_count; job += waves) {
-                const int tile = job & 3, kh = job >> 2;
-                const int dt = tile & 1, qt = tile >> 1;
-                f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-                for (int ks = kh; ks < nks; ks += kh_count) {
-                    const int rowk = (32 * ks + 8 * g + (l16 >> 2)) * kRow + 4 * (l16 & 3);
-                    const V8 a_k = lds_tr8<DT>(L.Ks + rowk + 16 * dt, L.Ks + rowk + 16 * dt + 4 * kRow);
-                    const V8 b_z = lds_tr8<DT>(dZbuf + rowk + 16 * qt, dZbuf + rowk + 16 * qt + 4 * kRow);
-                    acc = Elem<DT>::mfma16(a_k, b_z, acc);
-                }
-                L.parts[qb & 1][kh][tile][lane] = acc;
-            }
-            // ---- the previous block's partial tiles are complete: finish its dq rows ----
-            if (qb > 0) {
-#pragma unroll
-                for (int qt = 0; qt < 2; qt++)
-                    if ((my_jobs >> (2 * (qb - 1) + qt)) & 1u)
-                        finish_dq<DT, NQB>(L, u, qb - 1, qt, kh_count, lane, l16, g, n, s_true, ds_part);
-            }
         }
     }
-    __syncthreads();
-#pragma unroll
-    for (int qt = 0; qt < 2; qt++)
-        if ((my_jobs >> (2 * (nqb - 1) + qt)) & 1u)
-            finish_dq<DT, NQB>(L, u, nqb - 1, qt, kh_count, lane, l16, g, n, s_true, ds_part);
 }
 
 // KT = key tiles of 16 owned by one wavefront, NQB = compile-time bound on query blocks of 32.
@@ -248,7 +147,7 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
     typedef typename Elem<DT>::E E;
     typedef typename Elem<DT>::V8 V8;
     typedef typename Elem<DT>::V4 V4;
-    typedef typename MaskElemB<DT, MASK_DT>::E ME;
+    typedef typename MaskElem<DT, MASK_DT>::E ME;
 
     const int N = p.n;
     constexpr int R = 32 * NQB;            // padded rows of every LDS tile and of the key-major side tables
@@ -287,14 +186,6 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
         for (int kt = 0; kt < KT; kt++)
 #pragma unroll
             for (int j = 0; j < 8; j++) w.dbacc[a][kt][j] = 0.f;
-    float ds_part = 0.f;
-    // bit (2 qb + qt) set: this wavefront finishes dq for queries 32 qb + 16 qt .. + 16
-    uint32_t my_jobs = 0;
-    for (int j = wave; j < 2 * NQB; j += p.waves) my_jobs |= 1u << j;
-
-    // dZ staging rows that no wavefront writes must read as zeros in phase B
-    for (int i = tid; i < 2 * R * kRow / 8; i += nthreads) st8<V8>(&L.dZs[0][0] + i * 8, zero8<V8>());
-
     const E* bias_t = nullptr;
     if (HAS_BIAS) bias_t = reinterpret_cast<const E*>(p.bias_t) + ((int64_t)h * NPk + key0) * R;
 
@@ -306,9 +197,6 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
         const E* optr = reinterpret_cast<const E*>(p.o.ptr) + b * p.o.sb + h * p.o.sh;
         const E* doptr = reinterpret_cast<const E*>(p.d_o.ptr) + b * p.d_o.sb + h * p.d_o.sh;
         const float* lseptr = p.lse + b * p.lse_sb + h * p.lse_sh;
-        UnitPtrs u;
-        u.q = qptr; u.k = kptr; u.q_sn = p.q.sn; u.dq_sn = p.dq.sn;
-        u.dq = reinterpret_cast<E*>(const_cast<void*>(p.dq.ptr)) + b * p.dq.sb + h * p.dq.sh;
 
         const ME* mask_t = nullptr;
         if (MASK_DT >= 0) {
@@ -332,7 +220,7 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
                 o8 = ld8<V8>(optr + (int64_t)r * p.o.sn + dc);
             }
             float xq[8], xk[8], xd[8], xo[8];
-            unpack8b(q8, xq); unpack8b(k8, xk); unpack8b(do8, xd); unpack8b(o8, xo);
+            unpack8(q8, xq); unpack8(k8, xk); unpack8(do8, xd); unpack8(o8, xo);
             float sq = 0.f, sk = 0.f, dl = 0.f;
 #pragma unroll
             for (int j = 0; j < 8; j++) { sq += xq[j] * xq[j]; sk += xk[j] * xk[j]; dl += xo[j] * xd[j]; }
@@ -366,8 +254,7 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
 #pragma unroll
                 for (int i = 0; i < 4; i++) { w.dvacc[kt][dt][i] = 0.f; w.dkacc[kt][dt][i] = 0.f; }
 
-        unit_blocks<DT, HAS_BIAS, ME, NQB, KT, MASKED>(L, w, u, bias_t, mask_t, N, nqb, p.waves, wave, lane, l16, g, key0,
-                                                       tail_keys, my_jobs, s_true, ds_part);
+        unit_blocks<DT, HAS_BIAS, ME, NQB, KT, MASKED>(L, w, bias_t, mask_t, N, nqb, l16, g, key0, tail_keys);
 
         // ---- epilogue dk, dv: lane (key, g) holds d = 16dt + 4g + i ----
 #pragma unroll
@@ -441,20 +328,8 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
             }
         }
     }
-    if (p.scale_kind == FWA2_SCALE_TENSOR) {
-        const float wsum = wave_sum(ds_part);
-        __syncthreads();
-        if (lane == 0) L.red[wave] = wsum;
-        __syncthreads();
-        if (tid == 0) {
-            float tot = 0.f;
-            for (int i = 0; i < p.waves; i++) tot += L.red[i];
-            p.part_dscale[h * p.groups + grp] = tot * s_true;
-        }
-    }
 }
 
-// bias [H,N,N] / mask [nW,N,N] (query-major) -> key-major, zero padded to [*, NPk, R].
 // Key rows >= n read as `key_pad` (-inf for the bias, so padded keys drop out of the softmax).
 template <class T>
 __global__ void __launch_bounds__(256) transpose_pad_kernel(const T* src, int64_t sa, int64_t sn, int n, int npk, int r,
@@ -500,7 +375,7 @@ __global__ void __launch_bounds__(256) reduce_kernel(const BwdParams p, int npk,
     }
     if (p.scale_kind == FWA2_SCALE_TENSOR && blockIdx.x == 0 && blockIdx.y == 0) {
         float v = 0.f;
-        for (int gi = threadIdx.x; gi < p.groups; gi += 256) v += p.part_dscale[h * p.groups + gi];
+        for (int gi = threadIdx.x; gi < p.ds_parts; gi += 256) v += p.part_dscale[(int64_t)h * p.ds_parts + gi];
         __shared__ float red[256];
         red[threadIdx.x] = v;
         __syncthreads();
@@ -520,8 +395,11 @@ static size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
 int backward_supported(int n) { return n >= 1 && n <= 256; }
 
+void dq_geometry(int n, int* waves, int* chunks);
+hipError_t launch_backward_dq(const BwdParams& p, int dtype, bool has_bias, int mask_dt, hipStream_t st);
+
 struct BwdPlan {
-    int waves, groups, npk, r, nqb_t, kt;
+    int waves, groups, npk, r, nqb_t, kt, dq_waves, dq_chunks, ds_parts;
     size_t off_dbias, off_dscale, off_bias_t, off_mask_t, total;
     size_t smem;
 };
@@ -544,8 +422,10 @@ static BwdPlan make_plan(int heads, int n, int bw, bool has_bias, bool has_mask,
     size_t off = 0;
     pl.off_dbias = off;
     if (has_bias) off += align256((size_t)heads * groups * pl.npk * pl.r * 4);
+    dq_geometry(n, &pl.dq_waves, &pl.dq_chunks);
+    pl.ds_parts = bw * pl.dq_chunks;
     pl.off_dscale = off;
-    off += align256((size_t)heads * groups * 4);
+    off += align256((size_t)heads * pl.ds_parts * 4);
     pl.off_bias_t = off;
     if (has_bias) off += align256((size_t)heads * pl.npk * pl.r * 2);
     pl.off_mask_t = off;
@@ -584,6 +464,9 @@ static hipError_t launch_bwd_dt(BwdParams p, bool has_bias, int mask_dt, hipStre
     unsigned char* ws = reinterpret_cast<unsigned char*>(p.workspace);
     p.waves = pl.waves;
     p.groups = pl.groups;
+    p.dq_waves = pl.dq_waves;
+    p.dq_chunks = pl.dq_chunks;
+    p.ds_parts = pl.ds_parts;
     p.part_dbias = reinterpret_cast<float*>(ws + pl.off_dbias);
     p.part_dscale = reinterpret_cast<float*>(ws + pl.off_dscale);
     p.bias_t = ws + pl.off_bias_t;
@@ -617,6 +500,8 @@ static hipError_t launch_bwd_dt(BwdParams p, bool has_bias, int mask_dt, hipStre
         else if (mask_dt == FWA2_F32) e = launch_nqb<DT, false, FWA2_F32>(p, pl, st);
         else e = launch_nqb<DT, false, DT>(p, pl, st);
     }
+    if (e != hipSuccess) return e;
+    e = launch_backward_dq(p, DT, has_bias, mask_dt, st);
     if (e != hipSuccess) return e;
     if (has_bias || p.scale_kind == FWA2_SCALE_TENSOR) {
         dim3 gr(has_bias ? pl.r / 32 : 1, has_bias ? (pl.npk + 7) / 8 : 1, p.heads);

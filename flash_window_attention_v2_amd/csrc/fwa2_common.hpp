@@ -122,6 +122,45 @@ __host__ __device__ constexpr int swap_bits23(int r) {
     return (r & ~12) | ((r & 4) << 1) | ((r & 8) >> 1);
 }
 
+
+// ---- small shared device helpers ------------------------------------------------
+template <class V8>
+__device__ __forceinline__ void unpack8(V8 v, float* x) {
+#pragma unroll
+    for (int j = 0; j < 8; j++) x[j] = (float)v[j];
+}
+
+// 8 consecutive elements starting at column c0 of one row of bias / mask, as floats.
+// VEC: the row may be read with 16-byte loads and n is a multiple of 8; columns at or
+// beyond n are then read from the last 8 real columns instead (the caller overwrites the
+// scores of such padded keys with -inf), which keeps the load in bounds without a branch.
+// !VEC: element loads with a bounds check, padded columns read as 0.
+template <bool VEC, class E>
+__device__ __forceinline__ void load_row8(const E* row, int c0, int n, float* x) {
+    typedef E V8 __attribute__((ext_vector_type(8)));
+    if (VEC) {
+        const V8 v = *reinterpret_cast<const V8*>(row + min(c0, n - 8));
+#pragma unroll
+        for (int j = 0; j < 8; j++) x[j] = (float)v[j];
+    } else {
+#pragma unroll
+        for (int j = 0; j < 8; j++) x[j] = (c0 + j < n) ? (float)row[c0 + j] : 0.f;
+    }
+}
+
+// Element type of the mask: the input dtype, or float for an fp32 mask.
+template <int DT, int MASK_DT> struct MaskElem { typedef typename Elem<DT>::E E; };
+template <int DT> struct MaskElem<DT, FWA2_F32> { typedef float E; };
+
+__device__ __forceinline__ float wave_sum(float x) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) x += __shfl_xor(x, off);
+    return x;
+}
+
+constexpr int kKeyChunk = 256;   // keys staged in LDS at a time by the query-owning kernels
+constexpr int kLdsStride = 40;   // elements per staged row (32 + 8 pad): 80-byte rows
+
 // ---- launch parameters -------------------------------------------------------
 struct T4 {
     const void* ptr;
@@ -140,7 +179,7 @@ struct FwdParams {
     int bw, heads, n, n_windows;
     int scale_kind;
     float default_scale;  // 1/sqrt(head_dim), used when no logit scale is given
-    bool bias_vec, mask_vec;  // rows of bias / mask may be read with 16-byte loads
+    bool side_vec;    // rows of bias and mask may be read with 16-byte loads and n % 8 == 0
     int waves;        // wavefronts per workgroup
     int q_chunks;     // workgroups per (bw, head)
 };
@@ -167,7 +206,11 @@ struct BwdParams {
     int waves;        // wavefronts per workgroup = key tiles of 16
     int groups;       // workgroups per head (each walks bw = g, g + groups, ...)
     float* part_dbias;   // [H, groups, NP, NQ] fp32, key-major
-    float* part_dscale;  // [H, groups] fp32
+    float* part_dscale;  // [H, ds_parts] fp32, one per workgroup of the dq kernel
+    int ds_parts;        // bw * dq_chunks
+    int dq_waves;        // wavefronts per workgroup of the dq kernel
+    int dq_chunks;       // dq workgroups per (bw, head)
+    bool side_vec;       // rows of bias and mask (query-major) may be read with 16-byte loads, n % 8 == 0
     const void* bias_t;  // [H, NP, NQ] input dtype: bias transposed to key-major, zero padded
     const void* mask_t;  // [nW, NP, NQ] mask dtype: mask transposed to key-major, zero padded
 };

@@ -27,35 +27,7 @@
 
 namespace fwa2 {
 
-constexpr int kKeyChunk = 256;   // keys staged in LDS at a time
-constexpr int kLdsStride = 40;   // elements per staged row (32 + 8 pad): 80-byte rows
-
-template <class V8>
-__device__ __forceinline__ void unpack8(V8 v, float* x) {
-#pragma unroll
-    for (int j = 0; j < 8; j++) x[j] = (float)v[j];
-}
-
-// 8 consecutive elements starting at column c0 of one row of bias / mask, as
-// floats; columns >= n read as `fill`.  `vec` says 16-byte loads are legal.
-template <class E>
-__device__ __forceinline__ void load_row8(const E* row, int c0, int n, bool vec, float fill, float* x) {
-    typedef E V8 __attribute__((ext_vector_type(8)));
-    if (vec && c0 + 8 <= n) {
-        V8 v = *reinterpret_cast<const V8*>(row + c0);
-#pragma unroll
-        for (int j = 0; j < 8; j++) x[j] = (float)v[j];
-    } else {
-#pragma unroll
-        for (int j = 0; j < 8; j++) x[j] = (c0 + j < n) ? (float)row[c0 + j] : fill;
-    }
-}
-
-// Element type of the mask: the input dtype, or float for an fp32 mask.
-template <int DT, int MASK_DT> struct MaskElem { typedef typename Elem<DT>::E E; };
-template <int DT> struct MaskElem<DT, FWA2_F32> { typedef float E; };
-
-template <int DT, bool HAS_BIAS, int MASK_DT>
+template <int DT, bool HAS_BIAS, int MASK_DT, bool VEC>
 __global__ void __launch_bounds__(512) fwd_kernel(const FwdParams p) {
     typedef typename Elem<DT>::E E;
     typedef typename Elem<DT>::V8 V8;
@@ -188,7 +160,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdParams p) {
 #pragma unroll
                     for (int u = 0; u < 2; u++) {
                         float x[8];
-                        load_row8<E>(bias_row, kbase + 32 * t + 16 * u + 8 * hf, N, p.bias_vec, 0.f, x);
+                        load_row8<VEC, E>(bias_row, kbase + 32 * t + 16 * u + 8 * hf, N, x);
 #pragma unroll
                         for (int j = 0; j < 8; j++) acc[t][8 * u + j] = fmaf(x[j], kLog2e, acc[t][8 * u + j]);
                     }
@@ -200,7 +172,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdParams p) {
 #pragma unroll
                         for (int u = 0; u < 2; u++) {
                             float x[8];
-                            load_row8<ME>(mask_row, kbase + 32 * t + 16 * u + 8 * hf, N, p.mask_vec, 0.f, x);
+                            load_row8<VEC, ME>(mask_row, kbase + 32 * t + 16 * u + 8 * hf, N, x);
 #pragma unroll
                             for (int j = 0; j < 8; j++) acc[t][8 * u + j] = fmaf(x[j], kLog2e, acc[t][8 * u + j]);
                         }
@@ -286,7 +258,10 @@ __global__ void __launch_bounds__(256) mask_scan_kernel(const ME* mask, int64_t 
 
 template <int DT, bool HAS_BIAS, int MASK_DT>
 static hipError_t launch_one(const FwdParams& p, dim3 grid, dim3 block, size_t smem, hipStream_t st) {
-    hipLaunchKernelGGL((fwd_kernel<DT, HAS_BIAS, MASK_DT>), grid, block, smem, st, p);
+    if (p.side_vec)
+        hipLaunchKernelGGL((fwd_kernel<DT, HAS_BIAS, MASK_DT, true>), grid, block, smem, st, p);
+    else
+        hipLaunchKernelGGL((fwd_kernel<DT, HAS_BIAS, MASK_DT, false>), grid, block, smem, st, p);
     return hipGetLastError();
 }
 
