@@ -28,8 +28,6 @@
 // bias and mask are read key-major (transposed once per call by a small
 // pre-pass into the workspace) so that a lane's scores are one vector load,
 // and are fetched one block ahead of their use.
-#include <type_traits>
-
 #include "fwa2_common.hpp"
 
 namespace fwa2 {
@@ -46,24 +44,41 @@ struct WaveRegs {
     typename Elem<DT>::V8 bk[KT], bv[KT];
 };
 
-// LDS of one workgroup; all sizes are compile-time so tile addresses are lane offset + immediate.
+// LDS views of one workgroup.  The arrays behind them are separate __shared__ variables with
+// compile-time sizes: tile addresses are lane offset + immediate, and the compiler can tell the
+// landing area (written by global_load_lds) from the tiles, so reads of the tiles do not wait
+// for fetches in flight.
 template <int DT, int NQB>
 struct BwdLds {
     typedef typename Elem<DT>::E E;
     static constexpr int R = 32 * NQB;
-    E Qs[R * kRow];          // q_hat * s * log2e, row-major [query][d]
-    E Ks[R * kRow];          // k_hat, [key][d]
-    E dOs[R * kRow];         // dO, [query][d]
-    float nlse2[R];          // -lse * log2e   (-inf for padded / fully masked rows)
-    float ndelta[R];         // -rowsum(o * dO)
+    E* Qs;          // q_hat * s * log2e, row-major [query][kRow]
+    E* Ks;          // k_hat, [key][kRow]
+    E* dOs;         // dO, [query][kRow]
+    float* nlse2;   // -lse * log2e   (-inf for padded / fully masked rows)
+    float* ndelta;  // -rowsum(o * dO)
+    float* kinv;    // 1 / max(|k|, eps), negated when |k| <= eps
+    // landing area of the next unit's rows: unpadded 64-byte rows, rows >= n stay zero
+    E *rawQ, *rawK, *rawV, *rawDO, *rawO;
+    float* rawLse;
 };
+
+// 16 bytes per lane straight from global memory into LDS (no registers held while in flight):
+// lane i of the wavefront lands at lds_wave_base + 16 i.
+template <class E>
+__device__ __forceinline__ void async_row_chunk(const E* gsrc, E* lds_wave_base) {
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gsrc,
+                                     (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
+}
 
 // All query blocks of one unit.  MASKED is uniform per unit (the window's mask is live or not),
 // so the whole block sequence exists twice instead of branching inside every block.
-template <int DT, bool HAS_BIAS, class ME, int NQB, int KT, bool MASKED>
+// `block_start(qb)` runs at the top of every block, after every side value fetched for that block
+// has arrived (the kernel uses it to start the next unit's fetch behind them).
+template <int DT, bool HAS_BIAS, class ME, int NQB, int KT, bool MASKED, class Hook>
 __device__ __forceinline__ void unit_blocks(BwdLds<DT, NQB>& L, WaveRegs<DT, NQB, KT>& w,
                                             const typename Elem<DT>::E* bias_t, const ME* mask_t, int n, int nqb,
-                                            int l16, int g, int key0, bool tail_keys) {
+                                            int l16, int g, int key0, bool tail_keys, Hook block_start) {
     typedef typename Elem<DT>::E E;
     typedef typename Elem<DT>::V8 V8;
     typedef typename Elem<DT>::V4 V4;
@@ -90,6 +105,15 @@ __device__ __forceinline__ void unit_blocks(BwdLds<DT, NQB>& L, WaveRegs<DT, NQB
     for (int qb = 0; qb < NQB; qb++) {
         if (qb < nqb) {
             const int q8 = 32 * qb + 8 * g;          // first of this lane's 8 queries
+            // every side value of this block is waited for here, in one go ...
+#pragma unroll
+            for (int kt = 0; kt < KT; kt++)
+#pragma unroll
+                for (int t = 0; t < 2; t++) {
+                    if (HAS_BIAS) asm volatile("" : "+v"(bcur[kt][t]));
+                    if (MASKED) asm volatile("" : "+v"(mcur[kt][t]));
+                }
+            block_start(qb);   // ... so that whatever this issues is younger than all of them
             // ---- phase A, one key tile at a time ----
 #pragma unroll
             for (int kt = 0; kt < KT; kt++) {
@@ -142,7 +166,10 @@ __device__ __forceinline__ void unit_blocks(BwdLds<DT, NQB>& L, WaveRegs<DT, NQB
 }
 
 // KT = key tiles of 16 owned by one wavefront, NQB = compile-time bound on query blocks of 32.
-template <int DT, bool HAS_BIAS, int MASK_DT, int NQB, int KT>
+// MASKED: this launch handles the units whose window mask is live (and adds the mask); the units
+// with an all-zero mask go through a second launch of the MASKED = false instantiation, so no
+// block ever branches on the mask and each launch has a single copy of the block sequence.
+template <int DT, bool HAS_BIAS, int MASK_DT, int NQB, int KT, bool MASKED>
 __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) {
     typedef typename Elem<DT>::E E;
     typedef typename Elem<DT>::V8 V8;
@@ -154,12 +181,28 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
     const int NPk = p.waves * 16 * KT;     // padded key rows
     const int nqb = (N + 31) >> 5;         // query blocks of 32 that hold real rows
 
-    __shared__ __attribute__((aligned(16))) BwdLds<DT, NQB> L;
+    __shared__ __attribute__((aligned(16))) E lds_Qs[R * kRow];
+    __shared__ __attribute__((aligned(16))) E lds_Ks[R * kRow];
+    __shared__ __attribute__((aligned(16))) E lds_dOs[R * kRow];
+    __shared__ __attribute__((aligned(16))) float lds_nlse2[R];
+    __shared__ __attribute__((aligned(16))) float lds_ndelta[R];
+    __shared__ __attribute__((aligned(16))) float lds_kinv[R];
+    __shared__ __attribute__((aligned(16))) E lds_rawQ[R * 32];
+    __shared__ __attribute__((aligned(16))) E lds_rawK[R * 32];
+    __shared__ __attribute__((aligned(16))) E lds_rawV[R * 32];
+    __shared__ __attribute__((aligned(16))) E lds_rawDO[R * 32];
+    __shared__ __attribute__((aligned(16))) E lds_rawO[R * 32];
+    __shared__ __attribute__((aligned(16))) float lds_rawLse[R];
+    BwdLds<DT, NQB> L;
+    L.Qs = lds_Qs; L.Ks = lds_Ks; L.dOs = lds_dOs; L.nlse2 = lds_nlse2; L.ndelta = lds_ndelta; L.kinv = lds_kinv;
+    L.rawQ = lds_rawQ; L.rawK = lds_rawK; L.rawV = lds_rawV; L.rawDO = lds_rawDO; L.rawO = lds_rawO;
+    L.rawLse = lds_rawLse;
 
     const int tid = threadIdx.x;
     const int nthreads = blockDim.x;
-    const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int lane_0 = tid & 63;
+    const int wave_0 = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = lane_0, wave = wave_0;
     const int l16_0 = lane & 15;
     const int g_0 = lane >> 4;
     int l16 = l16_0, g = g_0;
@@ -189,15 +232,66 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
     const E* bias_t = nullptr;
     if (HAS_BIAS) bias_t = reinterpret_cast<const E*>(p.bias_t) + ((int64_t)h * NPk + key0) * R;
 
-    auto process_unit = [&](auto masked_tag, int b) __attribute__((always_inline)) {
-        constexpr bool MASKED = decltype(masked_tag)::value;
+    // ---- which units belong to this launch ----
+    auto mine = [&](int b) -> bool {
+        if (MASK_DT >= 0 && p.mask_live) return (p.mask_live[b % p.n_windows] != 0) == MASKED;
+        return true;
+    };
+    auto next_unit = [&](int b) -> int {
+        for (b += p.groups; b < p.bw; b += p.groups)
+            if (mine(b)) return b;
+        return p.bw;
+    };
+    // ---- asynchronous fetch of one unit's rows into the landing area ----
+    auto fetch_unit = [&](int b) __attribute__((always_inline)) {
         const E* qptr = reinterpret_cast<const E*>(p.q.ptr) + b * p.q.sb + h * p.q.sh;
         const E* kptr = reinterpret_cast<const E*>(p.k.ptr) + b * p.k.sb + h * p.k.sh;
         const E* vptr = reinterpret_cast<const E*>(p.v.ptr) + b * p.v.sb + h * p.v.sh;
         const E* optr = reinterpret_cast<const E*>(p.o.ptr) + b * p.o.sb + h * p.o.sh;
         const E* doptr = reinterpret_cast<const E*>(p.d_o.ptr) + b * p.d_o.sb + h * p.d_o.sh;
         const float* lseptr = p.lse + b * p.lse_sb + h * p.lse_sh;
+        // re-materialised here so that no per-row address is computed ahead of time and spilled
+        // (a spill reload would wait for every fetch already in flight)
+        int lane = lane_0, wave = wave_0;
+        asm volatile("" : "+v"(lane));
+        asm volatile("" : "+s"(wave));
+        const int dc = (lane & 3) * 8;
+        for (int row0 = wave * 16; row0 < R; row0 += 16 * p.waves) {   // 16 rows per wavefront and instruction
+            const int r = row0 + (lane >> 2);
+            if (r < N) {
+                async_row_chunk(qptr + (int64_t)r * p.q.sn + dc, L.rawQ + row0 * 32);
+                async_row_chunk(kptr + (int64_t)r * p.k.sn + dc, L.rawK + row0 * 32);
+                async_row_chunk(doptr + (int64_t)r * p.d_o.sn + dc, L.rawDO + row0 * 32);
+                async_row_chunk(optr + (int64_t)r * p.o.sn + dc, L.rawO + row0 * 32);
+            }
+        }
+        // v: every wavefront fetches exactly the key rows it owns, so nobody else reads them
+#pragma unroll
+        for (int kt = 0; kt < KT; kt++) {
+            const int row0 = (wave * KT + kt) * 16;
+            const int r = row0 + (lane >> 2);
+            if (r < N) async_row_chunk(vptr + (int64_t)r * p.v.sn + dc, L.rawV + row0 * 32);
+        }
+        for (int r0 = wave * 64; r0 < N; r0 += 64 * p.waves) {
+            if (r0 + lane < N)
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(lseptr + r0 + lane),
+                                                 (__attribute__((address_space(3))) void*)(L.rawLse + r0), 4, 0, 0);
+        }
+    };
 
+    // landing rows beyond n must read as zeros for the whole kernel
+    for (int i = tid; i < R * 32 / 8; i += nthreads) {
+        st8<V8>(L.rawQ + i * 8, zero8<V8>()); st8<V8>(L.rawK + i * 8, zero8<V8>()); st8<V8>(L.rawV + i * 8, zero8<V8>());
+        st8<V8>(L.rawDO + i * 8, zero8<V8>()); st8<V8>(L.rawO + i * 8, zero8<V8>());
+    }
+    __syncthreads();
+
+    int b = grp;
+    if (!mine(b)) b = next_unit(b);
+    if (b < p.bw) fetch_unit(b);
+
+    while (b < p.bw) {
+        const int b_next = next_unit(b);
         const ME* mask_t = nullptr;
         if (MASK_DT >= 0) {
             const int wnd = b % p.n_windows;
@@ -208,43 +302,41 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
         // dozens of per-block addresses alive (and spilled) across the whole unit loop
         l16 = l16_0; g = g_0;
         asm volatile("" : "+v"(l16), "+v"(g));
-        __syncthreads();   // the previous unit is done with LDS
-        // ---- load: one 8-element chunk of one row per thread and pass ----
-        for (int r = tid >> 2; r < R; r += nthreads >> 2) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wavefront's share of the unit has landed
+        __syncthreads();   // ... and everybody's; the previous unit is done with the tiles
+        // ---- landing area -> MFMA tiles: one 8-element chunk of a row per thread and pass ----
+        {
             const int dc = (tid & 3) * 8;
-            V8 q8 = zero8<V8>(), k8 = zero8<V8>(), do8 = zero8<V8>(), o8 = zero8<V8>();
-            if (r < N) {
-                q8 = ld8<V8>(qptr + (int64_t)r * p.q.sn + dc);
-                k8 = ld8<V8>(kptr + (int64_t)r * p.k.sn + dc);
-                do8 = ld8<V8>(doptr + (int64_t)r * p.d_o.sn + dc);
-                o8 = ld8<V8>(optr + (int64_t)r * p.o.sn + dc);
-            }
-            float xq[8], xk[8], xd[8], xo[8];
-            unpack8(q8, xq); unpack8(k8, xk); unpack8(do8, xd); unpack8(o8, xo);
-            float sq = 0.f, sk = 0.f, dl = 0.f;
+            for (int r = tid >> 2; r < R; r += nthreads >> 2) {
+                float xq[8], xk[8], xd[8], xo[8];
+                const V8 do8 = ld8<V8>(L.rawDO + r * 32 + dc);
+                unpack8(ld8<V8>(L.rawQ + r * 32 + dc), xq);
+                unpack8(ld8<V8>(L.rawK + r * 32 + dc), xk);
+                unpack8(do8, xd);
+                unpack8(ld8<V8>(L.rawO + r * 32 + dc), xo);
+                float sq = 0.f, sk = 0.f, dl = 0.f;
 #pragma unroll
-            for (int j = 0; j < 8; j++) { sq += xq[j] * xq[j]; sk += xk[j] * xk[j]; dl += xo[j] * xd[j]; }
-            sq = quad_add(sq); sk = quad_add(sk); dl = quad_add(dl);
-            const float iq = inv_norm(sq) * scale2, ik = inv_norm(sk);
-            V8 qn, kn;
+                for (int j = 0; j < 8; j++) { sq += xq[j] * xq[j]; sk += xk[j] * xk[j]; dl += xo[j] * xd[j]; }
+                sq = quad_add(sq); sk = quad_add(sk); dl = quad_add(dl);
+                const float iq = inv_norm(sq) * scale2, ik = inv_norm(sk);
+                V8 qn, kn;
 #pragma unroll
-            for (int j = 0; j < 8; j++) { qn[j] = (E)(xq[j] * iq); kn[j] = (E)(xk[j] * ik); }
-            st8<V8>(L.Qs + r * kRow + dc, qn);
-            st8<V8>(L.Ks + r * kRow + dc, kn);
-            st8<V8>(L.dOs + r * kRow + dc, do8);
-            if ((tid & 3) == 0) L.ndelta[r] = -dl;
-            if ((tid & 3) == 1) {
-                float l2 = -INFINITY;          // padded / fully masked rows: P = 0
-                if (r < N) { const float l = lseptr[r]; l2 = (l == -INFINITY) ? -INFINITY : -l * kLog2e; }
-                L.nlse2[r] = l2;
+                for (int j = 0; j < 8; j++) { qn[j] = (E)(xq[j] * iq); kn[j] = (E)(xk[j] * ik); }
+                st8<V8>(L.Qs + r * kRow + dc, qn);
+                st8<V8>(L.Ks + r * kRow + dc, kn);
+                st8<V8>(L.dOs + r * kRow + dc, do8);
+                if ((tid & 3) == 0) L.ndelta[r] = -dl;
+                if ((tid & 3) == 1) {
+                    float l2 = -INFINITY;          // padded / fully masked rows: P = 0
+                    if (r < N) { const float l = L.rawLse[r]; l2 = (l == -INFINITY) ? -INFINITY : -l * kLog2e; }
+                    L.nlse2[r] = l2;
+                }
+                if ((tid & 3) == 2) L.kinv[r] = (sqrtf(sk) > kNormEps) ? ik : -ik;
             }
         }
 #pragma unroll
-        for (int kt = 0; kt < KT; kt++) {
-            w.bv[kt] = zero8<V8>();
-            if (key0 + 16 * kt < N) w.bv[kt] = ld8<V8>(vptr + (int64_t)(key0 + 16 * kt) * p.v.sn + 8 * g);
-        }
-        __syncthreads();
+        for (int kt = 0; kt < KT; kt++) w.bv[kt] = ld8<V8>(L.rawV + (key0 + 16 * kt) * 32 + 8 * g);
+        __syncthreads();   // tiles complete; the landing area is free again
 #pragma unroll
         for (int kt = 0; kt < KT; kt++) w.bk[kt] = ld8<V8>(L.Ks + (key0 + 16 * kt) * kRow + 8 * g);
 #pragma unroll
@@ -254,35 +346,34 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
 #pragma unroll
                 for (int i = 0; i < 4; i++) { w.dvacc[kt][dt][i] = 0.f; w.dkacc[kt][dt][i] = 0.f; }
 
-        unit_blocks<DT, HAS_BIAS, ME, NQB, KT, MASKED>(L, w, bias_t, mask_t, N, nqb, l16, g, key0, tail_keys);
+        // The next unit's fetch starts at the top of the last block: memory returns in issue order,
+        // so an earlier start would make every later wait for bias values also wait for the fetch.
+        const int fetch_at = nqb - 1;
+        unit_blocks<DT, HAS_BIAS, ME, NQB, KT, MASKED>(L, w, bias_t, mask_t, N, nqb, l16, g, key0, tail_keys, [&](int qb) {
+            if (qb == fetch_at && b_next < p.bw) fetch_unit(b_next);
+        });
 
-        // ---- epilogue dk, dv: lane (key, g) holds d = 16dt + 4g + i ----
+        // ---- epilogue dk, dv: lane (key, g) holds d = 16dt + 4g + i; k_hat and 1/|k| come from LDS ----
 #pragma unroll
         for (int kt = 0; kt < KT; kt++) {
             const int key = key0 + 16 * kt;
             const bool key_ok = key < N;
             float x[8], a[8];
-            float ss = 0.f, dot = 0.f;
+            float dot = 0.f;
 #pragma unroll
             for (int dt = 0; dt < 2; dt++) {
-                V4 k4;
-#pragma unroll
-                for (int i = 0; i < 4; i++) k4[i] = 0;
-                if (key_ok) k4 = *reinterpret_cast<const V4*>(kptr + (int64_t)key * p.k.sn + 16 * dt + 4 * g);
+                const V4 k4 = *reinterpret_cast<const V4*>(L.Ks + key * kRow + 16 * dt + 4 * g);
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     x[4 * dt + i] = (float)k4[i];
                     a[4 * dt + i] = w.dkacc[kt][dt][i] * kLn2;      // undo the log2e folded into Q_hat
-                    ss += x[4 * dt + i] * x[4 * dt + i];
+                    dot += a[4 * dt + i] * x[4 * dt + i];
                 }
             }
-            ss = xor32_add(xor16_add(ss));
-            const float nrm = sqrtf(ss);
-            const float inv = 1.0f / fmaxf(nrm, kNormEps);
-#pragma unroll
-            for (int j = 0; j < 8; j++) { x[j] *= inv; dot += a[j] * x[j]; }
             dot = xor32_add(xor16_add(dot));
-            const float proj = nrm > kNormEps ? dot : 0.f;
+            const float ki = L.kinv[key];
+            const float inv = fabsf(ki);
+            const float proj = ki > 0.f ? dot : 0.f;
             if (key_ok) {
                 E* dkp = reinterpret_cast<E*>(const_cast<void*>(p.dk.ptr)) + b * p.dk.sb + h * p.dk.sh + (int64_t)key * p.dk.sn;
                 E* dvp = reinterpret_cast<E*>(const_cast<void*>(p.dv.ptr)) + b * p.dv.sb + h * p.dv.sh + (int64_t)key * p.dv.sn;
@@ -299,23 +390,14 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
                 }
             }
         }
-    };
-    // units whose window mask is all zero first, then the masked ones: two straight loops, each with
-    // its own copy of the block sequence, instead of a branch inside every block
-    if (MASK_DT >= 0) {
-        for (int b = grp; b < p.bw; b += p.groups)
-            if (p.mask_live && !p.mask_live[b % p.n_windows]) process_unit(std::false_type{}, b);
-        for (int b = grp; b < p.bw; b += p.groups)
-            if (!p.mask_live || p.mask_live[b % p.n_windows]) process_unit(std::true_type{}, b);
-    } else {
-        for (int b = grp; b < p.bw; b += p.groups) process_unit(std::false_type{}, b);
+        b = b_next;
     }
 
     // ---- flush the per-workgroup partial sums ----
     if (HAS_BIAS) {
 #pragma unroll
         for (int kt = 0; kt < KT; kt++) {
-            float* dst = p.part_dbias + (((int64_t)h * p.groups + grp) * NPk + key0 + 16 * kt) * R;
+            float* dst = p.part_dbias + (((int64_t)h * p.db_parts + p.db_slot0 + grp) * NPk + key0 + 16 * kt) * R;
 #pragma unroll
             for (int qb = 0; qb < NQB; qb++) {
                 if (qb < nqb) {
@@ -361,10 +443,10 @@ __global__ void __launch_bounds__(256) reduce_kernel(const BwdParams p, int npk,
         const int q0 = blockIdx.x * 32, k0 = blockIdx.y * 8;
         float acc = 0.f;
         if (k0 + ty < npk) {
-            const float* src = p.part_dbias + (((int64_t)h * p.groups) * npk + k0 + ty) * r + q0 + tx;
+            const float* src = p.part_dbias + (((int64_t)h * p.db_parts) * npk + k0 + ty) * r + q0 + tx;
             const int64_t gs = (int64_t)npk * r;
 #pragma unroll 4
-            for (int gi = 0; gi < p.groups; gi++) acc += src[gi * gs];
+            for (int gi = 0; gi < p.db_parts; gi++) acc += src[gi * gs];
         }
         tile[ty][tx] = acc;
         __syncthreads();
@@ -421,7 +503,7 @@ static BwdPlan make_plan(int heads, int n, int bw, bool has_bias, bool has_mask,
     pl.groups = groups;
     size_t off = 0;
     pl.off_dbias = off;
-    if (has_bias) off += align256((size_t)heads * groups * pl.npk * pl.r * 4);
+    if (has_bias) off += align256((size_t)heads * 2 * groups * pl.npk * pl.r * 4);
     dq_geometry(n, &pl.dq_waves, &pl.dq_chunks);
     pl.ds_parts = bw * pl.dq_chunks;
     pl.off_dscale = off;
@@ -440,21 +522,52 @@ size_t backward_workspace_bytes(int heads, int n, int bw, bool has_bias, bool ha
     return make_plan(heads, n, bw, has_bias, has_mask, n_windows, cus).total;
 }
 
+// Persistent workgroups must all be resident at once: ask the runtime how many fit on a CU.
+template <class K>
+static int resident_per_cu(K kern, int threads) {
+    int n = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kern, threads, 0) != hipSuccess || n < 1) n = 1;
+    return n;
+}
+
 template <int DT, bool HAS_BIAS, int MASK_DT, int NQB, int KT>
-static hipError_t launch_main(const BwdParams& p, const BwdPlan& pl, hipStream_t st) {
-    auto kern = bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT>;
+static hipError_t launch_main(BwdParams p, const BwdPlan& pl, hipStream_t st, int* groups_out) {
+    // never more workgroups per head than the plan sized the workspace for
+    static const int fit = [&] {
+        const int a = resident_per_cu(bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, false>, 64 * pl.waves);
+        const int b = resident_per_cu(bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, true>, 64 * pl.waves);
+        return a < b ? a : b;
+    }();
+    int groups = (p.cus * fit) / p.heads;
+    if (groups < 1) groups = 1;
+    if (groups > pl.groups) groups = pl.groups;
+    p.groups = groups;
+    p.db_parts = (MASK_DT >= 0 && p.mask_live != nullptr) ? 2 * groups : groups;
+    const dim3 grid(p.heads * groups), block(64 * pl.waves);
     if (p.ev_start) (void)hipEventRecord(p.ev_start, st);
-    hipLaunchKernelGGL(kern, dim3(p.heads * pl.groups), dim3(64 * pl.waves), pl.smem, st, p);
+    // launch for the units whose mask is all zero (or every unit when there is no mask) ...
+    if (MASK_DT < 0 || p.mask_live != nullptr) {
+        p.db_slot0 = 0;
+        hipLaunchKernelGGL((bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, false>), grid, block, 0, st, p);
+    }
+    // ... and for the units whose mask is live
+    if (MASK_DT >= 0) {
+        p.db_slot0 = p.mask_live != nullptr ? groups : 0;
+        hipLaunchKernelGGL((bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, true>), grid, block, 0, st, p);
+    }
     if (p.ev_stop) (void)hipEventRecord(p.ev_stop, st);
-    return hipGetLastError();
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    if (groups_out) { groups_out[0] = groups; groups_out[1] = p.db_parts; }
+    return hipSuccess;
 }
 
 
 template <int DT, bool HAS_BIAS, int MASK_DT>
-static hipError_t launch_nqb(const BwdParams& p, const BwdPlan& pl, hipStream_t st) {
-    if (pl.nqb_t == 2) return launch_main<DT, HAS_BIAS, MASK_DT, 2, 1>(p, pl, st);
-    if (pl.nqb_t == 4) return launch_main<DT, HAS_BIAS, MASK_DT, 4, 1>(p, pl, st);
-    return launch_main<DT, HAS_BIAS, MASK_DT, 8, 2>(p, pl, st);
+static hipError_t launch_nqb(const BwdParams& p, const BwdPlan& pl, hipStream_t st, int* groups_out) {
+    if (pl.nqb_t == 2) return launch_main<DT, HAS_BIAS, MASK_DT, 2, 1>(p, pl, st, groups_out);
+    if (pl.nqb_t == 4) return launch_main<DT, HAS_BIAS, MASK_DT, 4, 1>(p, pl, st, groups_out);
+    return launch_main<DT, HAS_BIAS, MASK_DT, 8, 2>(p, pl, st, groups_out);
 }
 
 template <int DT>
@@ -491,16 +604,19 @@ static hipError_t launch_bwd_dt(BwdParams p, bool has_bias, int mask_dt, hipStre
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
+    int gr_out[2] = {pl.groups, pl.groups};
     if (has_bias) {
-        if (mask_dt < 0) e = launch_nqb<DT, true, -1>(p, pl, st);
-        else if (mask_dt == FWA2_F32) e = launch_nqb<DT, true, FWA2_F32>(p, pl, st);
-        else e = launch_nqb<DT, true, DT>(p, pl, st);
+        if (mask_dt < 0) e = launch_nqb<DT, true, -1>(p, pl, st, gr_out);
+        else if (mask_dt == FWA2_F32) e = launch_nqb<DT, true, FWA2_F32>(p, pl, st, gr_out);
+        else e = launch_nqb<DT, true, DT>(p, pl, st, gr_out);
     } else {
-        if (mask_dt < 0) e = launch_nqb<DT, false, -1>(p, pl, st);
-        else if (mask_dt == FWA2_F32) e = launch_nqb<DT, false, FWA2_F32>(p, pl, st);
-        else e = launch_nqb<DT, false, DT>(p, pl, st);
+        if (mask_dt < 0) e = launch_nqb<DT, false, -1>(p, pl, st, gr_out);
+        else if (mask_dt == FWA2_F32) e = launch_nqb<DT, false, FWA2_F32>(p, pl, st, gr_out);
+        else e = launch_nqb<DT, false, DT>(p, pl, st, gr_out);
     }
     if (e != hipSuccess) return e;
+    p.groups = gr_out[0];
+    p.db_parts = gr_out[1];
     e = launch_backward_dq(p, DT, has_bias, mask_dt, st);
     if (e != hipSuccess) return e;
     if (has_bias || p.scale_kind == FWA2_SCALE_TENSOR) {

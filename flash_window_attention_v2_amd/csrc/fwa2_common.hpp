@@ -205,7 +205,9 @@ struct BwdParams {
     // filled in by the launcher
     int waves;        // wavefronts per workgroup = key tiles of 16
     int groups;       // workgroups per head (each walks bw = g, g + groups, ...)
-    float* part_dbias;   // [H, groups, NP, NQ] fp32, key-major
+    float* part_dbias;   // [H, db_parts, NP, NQ] fp32, key-major
+    int db_parts;        // partial tiles per head: groups per launch of the key-side kernel
+    int db_slot0;        // first partial slot of the current launch
     float* part_dscale;  // [H, ds_parts] fp32, one per workgroup of the dq kernel
     int ds_parts;        // bw * dq_chunks
     int dq_waves;        // wavefronts per workgroup of the dq kernel
