@@ -170,7 +170,8 @@ def main():
     kern_ms = events.elapsed_ms()
     kern_avg = sum(kern_ms) / len(kern_ms)
     fl_all = flops_matmul(bw, cfg["heads"], cfg["n"], cfg["d"])
-    fl_bwd = flops_matmul(bw, cfg["heads"], cfg["n"], cfg["d"], fwd=False)
+    # the dominant kernel (key-side backward: S recompute, dP, dV, dK) does 8 N^2 d flops per unit
+    fl_bwd = 8 * cfg["n"] * cfg["n"] * cfg["d"] * bw * cfg["heads"]
     tflops = fl_all / (ms * 1e-3) * 1e-12
     achieved = fl_bwd / (kern_avg * 1e-3) * 1e-12
 
@@ -181,11 +182,11 @@ def main():
         "config": {"workload": "C3: B64 x 64 windows, H3, N256, d32, bf16, shift-8 mask, fwd+bwd", "bw": bw,
                    "heads": cfg["heads"], "n": cfg["n"], "head_dim": cfg["d"]},
         "pct_mfma_peak": round(100 * tflops / MFMA_BF16_PEAK_TFLOPS, 2),
-        "roofline": {"bound": "mfma", "kernel": "bwd_kernel", "achieved": round(achieved, 2),
+        "roofline": {"bound": "mfma", "kernel": "bwd_kernel (dk, dv, dbias; both launches)", "achieved": round(achieved, 2),
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": BWD_KERNEL_TRAFFIC_BYTES,
                      "kernel_ms": round(kern_avg, 4),
-                     "hbm_frac_of_8TBs": round(bytes_min(bw, cfg["heads"], cfg["n"], cfg["d"], cfg["n_windows"], fwd=False)
+                     "hbm_frac_of_8TBs": round(bw * cfg["heads"] * (7 * cfg["n"] * cfg["d"] * 2 + 4 * cfg["n"])
                                                / (kern_avg * 1e-3) / (HBM_PEAK_GBS * 1e9), 4)},
     }
 

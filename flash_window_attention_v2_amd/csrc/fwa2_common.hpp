@@ -24,6 +24,7 @@ constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 constexpr float kLn100 = 4.605170185988092f;
 constexpr float kNormEps = 1e-12f;
+constexpr int kScoreDT = FWA2_F16;   // element type of q_hat / k_hat in the forward score product
 
 // Element-type traits: E = storage element, V8 / V4 = 8- and 4-wide vectors.
 template <int DT> struct Elem;

@@ -19,7 +19,8 @@
 // ds_read_b64_tr_b16.
 //
 // Numerics.  Scores live in the log2 domain: q_hat is multiplied by
-// s * log2(e) in fp32 before it is rounded to the input dtype, bias and mask
+// s * log2(e) in fp32 before it is rounded to fp16 (also for bf16 inputs: the
+// normalised vectors fit fp16's range and gain 3 mantissa bits), bias and mask
 // are multiplied by log2(e) in fp32, exp is v_exp_f32 (2^x).  Softmax state,
 // accumulators and the log-sum-exp are fp32; P is rounded to the input dtype
 // for the second MFMA (as the reference does, attn_kernel_forward.py:225-226).
@@ -33,12 +34,16 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdParams p) {
     typedef typename Elem<DT>::V8 V8;
     typedef typename Elem<DT>::V4 V4;
     typedef typename MaskElem<DT, MASK_DT>::E ME;
+    // the cosine scores always go through the fp16 matrix path: q_hat and k_hat lie in [-1, 1]
+    // (times a scale <= 100 log2 e), where fp16 keeps 3 more mantissa bits than bf16
+    typedef typename Elem<kScoreDT>::E SE;
+    typedef typename Elem<kScoreDT>::V8 SV8;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     const int N = p.n;
     const int chunk_rows = (min(N, kKeyChunk) + 63) & ~63;
-    E* Ks = reinterpret_cast<E*>(smem_raw);
-    E* Vs = Ks + chunk_rows * kLdsStride;
+    SE* Ks = reinterpret_cast<SE*>(smem_raw);
+    E* Vs = reinterpret_cast<E*>(Ks + chunk_rows * kLdsStride);
 
     const int tid = threadIdx.x;
     const int nthreads = blockDim.x;
@@ -74,7 +79,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdParams p) {
     const bool wave_live = q0 < N;
 
     // ---- Q operand: normalise, fold the scale, round to the input dtype ----
-    V8 bq0 = zero8<V8>(), bq1 = zero8<V8>();
+    SV8 bq0 = zero8<SV8>(), bq1 = zero8<SV8>();
     if (wave_live) {
         V8 a = zero8<V8>(), c = zero8<V8>();
         if (qv) {
@@ -90,7 +95,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdParams p) {
         ss = xor32_add(ss);
         const float sc = scale2 * inv_norm(ss);
 #pragma unroll
-        for (int j = 0; j < 8; j++) { bq0[j] = (E)(xa[j] * sc); bq1[j] = (E)(xc[j] * sc); }
+        for (int j = 0; j < 8; j++) { bq0[j] = (SE)(xa[j] * sc); bq1[j] = (SE)(xc[j] * sc); }
     }
 
     const E* bias_row = nullptr;
@@ -128,10 +133,10 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdParams p) {
             for (int j = 0; j < 8; j++) ss += x[j] * x[j];
             ss = quad_add(ss);
             const float inv = inv_norm(ss);
-            V8 kn;
+            SV8 kn;
 #pragma unroll
-            for (int j = 0; j < 8; j++) kn[j] = (E)(x[j] * inv);
-            st8<V8>(Ks + r * kLdsStride + dch, kn);
+            for (int j = 0; j < 8; j++) kn[j] = (SE)(x[j] * inv);
+            st8<SV8>(Ks + r * kLdsStride + dch, kn);
             st8<V8>(Vs + r * kLdsStride + dch, vv);
         }
         __syncthreads();
@@ -143,14 +148,14 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdParams p) {
             f32x16 acc[2];
 #pragma unroll
             for (int t = 0; t < 2; t++) {
-                const E* krow = Ks + (kb * 64 + 32 * t + swap_bits23(col)) * kLdsStride + 8 * hf;
-                V8 a0 = ld8<V8>(krow);
-                V8 a1 = ld8<V8>(krow + 16);
+                const SE* krow = Ks + (kb * 64 + 32 * t + swap_bits23(col)) * kLdsStride + 8 * hf;
+                SV8 a0 = ld8<SV8>(krow);
+                SV8 a1 = ld8<SV8>(krow + 16);
                 f32x16 z;
 #pragma unroll
                 for (int i = 0; i < 16; i++) z[i] = 0.f;
-                z = Elem<DT>::mfma32(a0, bq0, z);
-                acc[t] = Elem<DT>::mfma32(a1, bq1, z);
+                z = Elem<kScoreDT>::mfma32(a0, bq0, z);
+                acc[t] = Elem<kScoreDT>::mfma32(a1, bq1, z);
             }
             // register i of tile t <-> key kbase + 32t + 16(i/8) + 8hf + i%8
             const int kbase = c0 + kb * 64;
