@@ -26,8 +26,8 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0     # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0              # MI355X HBM3E
 # HBM bytes per launch of the backward kernel at the benchmark shape, from
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a copy kernel of known size
-# (profiles/bwd_kernel_C3_pmc.txt); None until measured.
-BWD_KERNEL_TRAFFIC_BYTES = None
+# (profiles/kernels_C3_fwd_bwd.txt: FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, both launches).
+BWD_KERNEL_TRAFFIC_BYTES = 2.493e9
 
 
 def log(*a):
@@ -125,6 +125,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip forward-only, N=64 and memory figures")
+    ap.add_argument("--copy-bytes", type=int, default=0,
+                    help="also run one plain device copy of this many bytes (reference point for HBM counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (the hot path has no cross-GPU step); use --gpus 1")
@@ -230,6 +232,15 @@ def main():
         extras["c2_tflops"] = round(flops_matmul(bw2, c2["heads"], c2["n"], c2["d"]) / ms2 * 1e-9, 2)
         del dev2
         result["extras"] = extras
+
+    if args.copy_bytes:
+        src = torch.empty(args.copy_bytes, dtype=torch.uint8, device="cuda").fill_(1)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        result["copy_bytes"] = args.copy_bytes
+        del src, dst
 
     if not args.no_cpu:
         log("[bench] CPU baseline (classic fp32 on host cores)")

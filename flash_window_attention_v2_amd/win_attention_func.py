@@ -35,3 +35,16 @@ def win_attention_torch(q, k, v, logit_scale=None, bias=None, mask=None):
         scores = scores.view(bw // n_w, n_w, heads, n_q, n_k) + mask.unsqueeze(1).unsqueeze(0)
         scores = scores.view(bw, heads, n_q, n_k)
     return torch.softmax(scores, dim=-1) @ v
+
+
+_compiled_classic = None
+
+
+def win_attention_torch_compile(q, k, v, logit_scale=None, bias=None, mask=None):
+    """`win_attention_torch` under `torch.compile`, the third operator the reference
+    exports (flash_win_attn_v2/win_attention_func.py:42) as a comparison line for its
+    benchmarks.  Compiled on first use; nothing in the fused path depends on it."""
+    global _compiled_classic
+    if _compiled_classic is None:
+        _compiled_classic = torch.compile(win_attention_torch)
+    return _compiled_classic(q, k, v, logit_scale, bias, mask)

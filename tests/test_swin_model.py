@@ -1,0 +1,278 @@
+"""Caller side of the hot path: the Swin V2 harness around the operator.
+
+CPU tests pin the harness against closed forms (parameter counts, state_dict names, the
+shifted-window mask, index buffers, patch merging order).  GPU tests run WindowAttention and
+the whole model through the fused kernels and compare with the classic path in fp32.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import swin_inputs as si
+from oracle.classic_torch import win_attention_classic
+import flash_window_attention_v2_amd as fwa
+from flash_window_attention_v2_amd import swin_transformer_v2 as swin
+
+
+def test_alias_package_exports():
+    import flash_win_attn_v2 as ref_name
+    from flash_win_attn_v2.swin_transformer_v2 import WindowAttention as wa
+    for name in ("WindowAttention", "SwinTransformerV2", "flash_win_attn_v2_func", "win_attention_torch",
+                 "win_attention_torch_compile"):
+        assert getattr(ref_name, name) is getattr(fwa, name)
+    assert wa is swin.WindowAttention
+
+
+@pytest.mark.parametrize("patch,img,expected", [(4, 256, 28_347_154), (2, 128, 28_343_698)])
+def test_parameter_count(patch, img, expected):
+    model = swin.SwinTransformerV2(img_size=img, patch_size=patch, is_flash=False)
+    assert sum(p.numel() for p in model.parameters()) == expected
+
+
+def test_block_parameter_count_closed_form():
+    for c, h in ((96, 3), (192, 6), (384, 12)):
+        blk = swin.SwinTransformerBlock(c, (16, 16), h, window_size=8, shift_size=4, is_flash=False)
+        assert sum(p.numel() for p in blk.parameters()) == 12 * c * c + 12 * c + 1536 + 513 * h
+
+
+def test_state_dict_names():
+    model = swin.SwinTransformerV2(img_size=64, patch_size=4, embed_dim=32, depths=[2, 2], num_heads=[1, 2],
+                                   window_size=8, is_flash=False, num_classes=10)
+    keys = set(model.state_dict().keys())
+    block = "layers.0.blocks.1."
+    for name in ("attn.logit_scale", "attn.q_bias", "attn.v_bias", "attn.qkv.weight", "attn.proj.weight",
+                 "attn.proj.bias", "attn.cpb_mlp.0.weight", "attn.cpb_mlp.0.bias", "attn.cpb_mlp.2.weight",
+                 "attn.relative_coords_table", "attn.relative_position_index", "attn_mask", "norm1.weight",
+                 "norm2.bias", "mlp.fc1.weight", "mlp.fc2.bias"):
+        assert block + name in keys, name
+    assert "layers.0.blocks.0.attn_mask" not in keys            # unshifted block: buffer is None
+    assert "attn.qkv.bias" not in {k.split("blocks.1.")[-1] for k in keys}
+    for name in ("patch_embed.proj.weight", "patch_embed.norm.weight", "layers.0.downsample.reduction.weight",
+                 "layers.0.downsample.norm.weight", "norm.weight", "head.weight", "head.bias"):
+        assert name in keys, name
+    assert not any(k.startswith("layers.1.downsample") for k in keys)
+
+
+def test_initialisation():
+    model = swin.SwinTransformerV2(img_size=64, embed_dim=32, depths=[2], num_heads=[2], is_flash=False)
+    blk = model.layers[0].blocks[1]
+    assert float(blk.norm1.weight.detach().abs().max()) == 0.0 and float(blk.norm2.weight.detach().abs().max()) == 0.0
+    assert float(model.norm.weight.min()) == 1.0
+    assert torch.allclose(blk.attn.logit_scale, torch.full((2, 1, 1), math.log(10.0)))
+    assert float(blk.attn.q_bias.abs().max()) == 0.0
+    w = blk.mlp.fc1.weight
+    assert float(w.abs().max()) <= 2.0 and 0.015 < float(w.std()) < 0.025
+
+
+@pytest.mark.parametrize("res,ws,shift", [(32, 8, 4), (64, 8, 4), (128, 16, 8), (14, 7, 3)])
+def test_block_mask_matches_closed_form(res, ws, shift):
+    blk = swin.SwinTransformerBlock(32, (res, res), 1, window_size=ws, shift_size=shift, is_flash=False)
+    assert blk.attn_mask.dtype == torch.float32
+    assert torch.equal(blk.attn_mask, si.shifted_window_mask(res, ws, shift))
+
+
+def test_rectangular_mask_against_painting():
+    h, w, ws, shift = 16, 24, 8, 4
+    img = np.zeros((h, w))
+    label = 0
+    for r0, r1 in ((0, h - ws), (h - ws, h - shift), (h - shift, h)):
+        for c0, c1 in ((0, w - ws), (w - ws, w - shift), (w - shift, w)):
+            img[r0:r1, c0:c1] = label
+            label += 1
+    got = swin.shifted_window_attn_mask((h, w), ws, shift).numpy()
+    k = 0
+    for wr in range(h // ws):
+        for wc in range(w // ws):
+            tile = img[wr * ws:(wr + 1) * ws, wc * ws:(wc + 1) * ws].reshape(-1)
+            np.testing.assert_array_equal(got[k], np.where(tile[None, :] != tile[:, None], -100.0, 0.0))
+            k += 1
+
+
+def test_small_resolution_disables_shift():
+    blk = swin.SwinTransformerBlock(32, (8, 8), 1, window_size=8, shift_size=4, is_flash=False)
+    assert blk.shift_size == 0 and blk.window_size == 8 and blk.attn_mask is None
+    blk = swin.SwinTransformerBlock(32, (4, 4), 1, window_size=8, shift_size=4, is_flash=False)
+    assert blk.window_size == 4 and blk.attn.window_size == (4, 4)
+
+
+def test_index_buffers_match_closed_forms():
+    attn = swin.WindowAttention(32, (8, 8), 2, is_flash=False)
+    assert torch.equal(attn.relative_position_index, si.relative_position_index(8, 8))
+    assert torch.allclose(attn.relative_coords_table, si.relative_coords_table(8, 8), atol=1e-6)
+    attn = swin.WindowAttention(32, (4, 6), 2, is_flash=False, pretrained_window_size=[12, 12])
+    assert torch.equal(attn.relative_position_index, si.relative_position_index(4, 6))
+    assert torch.allclose(attn.relative_coords_table, si.relative_coords_table(4, 6, (12, 12)), atol=1e-6)
+    bias = attn.relative_position_bias()
+    assert bias.shape == (2, 24, 24) and bias.is_contiguous()
+    assert float(bias.min()) > 0.0 and float(bias.max()) < 16.0
+    # the bias depends on (i, j) only through the relative offset
+    assert torch.equal(bias[:, 0, 1], bias[:, 7, 8])
+
+
+def test_window_partition_round_trip_and_order():
+    x = torch.arange(2 * 8 * 12 * 3, dtype=torch.float32).view(2, 8, 12, 3)
+    win = swin.window_partition(x, 4)
+    assert win.shape == (2 * 2 * 3, 4, 4, 3)
+    # window index = (batch, window row, window column), batch outermost
+    assert torch.equal(win[1 * 6 + 1 * 3 + 2], x[1, 4:8, 8:12])
+    assert torch.equal(swin.window_reverse(win, 4, 8, 12), x)
+
+
+def test_patch_merging_channel_order():
+    pm = swin.PatchMerging((4, 6), 2, norm_layer=torch.nn.Identity)
+    with torch.no_grad():
+        pm.reduction.weight.copy_(torch.eye(4, 8))       # output c = merged channel c
+    x = torch.randn(1, 4 * 6, 2)
+    y = pm(x).view(1, 2, 3, 4)
+    g = x.view(1, 4, 6, 2)
+    expect = torch.cat([g[:, 0::2, 0::2], g[:, 1::2, 0::2], g[:, 0::2, 1::2], g[:, 1::2, 1::2]], -1)[..., :4]
+    assert torch.equal(y, expect)
+
+
+def test_flash_rejects_attention_dropout():
+    with pytest.raises(AssertionError):
+        swin.WindowAttention(32, (8, 8), 1, is_flash=True, attn_drop=0.1)
+
+
+def _classic_module_output(attn, x, mask):
+    """WindowAttention.forward restated around the oracle's classic operator."""
+    b_, n, c = x.shape
+    w = attn.qkv.weight
+    qkv_bias = torch.cat((attn.q_bias, torch.zeros_like(attn.v_bias), attn.v_bias))
+    qkv = (x @ w.t() + qkv_bias).view(b_, n, 3, attn.num_heads, -1).permute(2, 0, 3, 1, 4)
+    out = win_attention_classic(qkv[0], qkv[1], qkv[2], attn.logit_scale, attn.relative_position_bias(), mask)
+    return out.transpose(1, 2).reshape(b_, n, c) @ attn.proj.weight.t() + attn.proj.bias
+
+
+def test_window_attention_classic_path_cpu():
+    torch.manual_seed(0)
+    attn = swin.WindowAttention(64, (4, 4), 2, is_flash=False).double()
+    with torch.no_grad():
+        attn.q_bias.normal_()
+        attn.v_bias.normal_()
+    mask = si.shifted_window_mask(8, 4, 2).double()
+    x = torch.randn(2 * 4, 16, 64, dtype=torch.float64)
+    assert torch.allclose(attn(x, mask), _classic_module_output(attn, x, mask), atol=1e-10)
+    assert torch.allclose(attn(x), _classic_module_output(attn, x, None), atol=1e-10)
+
+
+def test_model_cpu_forward_backward():
+    torch.manual_seed(0)
+    model = swin.SwinTransformerV2(img_size=32, patch_size=2, embed_dim=32, depths=[2, 2], num_heads=[1, 2],
+                                   window_size=4, is_flash=False, num_classes=7, use_checkpoint=True, ape=True)
+    out = model(torch.randn(2, 3, 32, 32))
+    assert out.shape == (2, 7)
+    out.sum().backward()
+    assert model.patch_embed.proj.weight.grad is not None
+    assert model.no_weight_decay() == {"absolute_pos_embed"}
+
+
+# ---- GPU: the module and the model through the fused kernels ---------------------------------
+
+def _randomise_norms(model, seed=1):
+    g = torch.Generator().manual_seed(seed)
+    with torch.no_grad():
+        for m in model.modules():
+            if isinstance(m, torch.nn.LayerNorm):
+                m.weight.copy_(1.0 + 0.1 * torch.randn(m.weight.shape, generator=g))
+                m.bias.copy_(0.1 * torch.randn(m.bias.shape, generator=g))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_window_attention_module_gpu(dtype):
+    torch.manual_seed(0)
+    dev = torch.device("cuda")
+    flash = swin.WindowAttention(96, (8, 8), 3, is_flash=True).to(dev)
+    with torch.no_grad():
+        flash.q_bias.normal_(std=0.5)
+        flash.v_bias.normal_(std=0.5)
+    classic = swin.WindowAttention(96, (8, 8), 3, is_flash=False).to(dev)
+    classic.load_state_dict(flash.state_dict())
+    flash = flash.to(dtype)
+    mask = si.shifted_window_mask(32, 8, 4).to(dev)          # fp32 mask, as the block holds it
+    x = torch.randn(2 * 16, 64, 96, device=dev)
+    g = torch.randn(2 * 16, 64, 96, device=dev)
+
+    xf = x.to(dtype).requires_grad_()
+    yf = flash(xf, mask)
+    yf.backward(g.to(dtype))
+    # classic in fp32 on the values the low-precision module actually holds
+    classic.load_state_dict({k: v.float() for k, v in flash.state_dict().items()})
+    xc = x.to(dtype).float().requires_grad_()
+    yc = classic(xc, mask)
+    yc.backward(g.to(dtype).float())
+
+    def rel(a, b):
+        return float((a.float() - b).abs().max() / b.abs().max())
+
+    tol = 3e-2 if dtype == torch.bfloat16 else 1e-2
+    assert yf.dtype == dtype
+    assert rel(yf, yc) < tol
+    assert rel(xf.grad, xc.grad) < tol
+    for name in ("qkv.weight", "q_bias", "v_bias", "logit_scale", "cpb_mlp.0.weight", "cpb_mlp.2.weight",
+                 "proj.weight"):
+        pf = dict(flash.named_parameters())[name].grad
+        pc = dict(classic.named_parameters())[name].grad
+        assert pf is not None and rel(pf, pc) < 2 * tol, name
+
+
+@pytest.mark.gpu
+def test_model_flash_matches_classic_gpu():
+    """Whole-model step at a reduced width: bf16 model on the fused kernels against the same weights
+    on the classic path in fp32, LayerNorms away from their zero initialisation and no stochastic
+    depth so both runs are deterministic functions of the weights."""
+    torch.manual_seed(0)
+    dev = torch.device("cuda")
+    kw = dict(img_size=64, patch_size=2, embed_dim=96, depths=[2, 2], num_heads=[3, 6], window_size=8,
+              num_classes=10, drop_path_rate=0.0)
+    ref = swin.SwinTransformerV2(is_flash=False, **kw)
+    _randomise_norms(ref)
+    ref = ref.to(dev)
+    fused = swin.SwinTransformerV2(is_flash=True, **kw).to(dev)
+    fused.load_state_dict(ref.state_dict())
+    fused = fused.to(torch.bfloat16)
+    eager = swin.SwinTransformerV2(is_flash=False, **kw).to(dev)
+    eager.load_state_dict(ref.state_dict())
+    eager = eager.to(torch.bfloat16)
+
+    x = torch.randn(4, 3, 64, 64, device=dev)
+    labels = torch.randint(0, 10, (4,), device=dev)
+    losses, grads = {}, {}
+    for name, model, inp in (("ref", ref, x), ("fused", fused, x.bfloat16()), ("eager", eager, x.bfloat16())):
+        logits = model(inp)
+        loss = torch.nn.functional.cross_entropy(logits.float(), labels)
+        loss.backward()
+        losses[name] = float(loss)
+        grads[name] = {k: p.grad.float() for k, p in model.named_parameters()}
+    assert abs(losses["fused"] - losses["ref"]) < 3e-2
+
+    def worst(name):
+        return max(float((grads[name][k] - grads["ref"][k]).abs().max() / (grads["ref"][k].abs().max() + 1e-6))
+                   for k in grads["ref"])
+
+    # the fused path in bf16 must be about as close to fp32 as the eager bf16 model is
+    assert worst("fused") < max(2.0 * worst("eager"), 5e-2)
+
+
+@pytest.mark.gpu
+def test_model_checkpointing_gpu():
+    torch.manual_seed(0)
+    dev = torch.device("cuda")
+    kw = dict(img_size=64, patch_size=2, embed_dim=96, depths=[2], num_heads=[3], window_size=8, num_classes=5,
+              drop_path_rate=0.0)
+    plain = swin.SwinTransformerV2(use_checkpoint=False, **kw)
+    _randomise_norms(plain)
+    plain = plain.to(dev).to(torch.bfloat16)
+    ckpt = swin.SwinTransformerV2(use_checkpoint=True, **kw).to(dev).to(torch.bfloat16)
+    ckpt.load_state_dict(plain.state_dict())
+    x = torch.randn(2, 3, 64, 64, device=dev, dtype=torch.bfloat16)
+    plain(x).float().sum().backward()
+    ckpt(x).float().sum().backward()
+    for (k, a), (_, b) in zip(plain.named_parameters(), ckpt.named_parameters()):
+        # recompute replays the same deterministic kernels; torch's own scatter-adds (bias gather
+        # backward) may reorder their sums, hence a tolerance rather than bit equality
+        scale = float(a.grad.float().abs().max()) + 1e-6
+        assert float((a.grad.float() - b.grad.float()).abs().max()) <= 2e-2 * scale, k
