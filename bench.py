@@ -40,6 +40,13 @@ def flops_matmul(bw, heads, n, d, fwd=True, bwd=True):
     return per * n * n * d * bw * heads
 
 
+def flops_reference_convention(bw, heads, n, d, fwd_bwd=True):
+    """FLOP count the reference's own benchmark quotes (benchmark/utils.py:26-67): per (bw, head)
+    6 N d + 4 N^2 d + 6 N^2, and three times that for forward+backward (benchmark/bench_attn.py:99)."""
+    per = 6 * n * d + 4 * n * n * d + 6 * n * n
+    return per * bw * heads * (3 if fwd_bwd else 1)
+
+
 def bytes_min(bw, heads, n, d, n_windows, fwd=True, bwd=True, e=2):
     """Algorithmic HBM bytes: q,k,v,o (+lse) forward; q,k,v,o,do,dq,dk,dv (+lse, dbias) backward;
     bias and mask once per pass."""
@@ -200,6 +207,9 @@ def main():
                                                                dev["bias"], dev["mask"]), args.steps, args.warmup, torch)
         extras["fwd_ms"] = round(f_ms, 4)
         extras["fwd_tflops"] = round(flops_matmul(bw, cfg["heads"], cfg["n"], cfg["d"], bwd=False) / f_ms * 1e-9, 2)
+        extras["tflops_reference_convention"] = round(flops_reference_convention(bw, cfg["heads"], cfg["n"], cfg["d"]) / ms * 1e-9, 2)
+        extras["fwd_tflops_reference_convention"] = round(
+            flops_reference_convention(bw, cfg["heads"], cfg["n"], cfg["d"], fwd_bwd=False) / f_ms * 1e-9, 2)
         extras["fwd_hbm_gbs"] = round(bytes_min(bw, cfg["heads"], cfg["n"], cfg["d"], cfg["n_windows"], bwd=False) / f_ms * 1e-6, 1)
         extras["fwd_bwd_hbm_gbs"] = round(bytes_min(bw, cfg["heads"], cfg["n"], cfg["d"], cfg["n_windows"]) / ms * 1e-6, 1)
         # peak memory of the op against the classic path in the same dtype on the GPU
