@@ -166,6 +166,7 @@ int fwa2_forward(const fwa2_problem* p) {
     k.default_scale = 1.0f / sqrtf((float)p->head_dim);
     k.side_vec = (!p->bias.ptr || row_vec_ok(p->bias.ptr, p->bias.stride_a, p->bias.stride_n, p->n)) &&
                  (!p->mask.ptr || row_vec_ok(p->mask.ptr, p->mask.stride_a, p->mask.stride_n, p->n));
+    k.cus = cu_count();
     hipError_t e = fwa2::launch_forward(k, p->dtype, p->bias.ptr != nullptr, p->mask.ptr ? p->mask_dtype : -1,
                                         (hipStream_t)p->stream);
     if (e != hipSuccess) return fail(FWA2_ERR_HIP, "forward launch: %s", hipGetErrorString(e));

@@ -174,7 +174,9 @@ struct FwdParams {
     int64_t bias_sh, bias_sn;
     const void* mask;
     int64_t mask_sw, mask_sn;
-    const uint8_t* mask_live;  // [n_windows] 1 = window's mask has a non-zero entry; nullptr = assume all live
+    const uint8_t* mask_live;  // [n_windows] flags from the mask scan (0 = window's mask is all zero, bit 0 =
+                               // it has a non-zero entry, bit 1 = all entries <= 0 and every row keeps a 0);
+                               // nullptr = assume every window live and nothing known about it
     float* lse;
     int64_t lse_sb, lse_sh;
     int bw, heads, n, n_windows;
@@ -183,6 +185,8 @@ struct FwdParams {
     bool side_vec;    // rows of bias and mask may be read with 16-byte loads and n % 8 == 0
     int waves;        // wavefronts per workgroup
     int q_chunks;     // workgroups per (bw, head)
+    int cus;          // compute units of the device
+    int groups;       // persistent workgroups per head (resident-bias kernel)
 };
 
 struct BwdParams {

@@ -246,19 +246,29 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdParams p) {
     }
 }
 
-// One byte per window: does the window's [N, N] mask hold any non-zero entry?
+// One byte of flags per window.  0: the [N, N] mask is all zero.  Bit 0: it holds a non-zero entry.
+// Bit 1 (with bit 0): no entry is positive (or NaN) and every row keeps at least one exact zero, so
+// the mask can only remove keys and never removes all of a row.
 template <class ME>
 __global__ void __launch_bounds__(256) mask_scan_kernel(const ME* mask, int64_t sw, int64_t sn, int n,
                                                         uint8_t* live) {
     const int w = blockIdx.x;
     const ME* m = mask + w * sw;
-    int any = 0;
-    for (int i = threadIdx.x; i < n * n; i += blockDim.x) {
-        const int r = i / n, c = i - r * n;
-        any |= ((float)m[r * sn + c] != 0.f);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int any = 0, unsafe = 0;
+    for (int r = wave; r < n; r += 4) {       // one wavefront per row, coalesced along the row
+        int zero = 0;
+        for (int c = lane; c < n; c += 64) {
+            const float v = (float)m[r * sn + c];
+            any |= (v != 0.f);
+            unsafe |= !(v <= 0.f);
+            zero |= (v == 0.f);
+        }
+        if (!__any(zero)) unsafe = 1;
     }
     any = __syncthreads_or(any);
-    if (threadIdx.x == 0) live[w] = any ? 1 : 0;
+    unsafe = __syncthreads_or(unsafe);
+    if (threadIdx.x == 0) live[w] = any ? (unsafe ? 1 : 3) : 0;
 }
 
 template <int DT, bool HAS_BIAS, int MASK_DT>
@@ -282,7 +292,12 @@ static hipError_t launch_dt(const FwdParams& p, bool has_bias, int mask_dt, dim3
     return launch_one<DT, false, DT>(p, g, b, s, st);
 }
 
+int forward_resident_supported(int n);
+hipError_t launch_forward_resident(const FwdParams& p, int dtype, bool has_bias, int mask_dt, hipStream_t st);
+
 hipError_t launch_forward(FwdParams p, int dtype, bool has_bias, int mask_dt, hipStream_t st) {
+    // windows of up to 256 tokens keep the bias tile in registers; longer ones stream it
+    if (forward_resident_supported(p.n)) return launch_forward_resident(p, dtype, has_bias, mask_dt, st);
     const int q_tiles = (p.n + 31) / 32;
     p.waves = q_tiles < 8 ? q_tiles : 8;
     p.q_chunks = (q_tiles + p.waves - 1) / p.waves;

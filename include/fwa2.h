@@ -94,7 +94,7 @@ typedef struct fwa2_problem {
     const void*  logit_scale;/* [H] elements of `dtype`, stride 1; NULL unless FWA2_SCALE_TENSOR */
     fwa2_tensor3 bias;       /* [H, N, N] of `dtype`, or ptr NULL */
     fwa2_tensor3 mask;       /* [nW, N, N] of `mask_dtype`, or ptr NULL */
-    const uint8_t* mask_live;/* optional [nW] bytes from fwa2_mask_scan: 0 = that window's mask is all
+    const uint8_t* mask_live;/* optional [nW] flag bytes from fwa2_mask_scan: 0 = that window's mask is all
                                 zero and is skipped; NULL = every window's mask is read */
 
     float*  lse;             /* [BW, H, lse_stride_h] fp32 natural-log log-sum-exp per query row;
@@ -130,9 +130,12 @@ const char* fwa2_last_error(void);
 int fwa2_validate(const fwa2_problem* p, int backward);
 
 /*
- * live[w] = 1 if mask[w] holds any non-zero entry, else 0 (device bytes, one
- * per window).  Shifted-window masks are all zero for most windows; passing
- * the result as fwa2_problem.mask_live lets the kernels skip those reads.
+ * One byte of flags per window (device memory): live[w] = 0 if mask[w] is all
+ * zero; otherwise bit 0 is set, and bit 1 is set too when no entry is positive
+ * and every row keeps at least one exact zero (the mask only removes keys and
+ * never a whole row, as shifted-window masks do).  Shifted-window masks are all
+ * zero for most windows; passing the result as fwa2_problem.mask_live lets the
+ * kernels skip those reads and pick a cheaper softmax for the rest.
  * Has no counterpart in the reference, which always reads the mask.
  */
 int fwa2_mask_scan(const void* mask, int mask_dtype, int n_windows, int n, int64_t stride_w, int64_t stride_n,
