@@ -21,13 +21,17 @@
 // clamp of 100, masks with positive entries or fully masked rows) the same
 // loop runs with the usual running maximum.
 //
-// Per unit: K_hat (fp16) and V of the NEXT unit are fetched into registers
-// before the tiles of the current one are computed, normalised and written to
-// the other half of a double buffer afterwards; one barrier per unit.
+// Per unit: K and V rows of the NEXT unit are fetched straight into an LDS
+// landing area (global_load_lds, no registers held) before the tiles of the
+// current one are computed; afterwards every wavefront normalises the 16 rows
+// it fetched into the other half of a double buffer; one barrier per unit.
+// Units whose window mask is live go through a second launch of the MASKED
+// instantiation, so the common unmasked code carries no mask registers.
 #include "fwa2_common.hpp"
 
 namespace fwa2 {
 
+constexpr int kLiveCache = 1024;    // windows whose mask flags are cached in LDS
 constexpr float kGapLimit = 96.f;   // largest tolerated (row bound - largest logit), log2 domain
 
 __device__ __forceinline__ float xor16_max(float x) {
@@ -38,28 +42,30 @@ __device__ __forceinline__ float xor16_max(float x) {
 __device__ __forceinline__ float col_max(float x) { return xor32_max(xor16_max(x)); }
 __device__ __forceinline__ float col_add(float x) { return xor32_add(xor16_add(x)); }
 
-// 4 consecutive entries of a bias / mask row as floats; columns >= n read as `pad`.
+// 8 consecutive entries of a bias / mask row in their storage type; columns >= n read as `pad`.
 template <bool VEC, class T>
-__device__ __forceinline__ void load_side4(const T* row, int c0, int n, float pad, float* x) {
-    typedef T TV4 __attribute__((ext_vector_type(4)));
-    if (VEC) {   // n % 8 == 0 and rows 16-byte aligned: a group of 4 is all real or all padding
+__device__ __forceinline__ auto load_raw8(const T* row, int c0, int n, float pad) {
+    typedef T TV8 __attribute__((ext_vector_type(8)));
+    TV8 v;
+    if (VEC) {   // n % 8 == 0 and rows 16-byte aligned: a group of 8 is all real or all padding
         if (c0 < n) {
-            const TV4 v = *reinterpret_cast<const TV4*>(row + c0);
-#pragma unroll
-            for (int i = 0; i < 4; i++) x[i] = (float)v[i];
+            v = *reinterpret_cast<const TV8*>(row + c0);
         } else {
 #pragma unroll
-            for (int i = 0; i < 4; i++) x[i] = pad;
+            for (int i = 0; i < 8; i++) v[i] = (T)pad;
         }
     } else {
 #pragma unroll
-        for (int i = 0; i < 4; i++) x[i] = (c0 + i < n) ? (float)row[c0 + i] : pad;
+        for (int i = 0; i < 8; i++) v[i] = (c0 + i < n) ? row[c0 + i] : (T)pad;
     }
+    return v;
 }
 
 // NT = compile-time bound on the 16-key tiles of a unit (N <= 16 NT); the workgroup has
 // ceil(N / 16) wavefronts.
-template <int DT, bool HAS_BIAS, int MASK_DT, int NT, bool VEC>
+// MASKED: this launch handles the units whose window mask is live; the other units (or all, when
+// there is no mask) go through the MASKED = false instantiation.
+template <int DT, bool HAS_BIAS, int MASK_DT, int NT, bool VEC, bool MASKED>
 __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p) {
     typedef typename Elem<DT>::E E;
     typedef typename Elem<DT>::V8 V8;
@@ -72,6 +78,11 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
 
     __shared__ __attribute__((aligned(16))) SE lds_K[2][ROWS * S];
     __shared__ __attribute__((aligned(16))) E lds_V[2][ROWS * S];
+    __shared__ __attribute__((aligned(16))) E lds_rawK[ROWS * 32];   // landing area: unpadded 64-byte rows
+    __shared__ __attribute__((aligned(16))) E lds_rawV[ROWS * 32];
+    __shared__ uint8_t lds_live[kLiveCache];       // copy of the per-window mask flags
+    __shared__ uint16_t lds_list[kLiveCache];      // windows of this launch's class, ascending
+    __shared__ int lds_count;
 
     const int N = p.n;
     const int tid = threadIdx.x;
@@ -97,12 +108,18 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
         st8<SV8>(&lds_K[0][0] + i * 8, zero8<SV8>());
         st8<V8>(&lds_V[0][0] + i * 8, zero8<V8>());
     }
+    for (int i = tid; i < ROWS * 32 / 8; i += nthreads) {
+        st8<V8>(lds_rawK + i * 8, zero8<V8>());
+        st8<V8>(lds_rawV + i * 8, zero8<V8>());
+    }
 
     const int qi = wave * 16 + l16;
     const bool qv = qi < N;
     const int qc = min(qi, N - 1);
 
-    // ---- resident bias: acc0[kt][i] <-> key 16 kt + 4 g + i of query qi, log2 domain ----
+    // ---- resident bias, log2 domain.  Keys are taken 32 at a time; of such a group this lane holds
+    // keys 8g .. 8g+7: acc0[2kp][i] <-> key 32kp + 8g + i, acc0[2kp+1][i] <-> key 32kp + 8g + 4 + i
+    // (so bias and mask rows are read 8 consecutive entries at a time) ----
     f32x4 acc0[NT];
     float mb = 0.f, mn = 0.f;
     if (HAS_BIAS) {
@@ -110,15 +127,14 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
         mb = -INFINITY;
         mn = INFINITY;
 #pragma unroll
-        for (int kt = 0; kt < NT; kt++) {
-            float x[4];
-            load_side4<VEC, E>(brow, 16 * kt + 4 * g, N, -INFINITY, x);
+        for (int kp = 0; kp < NT / 2; kp++) {
+            const auto raw = load_raw8<VEC, E>(brow, 32 * kp + 8 * g, N, -INFINITY);
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const float v = x[i] * kLog2e;      // -inf stays -inf
-                acc0[kt][i] = v;
+            for (int j = 0; j < 8; j++) {
+                const float v = (float)raw[j] * kLog2e;      // -inf stays -inf
+                acc0[2 * kp + (j >> 2)][j & 3] = v;
                 mb = fmaxf(mb, v);
-                mn = fminf(mn, (16 * kt + 4 * g + i < N) ? v : INFINITY);
+                mn = fminf(mn, (32 * kp + 8 * g + j < N) ? v : INFINITY);
             }
         }
         mb = col_max(mb);
@@ -128,7 +144,8 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
 #pragma unroll
         for (int kt = 0; kt < NT; kt++)
 #pragma unroll
-            for (int i = 0; i < 4; i++) acc0[kt][i] = (16 * kt + 4 * g + i < N) ? 0.f : -INFINITY;
+            for (int i = 0; i < 4; i++)
+                acc0[kt][i] = (32 * (kt >> 1) + 8 * g + 4 * (kt & 1) + i < N) ? 0.f : -INFINITY;
     }
     const float m_fixed = mb + scale2;     // upper bound of every logit of this row (mask <= 0)
 #pragma unroll
@@ -141,18 +158,69 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
     for (int off = 8; off >= 1; off >>= 1) range = fmaxf(range, __shfl_xor(range, off));
     const bool wave_fast = (DT == FWA2_BF16) && (2.f * scale2 + range <= kGapLimit);
 
-    // ---- per-unit fetch (into registers) and staging (registers -> LDS) ----
-    const int srow = tid >> 2;             // staged row of this thread (< 16 * waves <= ROWS)
-    const int sc8 = (tid & 3) * 8;
-    auto fetch = [&](int b, V8& kk, V8& vv, V8& qq) __attribute__((always_inline)) {
-        kk = zero8<V8>(); vv = zero8<V8>(); qq = zero8<V8>();
-        if (srow < N) {
-            kk = ld8<V8>(reinterpret_cast<const E*>(p.k.ptr) + b * p.k.sb + h * p.k.sh + (int64_t)srow * p.k.sn + sc8);
-            vv = ld8<V8>(reinterpret_cast<const E*>(p.v.ptr) + b * p.v.sb + h * p.v.sh + (int64_t)srow * p.v.sn + sc8);
+    // ---- which units belong to this launch.  With cached flags the windows of this launch's class
+    // (mask live or not) are listed once, and the units are dealt out by their rank within the
+    // class, so every workgroup of the head gets the same number of them whatever the pattern of
+    // masked windows. ----
+    const bool listed = MASK_DT >= 0 && p.mask_live && p.n_windows <= kLiveCache;
+    if (listed) {
+        for (int i = tid; i < p.n_windows; i += nthreads) lds_live[i] = p.mask_live[i];
+        __syncthreads();
+        if (wave == 0) {
+            int cnt = 0;
+            for (int base = 0; base < p.n_windows; base += 64) {
+                const int w = base + lane;
+                const bool in = w < p.n_windows && ((lds_live[w] != 0) == MASKED);
+                const unsigned long long bal = __ballot(in);
+                if (in) lds_list[cnt + __popcll(bal & ((1ull << lane) - 1ull))] = (uint16_t)w;
+                cnt += __popcll(bal);
+            }
+            if (lane == 0) lds_count = cnt;
         }
+        __syncthreads();
+    }
+    const int cnt = listed ? lds_count : 0;
+    const int total = listed ? ((p.bw + p.n_windows - 1) / p.n_windows) * cnt : p.bw;   // ranks to deal out
+    auto unit_of = [&](int t) -> int {
+        if (!listed) return t;
+        const int img = t / cnt;
+        // the same for every lane: keep it (and the addresses derived from it) in scalar registers
+        return __builtin_amdgcn_readfirstlane(img * p.n_windows + (int)lds_list[t - img * cnt]);
+    };
+    auto flags_of = [&](int b) -> int {
+        const int w = b % p.n_windows;
+        return __builtin_amdgcn_readfirstlane(listed ? (int)lds_live[w] : (int)p.mask_live[w]);
+    };
+    // first rank >= t (in steps of the group count) that names an existing unit of this launch
+    auto rank_from = [&](int t) -> int {
+        for (; t < total; t += p.groups) {
+            const int b = unit_of(t);
+            if (b >= p.bw) continue;
+            if (listed || MASK_DT < 0 || !p.mask_live || ((flags_of(b) != 0) == MASKED)) return t;
+        }
+        return total;
+    };
+    // ---- per-unit fetch: every wavefront brings in the 16 K and V rows it will stage (lane i lands
+    // at 16 i bytes from the wavefront's base) and its own 16 query rows ----
+    const int frow = wave * 16 + (lane >> 2);      // K / V row of this lane
+    const int fc8 = (lane & 3) * 8;
+    auto fetch = [&](int b, V8& qq) __attribute__((always_inline)) {
+        if (frow < N) {
+            const E* kp = reinterpret_cast<const E*>(p.k.ptr) + b * p.k.sb + h * p.k.sh + (int64_t)frow * p.k.sn + fc8;
+            const E* vp = reinterpret_cast<const E*>(p.v.ptr) + b * p.v.sb + h * p.v.sh + (int64_t)frow * p.v.sn + fc8;
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)kp,
+                                             (__attribute__((address_space(3))) void*)(lds_rawK + wave * 16 * 32), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)vp,
+                                             (__attribute__((address_space(3))) void*)(lds_rawV + wave * 16 * 32), 16, 0, 0);
+        }
+        qq = zero8<V8>();
         if (qv) qq = ld8<V8>(reinterpret_cast<const E*>(p.q.ptr) + b * p.q.sb + h * p.q.sh + (int64_t)qi * p.q.sn + 8 * g);
     };
-    auto stage = [&](int buf, V8 kk, V8 vv) __attribute__((always_inline)) {
+    // landing area -> tiles: K normalised and rounded to fp16, V as is (rows >= n stay zero)
+    auto stage = [&](int buf) __attribute__((always_inline)) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");    // this wavefront's rows have landed
+        const V8 kk = ld8<V8>(lds_rawK + frow * 32 + fc8);
+        const V8 vv = ld8<V8>(lds_rawV + frow * 32 + fc8);
         float x[8];
         unpack8(kk, x);
         float ss = 0.f;
@@ -163,22 +231,24 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
         SV8 kn;
 #pragma unroll
         for (int j = 0; j < 8; j++) kn[j] = (SE)(x[j] * inv);
-        st8<SV8>(&lds_K[buf][srow * S + sc8], kn);
-        st8<V8>(&lds_V[buf][srow * S + sc8], vv);
+        st8<SV8>(&lds_K[buf][frow * S + fc8], kn);
+        st8<V8>(&lds_V[buf][frow * S + fc8], vv);
     };
 
-    int b = grp;
-    V8 kk, vv, qq;
     __syncthreads();                       // zero fill done
-    if (b < p.bw) {
-        fetch(b, kk, vv, qq);
-        stage(0, kk, vv);
+    int t = rank_from(grp);
+    V8 qq = zero8<V8>();
+    if (t < total) {
+        fetch(unit_of(t), qq);
+        stage(0);
     }
     __syncthreads();
     int cur = 0;
 
-    while (b < p.bw) {
-        const int bn = b + p.groups;
+    while (t < total) {
+        const int b = unit_of(t);
+        const int tn = rank_from(t + p.groups);
+        const int bn = tn < total ? unit_of(tn) : p.bw;
         // ---- Q operand: normalise, fold s log2e, round to fp16 ----
         SV8 bq;
         {
@@ -192,15 +262,14 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
 #pragma unroll
             for (int j = 0; j < 8; j++) bq[j] = (SE)(x[j] * sc);
         }
-        if (bn < p.bw) fetch(bn, kk, vv, qq);      // in flight while this unit is computed
+        if (bn < p.bw) fetch(bn, qq);      // in flight while this unit is computed
 
         const ME* mrow = nullptr;
-        bool masked = false, safe = false;
-        if (MASK_DT >= 0) {
+        constexpr bool masked = MASKED;
+        bool safe = false;
+        if (MASKED) {
             const int w = b % p.n_windows;
-            const int fl = p.mask_live ? p.mask_live[w] : 1;
-            masked = fl != 0;
-            safe = (fl & 2) != 0;
+            safe = p.mask_live ? (flags_of(b) & 2) != 0 : false;
             mrow = reinterpret_cast<const ME*>(p.mask) + w * p.mask_sw + (int64_t)qc * p.mask_sn;
         }
 
@@ -215,20 +284,20 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
         float m_run = 0.f;     // online path: running maximum relative to m_fixed
         bool fast_unit = false;
 
-        // scores of keys 32 kp .. 32 kp + 31 (tile A: rows 4g+i, tile B: rows 16+4g+i)
-        auto scores = [&](int kp, bool with_mask, f32x4& s0, f32x4& s1) __attribute__((always_inline)) {
-            const SV8 a0 = ld8<SV8>(Kb + (32 * kp + l16) * S + 8 * g);
-            const SV8 a1 = ld8<SV8>(Kb + (32 * kp + 16 + l16) * S + 8 * g);
+        typedef ME MV8 __attribute__((ext_vector_type(8)));
+        // scores of keys 32 kp .. 32 kp + 31: MFMA tile A holds keys 8r/4 + r%4 in its rows r, tile B
+        // the keys 4 further on, so that this lane's 8 values are keys 8g .. 8g+7 of the group
+        auto scores = [&](int kp, bool with_mask, const MV8& mk, f32x4& s0, f32x4& s1) __attribute__((always_inline)) {
+            const int krow = 32 * kp + 8 * (l16 >> 2) + (l16 & 3);
+            const SV8 a0 = ld8<SV8>(Kb + krow * S + 8 * g);
+            const SV8 a1 = ld8<SV8>(Kb + (krow + 4) * S + 8 * g);
             s0 = Elem<kScoreDT>::mfma16(a0, bq, acc0[2 * kp]);
             s1 = Elem<kScoreDT>::mfma16(a1, bq, acc0[2 * kp + 1]);
             if (MASK_DT >= 0 && with_mask) {
-                float x0[4], x1[4];
-                load_side4<VEC, ME>(mrow, 32 * kp + 4 * g, N, 0.f, x0);
-                load_side4<VEC, ME>(mrow, 32 * kp + 16 + 4 * g, N, 0.f, x1);
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
-                    s0[i] = fmaf(x0[i], kLog2e, s0[i]);
-                    s1[i] = fmaf(x1[i], kLog2e, s1[i]);
+                    s0[i] = fmaf((float)mk[i], kLog2e, s0[i]);
+                    s1[i] = fmaf((float)mk[4 + i], kLog2e, s1[i]);
                 }
             }
         };
@@ -248,8 +317,8 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
             if (sum_by_mfma) lacc = Elem<DT>::mfma16(ones, bp, lacc);
 #pragma unroll
             for (int dt = 0; dt < 2; dt++) {
-                const E* vlo = Vb + (32 * kp + 4 * g + (l16 >> 2)) * S + 16 * dt + 4 * (l16 & 3);
-                const V8 av = lds_tr8<DT>(vlo, vlo + 16 * S);
+                const E* vlo = Vb + (32 * kp + 8 * g + (l16 >> 2)) * S + 16 * dt + 4 * (l16 & 3);
+                const V8 av = lds_tr8<DT>(vlo, vlo + 4 * S);
                 oacc[dt] = Elem<DT>::mfma16(av, bp, oacc[dt]);
             }
         };
@@ -257,11 +326,19 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
         if (wave_fast && (!masked || safe)) {
             fast_unit = true;
             auto body = [&](bool with_mask) __attribute__((always_inline)) {
+                // mask rows travel two key groups ahead of their use
+                MV8 mq[2];
+                if (MASK_DT >= 0 && with_mask) {
+                    mq[0] = load_raw8<VEC, ME>(mrow, 8 * g, N, 0.f);
+                    mq[1] = load_raw8<VEC, ME>(mrow, 32 + 8 * g, N, 0.f);
+                }
 #pragma unroll
                 for (int kp = 0; kp < NT / 2; kp++) {
                     if (32 * kp < N) {
                         f32x4 s0, s1;
-                        scores(kp, with_mask, s0, s1);
+                        scores(kp, with_mask, mq[kp & 1], s0, s1);
+                        if (MASK_DT >= 0 && with_mask && kp + 2 < NT / 2)
+                            mq[kp & 1] = load_raw8<VEC, ME>(mrow, 32 * (kp + 2) + 8 * g, N, 0.f);
 #pragma unroll
                         for (int i = 0; i < 4; i++) {
                             s0[i] = fast_exp2(s0[i]);
@@ -271,14 +348,16 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
                     }
                 }
             };
-            if (masked) body(true); else body(false);
+            body(MASKED);
         } else {
             m_run = -INFINITY;
 #pragma unroll
             for (int kp = 0; kp < NT / 2; kp++) {
                 if (32 * kp < N) {
                     f32x4 s0, s1;
-                    scores(kp, masked, s0, s1);
+                    MV8 mk;
+                    if (MASK_DT >= 0 && masked) mk = load_raw8<VEC, ME>(mrow, 32 * kp + 8 * g, N, 0.f);
+                    scores(kp, masked, mk, s0, s1);
                     float bm = fmaxf(fmaxf(s0[0], s0[1]), fmaxf(s0[2], s0[3]));
                     bm = fmaxf(bm, fmaxf(fmaxf(s1[0], s1[1]), fmaxf(s1[2], s1[3])));
                     bm = col_max(bm);
@@ -303,6 +382,7 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
             }
         }
 
+        if (bn < p.bw) stage(cur ^ 1);     // before the stores below, so the wait covers only the fetch
         // ---- normalise, write o (input dtype) and lse (natural log, fp32) ----
         const float l_tot = fast_unit ? lacc[0] : col_add(l_run);
         const float inv_l = l_tot > 0.f ? 1.0f / l_tot : 0.f;
@@ -321,32 +401,46 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
             }
         }
 
-        if (bn < p.bw) stage(cur ^ 1, kk, vv);
         __syncthreads();       // next unit staged; everybody is done with the current buffers
         cur ^= 1;
-        b = bn;
+        t = tn;
     }
 }
 
 // ---- host side -----------------------------------------------------------------
 int forward_resident_supported(int n) { return n >= 1 && n <= 256; }
 
+template <class K>
+static int resident_fit(K kern, int threads) {
+    int n = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kern, threads, 0) != hipSuccess || n < 1) n = 1;
+    return n;
+}
+
 template <int DT, bool HAS_BIAS, int MASK_DT, int NT, bool VEC>
 static hipError_t launch_nt(FwdParams p, hipStream_t st) {
     const int waves = (p.n + 15) / 16;
-    static const int fit = [&] {
-        int n = 0;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, fwd_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC>,
-                                                         64 * NT, 0) != hipSuccess || n < 1)
-            n = 1;
-        return n;
-    }();
     // the runtime's figure is for full 64 NT-thread groups; smaller groups only fit better
-    int groups = (p.cus * fit) / p.heads;
-    if (groups < 1) groups = 1;
-    if (groups > p.bw) groups = p.bw;
-    p.groups = groups;
-    hipLaunchKernelGGL((fwd_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC>), dim3(p.heads * groups), dim3(64 * waves), 0, st, p);
+    static const int fit_plain = resident_fit(fwd_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, false>, 64 * NT);
+    static const int fit_masked = MASK_DT >= 0 ? resident_fit(fwd_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, true>, 64 * NT) : 1;
+    auto groups_for = [&](int fit) {
+        int groups = (p.cus * fit) / p.heads;
+        if (groups < 1) groups = 1;
+        if (groups > p.bw) groups = p.bw;
+        return groups;
+    };
+    // units with an all-zero mask (or every unit when there is no mask) ...
+    if (MASK_DT < 0 || p.mask_live != nullptr) {
+        p.groups = groups_for(fit_plain);
+        hipLaunchKernelGGL((fwd_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, false>), dim3(p.heads * p.groups),
+                           dim3(64 * waves), 0, st, p);
+    }
+    // ... and the units whose mask is live
+    if (MASK_DT >= 0) {
+        p.groups = groups_for(fit_masked);
+        hipLaunchKernelGGL((fwd_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, true>), dim3(p.heads * p.groups),
+                           dim3(64 * waves), 0, st, p);
+    }
     return hipGetLastError();
 }
 
