@@ -325,7 +325,10 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
                 st8<V8>(L.Qs + r * kRow + dc, qn);
                 st8<V8>(L.Ks + r * kRow + dc, kn);
                 st8<V8>(L.dOs + r * kRow + dc, do8);
-                if ((tid & 3) == 0) L.ndelta[r] = -dl;
+                if ((tid & 3) == 0) {
+                    L.ndelta[r] = -dl;
+                    if (r < N) p.delta[((int64_t)b * p.heads + h) * p.delta_stride + r] = dl;   // for the dq kernel
+                }
                 if ((tid & 3) == 1) {
                     float l2 = -INFINITY;          // padded / fully masked rows: P = 0
                     if (r < N) { const float l = L.rawLse[r]; l2 = (l == -INFINITY) ? -INFINITY : -l * kLog2e; }
@@ -479,10 +482,13 @@ int backward_supported(int n) { return n >= 1 && n <= 256; }
 
 void dq_geometry(int n, int* waves, int* chunks);
 hipError_t launch_backward_dq(const BwdParams& p, int dtype, bool has_bias, int mask_dt, hipStream_t st);
+int backward_dq_resident_supported(int n);
+hipError_t launch_backward_dq_resident(const BwdParams& p, int dtype, bool has_bias, int mask_dt, hipStream_t st,
+                                       int max_groups, int* ds_parts_out);
 
 struct BwdPlan {
-    int waves, groups, npk, r, nqb_t, kt, dq_waves, dq_chunks, ds_parts;
-    size_t off_dbias, off_dscale, off_bias_t, off_mask_t, total;
+    int waves, groups, npk, r, nqb_t, kt, dq_waves, dq_chunks, ds_parts, dq_max_groups;
+    size_t off_dbias, off_dscale, off_bias_t, off_mask_t, off_delta, total;
     size_t smem;
 };
 
@@ -506,8 +512,14 @@ static BwdPlan make_plan(int heads, int n, int bw, bool has_bias, bool has_mask,
     if (has_bias) off += align256((size_t)heads * 2 * groups * pl.npk * pl.r * 4);
     dq_geometry(n, &pl.dq_waves, &pl.dq_chunks);
     pl.ds_parts = bw * pl.dq_chunks;
+    // the resident dq kernel writes one partial per workgroup: at most this many per head and launch
+    pl.dq_max_groups = (cus * 8) / heads + 1;
+    if (pl.dq_max_groups > bw) pl.dq_max_groups = bw;
+    const int ds_slots = pl.ds_parts > 2 * pl.dq_max_groups ? pl.ds_parts : 2 * pl.dq_max_groups;
     pl.off_dscale = off;
-    off += align256((size_t)heads * pl.ds_parts * 4);
+    off += align256((size_t)heads * ds_slots * 4);
+    pl.off_delta = off;
+    off += align256((size_t)bw * heads * pl.r * 4);
     pl.off_bias_t = off;
     if (has_bias) off += align256((size_t)heads * pl.npk * pl.r * 2);
     pl.off_mask_t = off;
@@ -584,6 +596,8 @@ static hipError_t launch_bwd_dt(BwdParams p, bool has_bias, int mask_dt, hipStre
     p.part_dscale = reinterpret_cast<float*>(ws + pl.off_dscale);
     p.bias_t = ws + pl.off_bias_t;
     p.mask_t = ws + pl.off_mask_t;
+    p.delta = reinterpret_cast<float*>(ws + pl.off_delta);
+    p.delta_stride = pl.r;
     const dim3 tgrid(pl.r / 32, (pl.npk + 31) / 32, 1);
     if (has_bias) {
         dim3 gr(tgrid.x, tgrid.y, p.heads);
@@ -617,7 +631,13 @@ static hipError_t launch_bwd_dt(BwdParams p, bool has_bias, int mask_dt, hipStre
     if (e != hipSuccess) return e;
     p.groups = gr_out[0];
     p.db_parts = gr_out[1];
-    e = launch_backward_dq(p, DT, has_bias, mask_dt, st);
+    if (backward_dq_resident_supported(p.n)) {
+        int parts = 0;
+        e = launch_backward_dq_resident(p, DT, has_bias, mask_dt, st, pl.dq_max_groups, &parts);
+        p.ds_parts = parts;
+    } else {
+        e = launch_backward_dq(p, DT, has_bias, mask_dt, st);
+    }
     if (e != hipSuccess) return e;
     if (has_bias || p.scale_kind == FWA2_SCALE_TENSOR) {
         dim3 gr(has_bias ? pl.r / 32 : 1, has_bias ? (pl.npk + 7) / 8 : 1, p.heads);

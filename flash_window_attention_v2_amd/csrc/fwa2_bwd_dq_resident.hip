@@ -1,0 +1,442 @@
+// Backward, query side, for windows of up to 256 tokens: dq and the per-row
+// terms of dlogit_scale from persistent workgroups that keep the bias tile
+// resident in registers (longer windows use the streaming kernel in
+// fwa2_bwd_dq.hip).
+//
+// Replaces the dq half of _bwd_kernel
+// (flash_win_attn_v2/kernels/attn_kernel_backward.py:84-564; the reference adds
+// every key block's dq contribution into an fp32 buffer with atomics, :314).
+//
+// Same skeleton as the resident forward kernel: a workgroup belongs to one
+// head, every wavefront owns 16 query rows and holds bias[h] * log2e - m for
+// them in the register layout of the score accumulators (m = the row's logit
+// bound s log2e + max bias2), K_hat (fp16) and V of the next unit land in LDS by
+// DMA while the current unit is computed.  Per 32 keys:
+//   S^T - m   = K_hat Q_hat^T        (fp16 MFMA, C operand = resident bias)
+//   dP^T      = V dO^T               (input dtype MFMA, C operand = -delta)
+//   dZ^T      = 2^(S^T - lse2) (dP^T - delta), rounded to fp16
+//   dQ_hat^T += K_hat^T dZ^T         (fp16 MFMA, K_hat^T by transposing LDS reads)
+// When the row bound is tight (bf16, moderate scale, masks that only remove
+// keys) the factor w = 2^(m - lse2) is folded into dO and delta once per row,
+// so that dZ^T = 2^acc * acc' costs one exp and one multiply per score.
+// delta = rowsum(o * dO) is read from the buffer the key-side kernel wrote.
+#include "fwa2_common.hpp"
+
+namespace fwa2 {
+
+template <int DT, bool HAS_BIAS, int MASK_DT, int NT, bool VEC, bool MASKED>
+__global__ void __launch_bounds__(64 * NT) bwd_dq_resident_kernel(const BwdParams p) {
+    typedef typename Elem<DT>::E E;
+    typedef typename Elem<DT>::V8 V8;
+    typedef typename Elem<DT>::V4 V4;
+    typedef typename MaskElem<DT, MASK_DT>::E ME;
+    typedef typename Elem<kScoreDT>::E SE;
+    typedef typename Elem<kScoreDT>::V8 SV8;
+    typedef ME MV8 __attribute__((ext_vector_type(8)));
+    constexpr int ROWS = 16 * NT;
+    constexpr int S = kLdsStride;
+
+    __shared__ __attribute__((aligned(16))) SE lds_K[2][ROWS * S];
+    __shared__ __attribute__((aligned(16))) E lds_V[2][ROWS * S];
+    __shared__ __attribute__((aligned(16))) E lds_rawK[ROWS * 32];   // landing area: unpadded 64-byte rows
+    __shared__ __attribute__((aligned(16))) E lds_rawV[ROWS * 32];
+    __shared__ __attribute__((aligned(16))) E lds_rawQ[ROWS * 32];   // this wavefront's 16 query rows
+    __shared__ __attribute__((aligned(16))) E lds_rawDO[ROWS * 32];
+    __shared__ uint8_t lds_live[kLiveCache];
+    __shared__ uint16_t lds_list[kLiveCache];
+    __shared__ int lds_count;
+    __shared__ float lds_red[NT];
+
+    const int N = p.n;
+    const int tid = threadIdx.x;
+    const int nthreads = blockDim.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int l16 = lane & 15;
+    const int g = lane >> 4;
+
+    const int groups = p.dq_groups;
+    const int h = blockIdx.x / groups;
+    const int grp = blockIdx.x - h * groups;
+
+    float s_true;
+    if (p.scale_kind == FWA2_SCALE_TENSOR) {
+        const float ls = (float)reinterpret_cast<const E*>(p.logit_scale)[h];
+        s_true = expf(fminf(ls, kLn100));
+    } else {
+        s_true = p.default_scale;
+    }
+    const float scale2 = s_true * kLog2e;
+
+    for (int i = tid; i < 2 * ROWS * S / 8; i += nthreads) {
+        st8<SV8>(&lds_K[0][0] + i * 8, zero8<SV8>());
+        st8<V8>(&lds_V[0][0] + i * 8, zero8<V8>());
+    }
+    for (int i = tid; i < ROWS * 32 / 8; i += nthreads) {
+        st8<V8>(lds_rawK + i * 8, zero8<V8>());
+        st8<V8>(lds_rawV + i * 8, zero8<V8>());
+        st8<V8>(lds_rawQ + i * 8, zero8<V8>());
+        st8<V8>(lds_rawDO + i * 8, zero8<V8>());
+    }
+
+    const int qi = wave * 16 + l16;
+    const bool qv = qi < N;
+    const int qc = min(qi, N - 1);
+
+    // ---- resident bias (see fwa2_fwd_resident.hip): acc0[2kp][i] <-> key 32kp + 8g + i,
+    // acc0[2kp+1][i] <-> key 32kp + 8g + 4 + i, log2 domain, minus the row bound ----
+    f32x4 acc0[NT];
+    float mb = 0.f, mn = 0.f;
+    if (HAS_BIAS) {
+        const E* brow = reinterpret_cast<const E*>(p.bias) + h * p.bias_sh + (int64_t)qc * p.bias_sn;
+        mb = -INFINITY;
+        mn = INFINITY;
+#pragma unroll
+        for (int kp = 0; kp < NT / 2; kp++) {
+            const auto raw = load_raw8<VEC, E>(brow, 32 * kp + 8 * g, N, -INFINITY);
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const float v = (float)raw[j] * kLog2e;
+                acc0[2 * kp + (j >> 2)][j & 3] = v;
+                mb = fmaxf(mb, v);
+                mn = fminf(mn, (32 * kp + 8 * g + j < N) ? v : INFINITY);
+            }
+        }
+        mb = col_max(mb);
+        mn = -col_max(-mn);
+        if (!(mb > -INFINITY)) { mb = 0.f; mn = 0.f; }
+    } else {
+#pragma unroll
+        for (int kt = 0; kt < NT; kt++)
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                acc0[kt][i] = (32 * (kt >> 1) + 8 * g + 4 * (kt & 1) + i < N) ? 0.f : -INFINITY;
+    }
+    const float m_fixed = mb + scale2;
+#pragma unroll
+    for (int kt = 0; kt < NT; kt++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) acc0[kt][i] -= m_fixed;
+    float range = (mb - mn == mb - mn) ? mb - mn : INFINITY;
+#pragma unroll
+    for (int off = 8; off >= 1; off >>= 1) range = fmaxf(range, __shfl_xor(range, off));
+    // w = 2^(m - lse2) may be folded into dO when it cannot leave the bf16 range
+    const bool wave_fold = (DT == FWA2_BF16) && (2.f * scale2 + range <= kGapLimit);
+
+    // ---- units of this launch, dealt out by rank within their mask class ----
+    const bool listed = MASK_DT >= 0 && p.mask_live && p.n_windows <= kLiveCache;
+    if (listed) {
+        for (int i = tid; i < p.n_windows; i += nthreads) lds_live[i] = p.mask_live[i];
+        __syncthreads();
+        if (wave == 0) {
+            int cnt = 0;
+            for (int base = 0; base < p.n_windows; base += 64) {
+                const int w = base + lane;
+                const bool in = w < p.n_windows && ((lds_live[w] != 0) == MASKED);
+                const unsigned long long bal = __ballot(in);
+                if (in) lds_list[cnt + __popcll(bal & ((1ull << lane) - 1ull))] = (uint16_t)w;
+                cnt += __popcll(bal);
+            }
+            if (lane == 0) lds_count = cnt;
+        }
+        __syncthreads();
+    }
+    const int cnt = listed ? lds_count : 0;
+    const int total = listed ? ((p.bw + p.n_windows - 1) / p.n_windows) * cnt : p.bw;
+    auto unit_of = [&](int t) -> int {
+        if (!listed) return t;
+        const int img = t / cnt;
+        return __builtin_amdgcn_readfirstlane(img * p.n_windows + (int)lds_list[t - img * cnt]);
+    };
+    auto flags_of = [&](int b) -> int {
+        const int w = b % p.n_windows;
+        return __builtin_amdgcn_readfirstlane(listed ? (int)lds_live[w] : (int)p.mask_live[w]);
+    };
+    auto rank_from = [&](int t) -> int {
+        for (; t < total; t += groups) {
+            const int b = unit_of(t);
+            if (b >= p.bw) continue;
+            if (listed || MASK_DT < 0 || !p.mask_live || ((flags_of(b) != 0) == MASKED)) return t;
+        }
+        return total;
+    };
+
+    // ---- per-unit fetch: K / V rows by DMA, this lane's share of its query row in registers ----
+    const int frow = wave * 16 + (lane >> 2);
+    const int fc8 = (lane & 3) * 8;
+    struct Row { float lse, delta; };
+    auto dma16 = [&](const E* src, E* lds_wave_base) __attribute__((always_inline)) {
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                         (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
+    };
+    auto fetch = [&](int b, Row& r) __attribute__((always_inline)) {
+        // lane-derived offsets are re-materialised here: hoisted out of the unit loop they would occupy
+        // a dozen registers for the whole kernel
+        int ln = lane;
+        asm volatile("" : "+v"(ln));
+        const int frow = wave * 16 + (ln >> 2);
+        const int fc8 = (ln & 3) * 8;
+        const int qi = wave * 16 + (ln & 15);
+        const bool qv = qi < N;
+        if (frow < N) {   // rows wave*16 .. +15 of k, v (to be staged by this wavefront) and of q, dO (its own queries)
+            dma16(reinterpret_cast<const E*>(p.k.ptr) + b * p.k.sb + h * p.k.sh + (int64_t)frow * p.k.sn + fc8,
+                  lds_rawK + wave * 16 * 32);
+            dma16(reinterpret_cast<const E*>(p.v.ptr) + b * p.v.sb + h * p.v.sh + (int64_t)frow * p.v.sn + fc8,
+                  lds_rawV + wave * 16 * 32);
+            dma16(reinterpret_cast<const E*>(p.q.ptr) + b * p.q.sb + h * p.q.sh + (int64_t)frow * p.q.sn + fc8,
+                  lds_rawQ + wave * 16 * 32);
+            dma16(reinterpret_cast<const E*>(p.d_o.ptr) + b * p.d_o.sb + h * p.d_o.sh + (int64_t)frow * p.d_o.sn + fc8,
+                  lds_rawDO + wave * 16 * 32);
+        }
+        r.lse = -INFINITY; r.delta = 0.f;
+        if (qv) {
+            r.lse = p.lse[b * p.lse_sb + h * p.lse_sh + qi];
+            r.delta = p.delta[((int64_t)b * p.heads + h) * p.delta_stride + qi];
+        }
+    };
+    auto stage = [&](int buf) __attribute__((always_inline)) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        const V8 kk = ld8<V8>(lds_rawK + frow * 32 + fc8);
+        const V8 vv = ld8<V8>(lds_rawV + frow * 32 + fc8);
+        float x[8];
+        unpack8(kk, x);
+        float ss = 0.f;
+#pragma unroll
+        for (int j = 0; j < 8; j++) ss += x[j] * x[j];
+        ss = quad_add(ss);
+        const float inv = inv_norm(ss);
+        SV8 kn;
+#pragma unroll
+        for (int j = 0; j < 8; j++) kn[j] = (SE)(x[j] * inv);
+        st8<SV8>(&lds_K[buf][frow * S + fc8], kn);
+        st8<V8>(&lds_V[buf][frow * S + fc8], vv);
+    };
+
+    __syncthreads();
+    int t = rank_from(grp);
+    Row row;
+    row.lse = -INFINITY; row.delta = 0.f;
+    if (t < total) {
+        fetch(unit_of(t), row);
+        stage(0);
+    }
+    __syncthreads();
+    int cur = 0;
+    float ds_acc = 0.f;        // sum over this lane's queries of q_hat . dq_hat
+
+    while (t < total) {
+        const int b = unit_of(t);
+        const int tn = rank_from(t + groups);
+        const int bn = tn < total ? unit_of(tn) : p.bw;
+
+        const ME* mrow = nullptr;
+        bool safe = false;
+        if (MASKED) {
+            const int w = b % p.n_windows;
+            safe = p.mask_live ? (flags_of(b) & 2) != 0 : false;
+            mrow = reinterpret_cast<const ME*>(p.mask) + w * p.mask_sw + (int64_t)qc * p.mask_sn;
+        }
+        const bool fold = wave_fold && (!MASKED || safe);
+
+        // ---- this unit's operands out of the prefetched row ----
+        SV8 bq;
+        V8 bd;
+        float nl, nd, inv, nrm;
+        {
+            // the rows landed before the previous unit's barrier (the first unit's before the one above)
+            const V8 qcur = ld8<V8>(lds_rawQ + (wave * 16 + l16) * 32 + 8 * g);
+            const V8 docur = ld8<V8>(lds_rawDO + (wave * 16 + l16) * 32 + 8 * g);
+            float x[8];
+            unpack8(qcur, x);
+            float ss = 0.f;
+#pragma unroll
+            for (int j = 0; j < 8; j++) ss += x[j] * x[j];
+            ss = col_add(ss);
+            nrm = sqrtf(ss);
+            inv = 1.0f / fmaxf(nrm, kNormEps);
+            const float sc = scale2 * inv;
+#pragma unroll
+            for (int j = 0; j < 8; j++) bq[j] = (SE)(x[j] * sc);
+            nl = (row.lse == -INFINITY) ? -INFINITY : m_fixed - row.lse * kLog2e;   // fully masked row: P = 0
+            if (fold) {
+                const float w = fast_exp2(nl);
+#pragma unroll
+                for (int j = 0; j < 8; j++) bd[j] = (E)((float)docur[j] * w);
+                nd = -row.delta * w;
+                nl = 0.f;
+            } else {
+                bd = docur;
+                nd = -row.delta;
+            }
+        }
+        if (bn < p.bw) fetch(bn, row);      // in flight while this unit is computed
+
+        const SE* Kb = &lds_K[cur][0];
+        const E* Vb = &lds_V[cur][0];
+        f32x4 dqacc[2], ndv;
+#pragma unroll
+        for (int i = 0; i < 4; i++) { dqacc[0][i] = 0.f; dqacc[1][i] = 0.f; ndv[i] = nd; }
+
+        auto group = [&](int kp, bool with_mask, bool folded, const MV8& mk) __attribute__((always_inline)) {
+            const int krow = 32 * kp + 8 * (l16 >> 2) + (l16 & 3);
+            SV8 bz;
+#pragma unroll
+            for (int half = 0; half < 2; half++) {
+                const SV8 ak = ld8<SV8>(Kb + (krow + 4 * half) * S + 8 * g);
+                const V8 av = ld8<V8>(Vb + (krow + 4 * half) * S + 8 * g);
+                f32x4 s = Elem<kScoreDT>::mfma16(ak, bq, acc0[2 * kp + half]);
+                const f32x4 dp = Elem<DT>::mfma16(av, bd, ndv);
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    if (MASK_DT >= 0 && with_mask) s[i] = fmaf((float)mk[4 * half + i], kLog2e, s[i]);
+                    const float e = folded ? fast_exp2(s[i]) : fast_exp2(s[i] + nl);
+                    bz[4 * half + i] = (SE)(e * dp[i]);
+                }
+            }
+#pragma unroll
+            for (int dt = 0; dt < 2; dt++) {
+                // A row m <-> d = 8 (m / 4) + 4 dt + m % 4, so that this lane's accumulators hold d = 8g + 4dt + i
+                const SE* klo = Kb + (32 * kp + 8 * g + (l16 >> 2)) * S + 8 * (l16 & 3) + 4 * dt;
+                const SV8 akt = lds_tr8<kScoreDT>(klo, klo + 4 * S);
+                dqacc[dt] = Elem<kScoreDT>::mfma16(akt, bz, dqacc[dt]);
+            }
+        };
+        auto body = [&](bool folded) __attribute__((always_inline)) {
+            MV8 mq[2];
+            if (MASKED) {
+                mq[0] = load_raw8<VEC, ME>(mrow, 8 * g, N, 0.f);
+                mq[1] = load_raw8<VEC, ME>(mrow, 32 + 8 * g, N, 0.f);
+            }
+#pragma unroll
+            for (int kp = 0; kp < NT / 2; kp++) {
+                if (32 * kp < N) {
+                    group(kp, MASKED, folded, mq[kp & 1]);
+                    __builtin_amdgcn_sched_barrier(0);   // keep the groups apart: their temporaries must not pile up
+                    if (MASKED && kp + 2 < NT / 2) mq[kp & 1] = load_raw8<VEC, ME>(mrow, 32 * (kp + 2) + 8 * g, N, 0.f);
+                }
+            }
+        };
+        if (fold) body(true); else body(false);
+
+        if (bn < p.bw) stage(cur ^ 1);     // before the stores below, so the wait covers only the fetch
+
+        // ---- back through q / max(|q|, eps); q_hat . dq_hat is this row's share of dlogit_scale ----
+        // q_hat is taken back from the fp16 score operand (q_hat s log2e), which is live anyway
+        float qh[8];
+        float dot = 0.f;
+        const float unscale = 1.0f / scale2;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            qh[j] = (float)bq[j] * unscale;
+            dot += dqacc[j >> 2][j & 3] * qh[j];
+        }
+        dot = col_add(dot);
+        const float proj = nrm > kNormEps ? dot : 0.f;
+        const float f = s_true * inv;
+        int ln2 = lane;
+        asm volatile("" : "+v"(ln2));
+        const int qi2 = wave * 16 + (ln2 & 15);
+        if (qv) {
+            E* dqrow = reinterpret_cast<E*>(const_cast<void*>(p.dq.ptr)) + b * p.dq.sb + h * p.dq.sh + (int64_t)qi2 * p.dq.sn;
+            V8 o8;
+#pragma unroll
+            for (int j = 0; j < 8; j++) o8[j] = (E)(f * (dqacc[j >> 2][j & 3] - qh[j] * proj));
+            st8<V8>(dqrow + 8 * (ln2 >> 4), o8);
+            if (g == 0) ds_acc += dot;
+        }
+
+        __syncthreads();
+        cur ^= 1;
+        t = tn;
+    }
+
+    // ---- dlogit_scale: one partial per workgroup ----
+    if (p.scale_kind == FWA2_SCALE_TENSOR) {
+        const float wsum = wave_sum(ds_acc);
+        if (lane == 0) lds_red[wave] = wsum;
+        __syncthreads();
+        if (tid == 0) {
+            float tot = 0.f;
+            for (int i = 0; i < (nthreads >> 6); i++) tot += lds_red[i];
+            p.part_dscale[(int64_t)h * p.ds_parts + p.ds_slot0 + grp] = tot * s_true;
+        }
+    }
+}
+
+// ---- host side -----------------------------------------------------------------
+int backward_dq_resident_supported(int n) { return n >= 1 && n <= 256; }
+
+template <class K>
+static int resident_fit(K kern, int threads) {
+    int n = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kern, threads, 0) != hipSuccess || n < 1) n = 1;
+    return n;
+}
+
+// Launches the kernel(s) and reports how many dscale partials per head they wrote.
+template <int DT, bool HAS_BIAS, int MASK_DT, int NT, bool VEC>
+static hipError_t launch_nt(BwdParams p, hipStream_t st, int max_groups, int* ds_parts_out) {
+    const int waves = (p.n + 15) / 16;
+    static const int fit_plain = resident_fit(bwd_dq_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, false>, 64 * NT);
+    static const int fit_masked =
+        MASK_DT >= 0 ? resident_fit(bwd_dq_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, true>, 64 * NT) : 1;
+    auto groups_for = [&](int fit) {
+        int groups = (p.cus * fit) / p.heads;
+        if (groups < 1) groups = 1;
+        if (groups > p.bw) groups = p.bw;
+        if (groups > max_groups) groups = max_groups;
+        return groups;
+    };
+    const bool two = MASK_DT >= 0 && p.mask_live != nullptr;
+    const int g_plain = (MASK_DT < 0 || two) ? groups_for(fit_plain) : 0;
+    const int g_masked = MASK_DT >= 0 ? groups_for(fit_masked) : 0;
+    p.ds_parts = g_plain + g_masked;
+    if (g_plain) {
+        p.dq_groups = g_plain;
+        p.ds_slot0 = 0;
+        hipLaunchKernelGGL((bwd_dq_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, false>), dim3(p.heads * g_plain),
+                           dim3(64 * waves), 0, st, p);
+    }
+    if (g_masked) {
+        p.dq_groups = g_masked;
+        p.ds_slot0 = g_plain;
+        hipLaunchKernelGGL((bwd_dq_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, true>), dim3(p.heads * g_masked),
+                           dim3(64 * waves), 0, st, p);
+    }
+    *ds_parts_out = p.ds_parts;
+    return hipGetLastError();
+}
+
+template <int DT, bool HAS_BIAS, int MASK_DT>
+static hipError_t launch_mask(const BwdParams& p, hipStream_t st, int mg, int* out) {
+    const int nt = p.n <= 64 ? 4 : (p.n <= 128 ? 8 : 16);
+    if (p.side_vec) {
+        if (nt == 4) return launch_nt<DT, HAS_BIAS, MASK_DT, 4, true>(p, st, mg, out);
+        if (nt == 8) return launch_nt<DT, HAS_BIAS, MASK_DT, 8, true>(p, st, mg, out);
+        return launch_nt<DT, HAS_BIAS, MASK_DT, 16, true>(p, st, mg, out);
+    }
+    if (nt == 4) return launch_nt<DT, HAS_BIAS, MASK_DT, 4, false>(p, st, mg, out);
+    if (nt == 8) return launch_nt<DT, HAS_BIAS, MASK_DT, 8, false>(p, st, mg, out);
+    return launch_nt<DT, HAS_BIAS, MASK_DT, 16, false>(p, st, mg, out);
+}
+
+template <int DT>
+static hipError_t launch_dt(const BwdParams& p, bool has_bias, int mask_dt, hipStream_t st, int mg, int* out) {
+    if (has_bias) {
+        if (mask_dt < 0) return launch_mask<DT, true, -1>(p, st, mg, out);
+        if (mask_dt == FWA2_F32) return launch_mask<DT, true, FWA2_F32>(p, st, mg, out);
+        return launch_mask<DT, true, DT>(p, st, mg, out);
+    }
+    if (mask_dt < 0) return launch_mask<DT, false, -1>(p, st, mg, out);
+    if (mask_dt == FWA2_F32) return launch_mask<DT, false, FWA2_F32>(p, st, mg, out);
+    return launch_mask<DT, false, DT>(p, st, mg, out);
+}
+
+// max_groups: workgroups per head and launch that the workspace has dscale slots for.
+hipError_t launch_backward_dq_resident(const BwdParams& p, int dtype, bool has_bias, int mask_dt, hipStream_t st,
+                                       int max_groups, int* ds_parts_out) {
+    if (dtype == FWA2_BF16) return launch_dt<FWA2_BF16>(p, has_bias, mask_dt, st, max_groups, ds_parts_out);
+    return launch_dt<FWA2_F16>(p, has_bias, mask_dt, st, max_groups, ds_parts_out);
+}
+
+}  // namespace fwa2

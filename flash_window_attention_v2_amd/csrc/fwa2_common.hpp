@@ -159,6 +159,37 @@ __device__ __forceinline__ float wave_sum(float x) {
     return x;
 }
 
+// ---- helpers of the kernels that keep the bias tile resident in registers ----
+constexpr int kLiveCache = 1024;    // windows whose mask flags are cached in LDS
+constexpr float kGapLimit = 96.f;   // largest tolerated (row bound - largest logit), log2 domain
+
+__device__ __forceinline__ float xor16_max(float x) {
+    u32x2 r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+// reductions over the 4 lanes (g = 0..3) that share a query column
+__device__ __forceinline__ float col_max(float x) { return xor32_max(xor16_max(x)); }
+__device__ __forceinline__ float col_add(float x) { return xor32_add(xor16_add(x)); }
+
+// 8 consecutive entries of a bias / mask row in their storage type; columns >= n read as `pad`.
+template <bool VEC, class T>
+__device__ __forceinline__ auto load_raw8(const T* row, int c0, int n, float pad) {
+    typedef T TV8 __attribute__((ext_vector_type(8)));
+    TV8 v;
+    if (VEC) {   // n % 8 == 0 and rows 16-byte aligned: a group of 8 is all real or all padding
+        if (c0 < n) {
+            v = *reinterpret_cast<const TV8*>(row + c0);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; i++) v[i] = (T)pad;
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; i++) v[i] = (c0 + i < n) ? row[c0 + i] : (T)pad;
+    }
+    return v;
+}
+
 constexpr int kKeyChunk = 256;   // keys staged in LDS at a time by the query-owning kernels
 constexpr int kLdsStride = 40;   // elements per staged row (32 + 8 pad): 80-byte rows
 
@@ -214,7 +245,11 @@ struct BwdParams {
     int db_parts;        // partial tiles per head: groups per launch of the key-side kernel
     int db_slot0;        // first partial slot of the current launch
     float* part_dscale;  // [H, ds_parts] fp32, one per workgroup of the dq kernel
-    int ds_parts;        // bw * dq_chunks
+    int ds_parts;        // partials per head that the reduction sums
+    int ds_slot0;        // first partial slot of the current launch of the resident dq kernel
+    int dq_groups;       // workgroups per head of the current launch of the resident dq kernel
+    float* delta;        // [BW * H, delta_stride] fp32 rowsum(o * dO), written by the key-side kernel
+    int delta_stride;
     int dq_waves;        // wavefronts per workgroup of the dq kernel
     int dq_chunks;       // dq workgroups per (bw, head)
     bool side_vec;       // rows of bias and mask (query-major) may be read with 16-byte loads, n % 8 == 0

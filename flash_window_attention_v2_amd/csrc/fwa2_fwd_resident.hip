@@ -31,36 +31,6 @@
 
 namespace fwa2 {
 
-constexpr int kLiveCache = 1024;    // windows whose mask flags are cached in LDS
-constexpr float kGapLimit = 96.f;   // largest tolerated (row bound - largest logit), log2 domain
-
-__device__ __forceinline__ float xor16_max(float x) {
-    u32x2 r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
-}
-// reductions over the 4 lanes (g = 0..3) that share a query column
-__device__ __forceinline__ float col_max(float x) { return xor32_max(xor16_max(x)); }
-__device__ __forceinline__ float col_add(float x) { return xor32_add(xor16_add(x)); }
-
-// 8 consecutive entries of a bias / mask row in their storage type; columns >= n read as `pad`.
-template <bool VEC, class T>
-__device__ __forceinline__ auto load_raw8(const T* row, int c0, int n, float pad) {
-    typedef T TV8 __attribute__((ext_vector_type(8)));
-    TV8 v;
-    if (VEC) {   // n % 8 == 0 and rows 16-byte aligned: a group of 8 is all real or all padding
-        if (c0 < n) {
-            v = *reinterpret_cast<const TV8*>(row + c0);
-        } else {
-#pragma unroll
-            for (int i = 0; i < 8; i++) v[i] = (T)pad;
-        }
-    } else {
-#pragma unroll
-        for (int i = 0; i < 8; i++) v[i] = (c0 + i < n) ? row[c0 + i] : (T)pad;
-    }
-    return v;
-}
-
 // NT = compile-time bound on the 16-key tiles of a unit (N <= 16 NT); the workgroup has
 // ceil(N / 16) wavefronts.
 // MASKED: this launch handles the units whose window mask is live; the other units (or all, when
