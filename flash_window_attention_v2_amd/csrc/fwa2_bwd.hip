@@ -75,15 +75,17 @@ __device__ __forceinline__ void async_row_chunk(const E* gsrc, E* lds_wave_base)
 // so the whole block sequence exists twice instead of branching inside every block.
 // `block_start(qb)` runs at the top of every block, after every side value fetched for that block
 // has arrived (the kernel uses it to start the next unit's fetch behind them).
-template <int DT, bool HAS_BIAS, class ME, int NQB, int KT, bool MASKED, class Hook>
+template <int DT, bool HAS_BIAS, class ME, int NQB, int KT, bool MASKED, bool BIG, class Hook>
 __device__ __forceinline__ void unit_blocks(BwdLds<DT, NQB>& L, WaveRegs<DT, NQB, KT>& w,
                                             const typename Elem<DT>::E* bias_t, const ME* mask_t, int n, int nqb,
-                                            int l16, int g, int key0, bool tail_keys, Hook block_start) {
+                                            int l16, int g, int key0, bool tail_keys, int side_stride_big,
+                                            Hook block_start) {
     typedef typename Elem<DT>::E E;
     typedef typename Elem<DT>::V8 V8;
     typedef typename Elem<DT>::V4 V4;
     typedef ME MV4 __attribute__((ext_vector_type(4)));
     constexpr int R = 32 * NQB;
+    const int SS = BIG ? side_stride_big : R;    // row stride of the key-major side tables
 
     // bias (and mask) values of the coming block travel in registers: they are fetched one block
     // ahead so that the L2 round trip overlaps the rest of the block instead of stalling it
@@ -95,8 +97,8 @@ __device__ __forceinline__ void unit_blocks(BwdLds<DT, NQB>& L, WaveRegs<DT, NQB
         for (int kt = 0; kt < KT; kt++)
 #pragma unroll
             for (int t = 0; t < 2; t++) {
-                if (HAS_BIAS) bcur[kt][t] = *reinterpret_cast<const V4*>(bias_t + (int64_t)16 * kt * R + q8n + 4 * t);
-                if (MASKED) mcur[kt][t] = *reinterpret_cast<const MV4*>(mask_t + (int64_t)16 * kt * R + q8n + 4 * t);
+                if (HAS_BIAS) bcur[kt][t] = *reinterpret_cast<const V4*>(bias_t + (int64_t)16 * kt * SS + q8n + 4 * t);
+                if (MASKED) mcur[kt][t] = *reinterpret_cast<const MV4*>(mask_t + (int64_t)16 * kt * SS + q8n + 4 * t);
             }
     };
     fetch_side(0);
@@ -169,16 +171,37 @@ __device__ __forceinline__ void unit_blocks(BwdLds<DT, NQB>& L, WaveRegs<DT, NQB
 // MASKED: this launch handles the units whose window mask is live (and adds the mask); the units
 // with an all-zero mask go through a second launch of the MASKED = false instantiation, so no
 // block ever branches on the mask and each launch has a single copy of the block sequence.
-template <int DT, bool HAS_BIAS, int MASK_DT, int NQB, int KT, bool MASKED>
+// BIG: windows of more than 256 tokens.  The N x N score matrix is cut into 256 x 256 super-tiles;
+// a workgroup then belongs to one (head, query chunk, key chunk), reads only those rows, keeps that
+// tile of dbias in registers and writes its share of dk / dv (already taken back through the
+// normalisation, which is linear) as fp32 partials that dkv_reduce_kernel sums over the query chunks.
+template <int DT, bool HAS_BIAS, int MASK_DT, int NQB, int KT, bool MASKED, bool BIG>
 __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) {
     typedef typename Elem<DT>::E E;
     typedef typename Elem<DT>::V8 V8;
     typedef typename Elem<DT>::V4 V4;
     typedef typename MaskElem<DT, MASK_DT>::E ME;
 
-    const int N = p.n;
-    constexpr int R = 32 * NQB;            // padded rows of every LDS tile and of the key-major side tables
-    const int NPk = p.waves * 16 * KT;     // padded key rows
+    constexpr int R = 32 * NQB;            // padded rows of every LDS tile (and of the side tables unless BIG)
+    const int NPk = p.waves * 16 * KT;     // padded key rows of this workgroup
+    // ---- which head (and, for BIG, which super-tile) this workgroup owns ----
+    int h, grp, q_off = 0, k_off = 0, qs = 0;
+    if (BIG) {
+        int idx = blockIdx.x;
+        grp = idx % p.groups; idx /= p.groups;
+        const int ks = idx % p.n_chunks; idx /= p.n_chunks;
+        qs = idx % p.n_chunks;
+        h = idx / p.n_chunks;
+        q_off = qs * R;
+        k_off = ks * NPk;
+    } else {
+        h = blockIdx.x / p.groups;
+        grp = blockIdx.x - h * p.groups;
+    }
+    const int N = BIG ? min(p.n - q_off, R) : p.n;        // query rows of this workgroup
+    const int NK = BIG ? min(p.n - k_off, NPk) : p.n;     // key rows of this workgroup
+    const int R_tot = BIG ? p.r_tot : R;                  // row stride / padded keys of the side tables
+    const int NPk_tot = BIG ? p.npk_tot : NPk;
     const int nqb = (N + 31) >> 5;         // query blocks of 32 that hold real rows
 
     __shared__ __attribute__((aligned(16))) E lds_Qs[R * kRow];
@@ -207,9 +230,6 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
     const int g_0 = lane >> 4;
     int l16 = l16_0, g = g_0;
 
-    const int h = blockIdx.x / p.groups;
-    const int grp = blockIdx.x - h * p.groups;
-
     float s_true;
     if (p.scale_kind == FWA2_SCALE_TENSOR) {
         float ls = (float)reinterpret_cast<const E*>(p.logit_scale)[h];
@@ -220,7 +240,7 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
     const float scale2 = s_true * kLog2e;
 
     const int key0 = wave * 16 * KT + l16;  // this lane's key in key tile 0 (tile kt: + 16 kt)
-    const bool tail_keys = NPk > N;         // some key columns are padding
+    const bool tail_keys = NPk > NK;        // some key columns are padding
 
     WaveRegs<DT, NQB, KT> w;
 #pragma unroll
@@ -230,26 +250,56 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
 #pragma unroll
             for (int j = 0; j < 8; j++) w.dbacc[a][kt][j] = 0.f;
     const E* bias_t = nullptr;
-    if (HAS_BIAS) bias_t = reinterpret_cast<const E*>(p.bias_t) + ((int64_t)h * NPk + key0) * R;
+    if (HAS_BIAS) bias_t = reinterpret_cast<const E*>(p.bias_t) + ((int64_t)h * NPk_tot + k_off + key0) * R_tot + q_off;
 
-    // ---- which units belong to this launch ----
-    auto mine = [&](int b) -> bool {
-        if (MASK_DT >= 0 && p.mask_live) return (p.mask_live[b % p.n_windows] != 0) == MASKED;
-        return true;
+    // ---- which units belong to this launch.  With the mask flags at hand the windows of this
+    // launch's class (mask live or not) are listed once and the units are dealt out by their rank
+    // within the class, so every workgroup of the head gets the same number of them whatever the
+    // pattern of masked windows. ----
+    __shared__ uint8_t lds_live[kLiveCache];
+    __shared__ uint16_t lds_list[kLiveCache];
+    __shared__ int lds_count;
+    const bool listed = MASK_DT >= 0 && p.mask_live && p.n_windows <= kLiveCache;
+    if (listed) {
+        for (int i = tid; i < p.n_windows; i += nthreads) lds_live[i] = p.mask_live[i];
+        __syncthreads();
+        if (wave_0 == 0) {
+            int cnt = 0;
+            for (int base = 0; base < p.n_windows; base += 64) {
+                const int w = base + lane_0;
+                const bool in = w < p.n_windows && ((lds_live[w] != 0) == MASKED);
+                const unsigned long long bal = __ballot(in);
+                if (in) lds_list[cnt + __popcll(bal & ((1ull << lane_0) - 1ull))] = (uint16_t)w;
+                cnt += __popcll(bal);
+            }
+            if (lane_0 == 0) lds_count = cnt;
+        }
+        __syncthreads();
+    }
+    const int cnt = listed ? __builtin_amdgcn_readfirstlane(lds_count) : 0;
+    const int total = listed ? ((p.bw + p.n_windows - 1) / p.n_windows) * cnt : p.bw;   // ranks to deal out
+    auto unit_of = [&](int t) -> int {
+        if (!listed) return t;
+        const int img = t / cnt;
+        return __builtin_amdgcn_readfirstlane(img * p.n_windows + (int)lds_list[t - img * cnt]);
     };
-    auto next_unit = [&](int b) -> int {
-        for (b += p.groups; b < p.bw; b += p.groups)
-            if (mine(b)) return b;
-        return p.bw;
+    // first rank >= t (in steps of the group count) that names an existing unit of this launch
+    auto rank_from = [&](int t) -> int {
+        for (; t < total; t += p.groups) {
+            const int b = unit_of(t);
+            if (b >= p.bw) continue;
+            if (listed || MASK_DT < 0 || !p.mask_live || ((p.mask_live[b % p.n_windows] != 0) == MASKED)) return t;
+        }
+        return total;
     };
     // ---- asynchronous fetch of one unit's rows into the landing area ----
     auto fetch_unit = [&](int b) __attribute__((always_inline)) {
-        const E* qptr = reinterpret_cast<const E*>(p.q.ptr) + b * p.q.sb + h * p.q.sh;
-        const E* kptr = reinterpret_cast<const E*>(p.k.ptr) + b * p.k.sb + h * p.k.sh;
-        const E* vptr = reinterpret_cast<const E*>(p.v.ptr) + b * p.v.sb + h * p.v.sh;
-        const E* optr = reinterpret_cast<const E*>(p.o.ptr) + b * p.o.sb + h * p.o.sh;
-        const E* doptr = reinterpret_cast<const E*>(p.d_o.ptr) + b * p.d_o.sb + h * p.d_o.sh;
-        const float* lseptr = p.lse + b * p.lse_sb + h * p.lse_sh;
+        const E* qptr = reinterpret_cast<const E*>(p.q.ptr) + b * p.q.sb + h * p.q.sh + q_off * p.q.sn;
+        const E* kptr = reinterpret_cast<const E*>(p.k.ptr) + b * p.k.sb + h * p.k.sh + k_off * p.k.sn;
+        const E* vptr = reinterpret_cast<const E*>(p.v.ptr) + b * p.v.sb + h * p.v.sh + k_off * p.v.sn;
+        const E* optr = reinterpret_cast<const E*>(p.o.ptr) + b * p.o.sb + h * p.o.sh + q_off * p.o.sn;
+        const E* doptr = reinterpret_cast<const E*>(p.d_o.ptr) + b * p.d_o.sb + h * p.d_o.sh + q_off * p.d_o.sn;
+        const float* lseptr = p.lse + b * p.lse_sb + h * p.lse_sh + q_off;
         // re-materialised here so that no per-row address is computed ahead of time and spilled
         // (a spill reload would wait for every fetch already in flight)
         int lane = lane_0, wave = wave_0;
@@ -260,17 +310,17 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
             const int r = row0 + (lane >> 2);
             if (r < N) {
                 async_row_chunk(qptr + (int64_t)r * p.q.sn + dc, L.rawQ + row0 * 32);
-                async_row_chunk(kptr + (int64_t)r * p.k.sn + dc, L.rawK + row0 * 32);
                 async_row_chunk(doptr + (int64_t)r * p.d_o.sn + dc, L.rawDO + row0 * 32);
                 async_row_chunk(optr + (int64_t)r * p.o.sn + dc, L.rawO + row0 * 32);
             }
+            if (r < NK) async_row_chunk(kptr + (int64_t)r * p.k.sn + dc, L.rawK + row0 * 32);
         }
         // v: every wavefront fetches exactly the key rows it owns, so nobody else reads them
 #pragma unroll
         for (int kt = 0; kt < KT; kt++) {
             const int row0 = (wave * KT + kt) * 16;
             const int r = row0 + (lane >> 2);
-            if (r < N) async_row_chunk(vptr + (int64_t)r * p.v.sn + dc, L.rawV + row0 * 32);
+            if (r < NK) async_row_chunk(vptr + (int64_t)r * p.v.sn + dc, L.rawV + row0 * 32);
         }
         for (int r0 = wave * 64; r0 < N; r0 += 64 * p.waves) {
             if (r0 + lane < N)
@@ -286,16 +336,17 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
     }
     __syncthreads();
 
-    int b = grp;
-    if (!mine(b)) b = next_unit(b);
-    if (b < p.bw) fetch_unit(b);
+    int t = rank_from(grp);
+    if (t < total) fetch_unit(unit_of(t));
 
-    while (b < p.bw) {
-        const int b_next = next_unit(b);
+    while (t < total) {
+        const int b = unit_of(t);
+        const int t_next = rank_from(t + p.groups);
+        const int b_next = t_next < total ? unit_of(t_next) : p.bw;
         const ME* mask_t = nullptr;
         if (MASK_DT >= 0) {
             const int wnd = b % p.n_windows;
-            mask_t = reinterpret_cast<const ME*>(p.mask_t) + ((int64_t)wnd * NPk + key0) * R;
+            mask_t = reinterpret_cast<const ME*>(p.mask_t) + ((int64_t)wnd * NPk_tot + k_off + key0) * R_tot + q_off;
         }
 
         // lane-derived values are re-materialised per unit so that the compiler does not keep
@@ -327,7 +378,7 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
                 st8<V8>(L.dOs + r * kRow + dc, do8);
                 if ((tid & 3) == 0) {
                     L.ndelta[r] = -dl;
-                    if (r < N) p.delta[((int64_t)b * p.heads + h) * p.delta_stride + r] = dl;   // for the dq kernel
+                    if (!BIG && r < N) p.delta[((int64_t)b * p.heads + h) * p.delta_stride + r] = dl;   // for the dq kernel
                 }
                 if ((tid & 3) == 1) {
                     float l2 = -INFINITY;          // padded / fully masked rows: P = 0
@@ -352,7 +403,7 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
         // The next unit's fetch starts at the top of the last block: memory returns in issue order,
         // so an earlier start would make every later wait for bias values also wait for the fetch.
         const int fetch_at = nqb - 1;
-        unit_blocks<DT, HAS_BIAS, ME, NQB, KT, MASKED>(L, w, bias_t, mask_t, N, nqb, l16, g, key0, tail_keys, [&](int qb) {
+        unit_blocks<DT, HAS_BIAS, ME, NQB, KT, MASKED, BIG>(L, w, bias_t, mask_t, NK, nqb, l16, g, key0, tail_keys, R_tot, [&](int qb) {
             if (qb == fetch_at && b_next < p.bw) fetch_unit(b_next);
         });
 
@@ -360,7 +411,7 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
 #pragma unroll
         for (int kt = 0; kt < KT; kt++) {
             const int key = key0 + 16 * kt;
-            const bool key_ok = key < N;
+            const bool key_ok = key < NK;
             float x[8], a[8];
             float dot = 0.f;
 #pragma unroll
@@ -378,29 +429,45 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
             const float inv = fabsf(ki);
             const float proj = ki > 0.f ? dot : 0.f;
             if (key_ok) {
-                E* dkp = reinterpret_cast<E*>(const_cast<void*>(p.dk.ptr)) + b * p.dk.sb + h * p.dk.sh + (int64_t)key * p.dk.sn;
-                E* dvp = reinterpret_cast<E*>(const_cast<void*>(p.dv.ptr)) + b * p.dv.sb + h * p.dv.sh + (int64_t)key * p.dv.sn;
+                if (BIG) {
+                    // fp32 partial of this query chunk: [qs][b][h][padded key][32]
+                    const int64_t row = (((int64_t)qs * p.bw + b) * p.heads + h) * NPk_tot + k_off + key;
 #pragma unroll
-                for (int dt = 0; dt < 2; dt++) {
-                    V4 o4, v4;
+                    for (int dt = 0; dt < 2; dt++) {
+                        f32x4 o4, v4;
 #pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        o4[i] = (E)(inv * (a[4 * dt + i] - x[4 * dt + i] * proj));
-                        v4[i] = (E)w.dvacc[kt][dt][i];
+                        for (int i = 0; i < 4; i++) {
+                            o4[i] = inv * (a[4 * dt + i] - x[4 * dt + i] * proj);
+                            v4[i] = w.dvacc[kt][dt][i];
+                        }
+                        *reinterpret_cast<f32x4*>(p.part_dk + row * 32 + 16 * dt + 4 * g) = o4;
+                        *reinterpret_cast<f32x4*>(p.part_dv + row * 32 + 16 * dt + 4 * g) = v4;
                     }
-                    *reinterpret_cast<V4*>(dkp + 16 * dt + 4 * g) = o4;
-                    *reinterpret_cast<V4*>(dvp + 16 * dt + 4 * g) = v4;
+                } else {
+                    E* dkp = reinterpret_cast<E*>(const_cast<void*>(p.dk.ptr)) + b * p.dk.sb + h * p.dk.sh + (int64_t)key * p.dk.sn;
+                    E* dvp = reinterpret_cast<E*>(const_cast<void*>(p.dv.ptr)) + b * p.dv.sb + h * p.dv.sh + (int64_t)key * p.dv.sn;
+#pragma unroll
+                    for (int dt = 0; dt < 2; dt++) {
+                        V4 o4, v4;
+#pragma unroll
+                        for (int i = 0; i < 4; i++) {
+                            o4[i] = (E)(inv * (a[4 * dt + i] - x[4 * dt + i] * proj));
+                            v4[i] = (E)w.dvacc[kt][dt][i];
+                        }
+                        *reinterpret_cast<V4*>(dkp + 16 * dt + 4 * g) = o4;
+                        *reinterpret_cast<V4*>(dvp + 16 * dt + 4 * g) = v4;
+                    }
                 }
             }
         }
-        b = b_next;
+        t = t_next;
     }
 
     // ---- flush the per-workgroup partial sums ----
     if (HAS_BIAS) {
 #pragma unroll
         for (int kt = 0; kt < KT; kt++) {
-            float* dst = p.part_dbias + (((int64_t)h * p.db_parts + p.db_slot0 + grp) * NPk + key0 + 16 * kt) * R;
+            float* dst = p.part_dbias + (((int64_t)h * p.db_parts + p.db_slot0 + grp) * NPk_tot + k_off + key0 + 16 * kt) * R_tot + q_off;
 #pragma unroll
             for (int qb = 0; qb < NQB; qb++) {
                 if (qb < nqb) {
@@ -475,10 +542,43 @@ __global__ void __launch_bounds__(256) reduce_kernel(const BwdParams p, int npk,
     }
 }
 
+// dk, dv = sum over the query chunks of the fp32 partials, cast to the input dtype.
+template <int DT>
+__global__ void __launch_bounds__(256) dkv_reduce_kernel(const BwdParams p) {
+    typedef typename Elem<DT>::E E;
+    typedef typename Elem<DT>::V8 V8;
+    const int64_t rows = (int64_t)p.bw * p.heads * p.n;
+    const int64_t i = (int64_t)blockIdx.x * 64 + (threadIdx.x >> 2);     // (b, h, key) row, 4 threads of 8 columns each
+    if (i >= rows) return;
+    const int key = (int)(i % p.n);
+    const int64_t bh = i / p.n;
+    const int h = (int)(bh % p.heads);
+    const int64_t b = bh / p.heads;
+    const int c8 = (threadIdx.x & 3) * 8;
+    float sk[8], sv[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) { sk[j] = 0.f; sv[j] = 0.f; }
+    for (int qs = 0; qs < p.n_chunks; qs++) {
+        const int64_t row = (((int64_t)qs * p.bw + b) * p.heads + h) * p.npk_tot + key;
+#pragma unroll
+        for (int v = 0; v < 2; v++) {
+            const f32x4 a = *reinterpret_cast<const f32x4*>(p.part_dk + row * 32 + c8 + 4 * v);
+            const f32x4 c = *reinterpret_cast<const f32x4*>(p.part_dv + row * 32 + c8 + 4 * v);
+#pragma unroll
+            for (int j = 0; j < 4; j++) { sk[4 * v + j] += a[j]; sv[4 * v + j] += c[j]; }
+        }
+    }
+    V8 ok, ov;
+#pragma unroll
+    for (int j = 0; j < 8; j++) { ok[j] = (E)sk[j]; ov[j] = (E)sv[j]; }
+    st8<V8>(reinterpret_cast<E*>(const_cast<void*>(p.dk.ptr)) + b * p.dk.sb + h * p.dk.sh + (int64_t)key * p.dk.sn + c8, ok);
+    st8<V8>(reinterpret_cast<E*>(const_cast<void*>(p.dv.ptr)) + b * p.dv.sb + h * p.dv.sh + (int64_t)key * p.dv.sn + c8, ov);
+}
+
 // ---- host side -----------------------------------------------------------------
 static size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
-int backward_supported(int n) { return n >= 1 && n <= 256; }
+int backward_supported(int n) { return n >= 1; }
 
 void dq_geometry(int n, int* waves, int* chunks);
 hipError_t launch_backward_dq(const BwdParams& p, int dtype, bool has_bias, int mask_dt, hipStream_t st);
@@ -488,22 +588,34 @@ hipError_t launch_backward_dq_resident(const BwdParams& p, int dtype, bool has_b
 
 struct BwdPlan {
     int waves, groups, npk, r, nqb_t, kt, dq_waves, dq_chunks, ds_parts, dq_max_groups;
-    size_t off_dbias, off_dscale, off_bias_t, off_mask_t, off_delta, total;
+    int n_chunks;   // > 1: windows of more than 256 tokens, cut into 256 x 256 super-tiles
+    size_t off_dbias, off_dscale, off_bias_t, off_mask_t, off_delta, off_dk, off_dv, total;
     size_t smem;
 };
 
 static BwdPlan make_plan(int heads, int n, int bw, bool has_bias, bool has_mask, int n_windows, int cus) {
     BwdPlan pl;
     const int nqb = (n + 31) / 32;
-    pl.nqb_t = nqb <= 2 ? 2 : (nqb <= 4 ? 4 : 8);
-    pl.r = 32 * pl.nqb_t;
-    // up to 128 queries a wavefront owns one 16-key tile (<= 128 registers, several workgroups
-    // per CU); above that two tiles (<= 256 registers, one workgroup of 8 wavefronts per CU)
-    pl.kt = nqb <= 4 ? 1 : 2;
-    pl.waves = (n + 16 * pl.kt - 1) / (16 * pl.kt);
-    pl.npk = pl.waves * 16 * pl.kt;
-    const int wg_per_cu = pl.nqb_t == 2 ? 4 : (pl.nqb_t == 4 ? 2 : 1);
-    int groups = (cus * wg_per_cu) / heads;
+    pl.n_chunks = (n + 255) / 256;
+    int wg_per_cu;
+    if (pl.n_chunks > 1) {
+        // every workgroup is a full 256 x 256 super-tile kernel; npk / r are the padded totals
+        pl.nqb_t = 8;
+        pl.kt = 2;
+        pl.waves = 8;
+        pl.npk = pl.r = 256 * pl.n_chunks;
+        wg_per_cu = 1;
+    } else {
+        pl.nqb_t = nqb <= 2 ? 2 : (nqb <= 4 ? 4 : 8);
+        pl.r = 32 * pl.nqb_t;
+        // up to 128 queries a wavefront owns one 16-key tile (<= 128 registers, several workgroups
+        // per CU); above that two tiles (<= 256 registers, one workgroup of 8 wavefronts per CU)
+        pl.kt = nqb <= 4 ? 1 : 2;
+        pl.waves = (n + 16 * pl.kt - 1) / (16 * pl.kt);
+        pl.npk = pl.waves * 16 * pl.kt;
+        wg_per_cu = pl.nqb_t == 2 ? 4 : (pl.nqb_t == 4 ? 2 : 1);
+    }
+    int groups = (cus * wg_per_cu) / (heads * pl.n_chunks * pl.n_chunks);
     if (groups < 1) groups = 1;
     if (groups > bw) groups = bw;
     pl.groups = groups;
@@ -519,7 +631,11 @@ static BwdPlan make_plan(int heads, int n, int bw, bool has_bias, bool has_mask,
     pl.off_dscale = off;
     off += align256((size_t)heads * ds_slots * 4);
     pl.off_delta = off;
-    off += align256((size_t)bw * heads * pl.r * 4);
+    if (pl.n_chunks == 1) off += align256((size_t)bw * heads * pl.r * 4);
+    pl.off_dk = off;
+    if (pl.n_chunks > 1) off += align256((size_t)pl.n_chunks * bw * heads * pl.npk * 32 * 4);
+    pl.off_dv = off;
+    if (pl.n_chunks > 1) off += align256((size_t)pl.n_chunks * bw * heads * pl.npk * 32 * 4);
     pl.off_bias_t = off;
     if (has_bias) off += align256((size_t)heads * pl.npk * pl.r * 2);
     pl.off_mask_t = off;
@@ -542,30 +658,31 @@ static int resident_per_cu(K kern, int threads) {
     return n;
 }
 
-template <int DT, bool HAS_BIAS, int MASK_DT, int NQB, int KT>
+template <int DT, bool HAS_BIAS, int MASK_DT, int NQB, int KT, bool BIG>
 static hipError_t launch_main(BwdParams p, const BwdPlan& pl, hipStream_t st, int* groups_out) {
-    // never more workgroups per head than the plan sized the workspace for
+    // never more workgroups per head (and super-tile) than the plan sized the workspace for
     static const int fit = [&] {
-        const int a = resident_per_cu(bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, false>, 64 * pl.waves);
-        const int b = resident_per_cu(bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, true>, 64 * pl.waves);
+        const int a = resident_per_cu(bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, false, BIG>, 64 * pl.waves);
+        const int b = resident_per_cu(bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, true, BIG>, 64 * pl.waves);
         return a < b ? a : b;
     }();
-    int groups = (p.cus * fit) / p.heads;
+    const int tiles = pl.n_chunks * pl.n_chunks;
+    int groups = (p.cus * fit) / (p.heads * tiles);
     if (groups < 1) groups = 1;
     if (groups > pl.groups) groups = pl.groups;
     p.groups = groups;
     p.db_parts = (MASK_DT >= 0 && p.mask_live != nullptr) ? 2 * groups : groups;
-    const dim3 grid(p.heads * groups), block(64 * pl.waves);
+    const dim3 grid(p.heads * tiles * groups), block(64 * pl.waves);
     if (p.ev_start) (void)hipEventRecord(p.ev_start, st);
     // launch for the units whose mask is all zero (or every unit when there is no mask) ...
     if (MASK_DT < 0 || p.mask_live != nullptr) {
         p.db_slot0 = 0;
-        hipLaunchKernelGGL((bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, false>), grid, block, 0, st, p);
+        hipLaunchKernelGGL((bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, false, BIG>), grid, block, 0, st, p);
     }
     // ... and for the units whose mask is live
     if (MASK_DT >= 0) {
         p.db_slot0 = p.mask_live != nullptr ? groups : 0;
-        hipLaunchKernelGGL((bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, true>), grid, block, 0, st, p);
+        hipLaunchKernelGGL((bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, true, BIG>), grid, block, 0, st, p);
     }
     if (p.ev_stop) (void)hipEventRecord(p.ev_stop, st);
     hipError_t e = hipGetLastError();
@@ -577,9 +694,10 @@ static hipError_t launch_main(BwdParams p, const BwdPlan& pl, hipStream_t st, in
 
 template <int DT, bool HAS_BIAS, int MASK_DT>
 static hipError_t launch_nqb(const BwdParams& p, const BwdPlan& pl, hipStream_t st, int* groups_out) {
-    if (pl.nqb_t == 2) return launch_main<DT, HAS_BIAS, MASK_DT, 2, 1>(p, pl, st, groups_out);
-    if (pl.nqb_t == 4) return launch_main<DT, HAS_BIAS, MASK_DT, 4, 1>(p, pl, st, groups_out);
-    return launch_main<DT, HAS_BIAS, MASK_DT, 8, 2>(p, pl, st, groups_out);
+    if (pl.n_chunks > 1) return launch_main<DT, HAS_BIAS, MASK_DT, 8, 2, true>(p, pl, st, groups_out);
+    if (pl.nqb_t == 2) return launch_main<DT, HAS_BIAS, MASK_DT, 2, 1, false>(p, pl, st, groups_out);
+    if (pl.nqb_t == 4) return launch_main<DT, HAS_BIAS, MASK_DT, 4, 1, false>(p, pl, st, groups_out);
+    return launch_main<DT, HAS_BIAS, MASK_DT, 8, 2, false>(p, pl, st, groups_out);
 }
 
 template <int DT>
@@ -598,6 +716,11 @@ static hipError_t launch_bwd_dt(BwdParams p, bool has_bias, int mask_dt, hipStre
     p.mask_t = ws + pl.off_mask_t;
     p.delta = reinterpret_cast<float*>(ws + pl.off_delta);
     p.delta_stride = pl.r;
+    p.n_chunks = pl.n_chunks;
+    p.r_tot = pl.r;
+    p.npk_tot = pl.npk;
+    p.part_dk = reinterpret_cast<float*>(ws + pl.off_dk);
+    p.part_dv = reinterpret_cast<float*>(ws + pl.off_dv);
     const dim3 tgrid(pl.r / 32, (pl.npk + 31) / 32, 1);
     if (has_bias) {
         dim3 gr(tgrid.x, tgrid.y, p.heads);
@@ -631,6 +754,12 @@ static hipError_t launch_bwd_dt(BwdParams p, bool has_bias, int mask_dt, hipStre
     if (e != hipSuccess) return e;
     p.groups = gr_out[0];
     p.db_parts = gr_out[1];
+    if (pl.n_chunks > 1) {
+        const int64_t rows = (int64_t)p.bw * p.heads * p.n;
+        hipLaunchKernelGGL(dkv_reduce_kernel<DT>, dim3((unsigned)((rows + 63) / 64)), dim3(256), 0, st, p);
+        e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
     if (backward_dq_resident_supported(p.n)) {
         int parts = 0;
         e = launch_backward_dq_resident(p, DT, has_bias, mask_dt, st, pl.dq_max_groups, &parts);

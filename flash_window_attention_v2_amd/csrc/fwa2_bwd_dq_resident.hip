@@ -24,8 +24,13 @@
 
 namespace fwa2 {
 
-template <int DT, bool HAS_BIAS, int MASK_DT, int NT, bool VEC, bool MASKED>
-__global__ void __launch_bounds__(64 * NT) bwd_dq_resident_kernel(const BwdParams p) {
+constexpr int kDqSub = 2;    // 16-row query tiles per wavefront (see below)
+
+// SUB = 16-row query tiles per wavefront.  With SUB = 2 a wavefront owns 32 query rows as two
+// independent tiles that share every K / V operand it reads from LDS; a unit of 256 rows then takes
+// 8 wavefronts of up to 256 registers instead of 16 of up to 128.
+template <int DT, bool HAS_BIAS, int MASK_DT, int NT, bool VEC, bool MASKED, int SUB>
+__global__ void __launch_bounds__(64 * NT / SUB) bwd_dq_resident_kernel(const BwdParams p) {
     typedef typename Elem<DT>::E E;
     typedef typename Elem<DT>::V8 V8;
     typedef typename Elem<DT>::V4 V4;
@@ -35,6 +40,7 @@ __global__ void __launch_bounds__(64 * NT) bwd_dq_resident_kernel(const BwdParam
     typedef ME MV8 __attribute__((ext_vector_type(8)));
     constexpr int ROWS = 16 * NT;
     constexpr int S = kLdsStride;
+    constexpr int WR = 16 * SUB;          // rows per wavefront (queries owned, K / V rows staged)
 
     __shared__ __attribute__((aligned(16))) SE lds_K[2][ROWS * S];
     __shared__ __attribute__((aligned(16))) E lds_V[2][ROWS * S];
@@ -79,45 +85,56 @@ __global__ void __launch_bounds__(64 * NT) bwd_dq_resident_kernel(const BwdParam
         st8<V8>(lds_rawDO + i * 8, zero8<V8>());
     }
 
-    const int qi = wave * 16 + l16;
-    const bool qv = qi < N;
-    const int qc = min(qi, N - 1);
+    int qi[SUB], qc[SUB];
+    bool qv[SUB];
+#pragma unroll
+    for (int u = 0; u < SUB; u++) {
+        qi[u] = wave * WR + 16 * u + l16;
+        qv[u] = qi[u] < N;
+        qc[u] = min(qi[u], N - 1);
+    }
 
     // ---- resident bias (see fwa2_fwd_resident.hip): acc0[2kp][i] <-> key 32kp + 8g + i,
     // acc0[2kp+1][i] <-> key 32kp + 8g + 4 + i, log2 domain, minus the row bound ----
-    f32x4 acc0[NT];
-    float mb = 0.f, mn = 0.f;
-    if (HAS_BIAS) {
-        const E* brow = reinterpret_cast<const E*>(p.bias) + h * p.bias_sh + (int64_t)qc * p.bias_sn;
-        mb = -INFINITY;
-        mn = INFINITY;
+    f32x4 acc0[SUB][NT];
+    float m_fixed[SUB];
+    float range = 0.f;
 #pragma unroll
-        for (int kp = 0; kp < NT / 2; kp++) {
-            const auto raw = load_raw8<VEC, E>(brow, 32 * kp + 8 * g, N, -INFINITY);
+    for (int u = 0; u < SUB; u++) {
+        float mb = 0.f, mn = 0.f;
+        if (HAS_BIAS) {
+            const E* brow = reinterpret_cast<const E*>(p.bias) + h * p.bias_sh + (int64_t)qc[u] * p.bias_sn;
+            mb = -INFINITY;
+            mn = INFINITY;
 #pragma unroll
-            for (int j = 0; j < 8; j++) {
-                const float v = (float)raw[j] * kLog2e;
-                acc0[2 * kp + (j >> 2)][j & 3] = v;
-                mb = fmaxf(mb, v);
-                mn = fminf(mn, (32 * kp + 8 * g + j < N) ? v : INFINITY);
+            for (int kp = 0; kp < NT / 2; kp++) {
+                const auto raw = load_raw8<VEC, E>(brow, 32 * kp + 8 * g, N, -INFINITY);
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    const float v = (float)raw[j] * kLog2e;
+                    acc0[u][2 * kp + (j >> 2)][j & 3] = v;
+                    mb = fmaxf(mb, v);
+                    mn = fminf(mn, (32 * kp + 8 * g + j < N) ? v : INFINITY);
+                }
             }
+            mb = col_max(mb);
+            mn = -col_max(-mn);
+            if (!(mb > -INFINITY)) { mb = 0.f; mn = 0.f; }
+        } else {
+#pragma unroll
+            for (int kt = 0; kt < NT; kt++)
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+                    acc0[u][kt][i] = (32 * (kt >> 1) + 8 * g + 4 * (kt & 1) + i < N) ? 0.f : -INFINITY;
         }
-        mb = col_max(mb);
-        mn = -col_max(-mn);
-        if (!(mb > -INFINITY)) { mb = 0.f; mn = 0.f; }
-    } else {
+        m_fixed[u] = mb + scale2;
 #pragma unroll
         for (int kt = 0; kt < NT; kt++)
 #pragma unroll
-            for (int i = 0; i < 4; i++)
-                acc0[kt][i] = (32 * (kt >> 1) + 8 * g + 4 * (kt & 1) + i < N) ? 0.f : -INFINITY;
+            for (int i = 0; i < 4; i++) acc0[u][kt][i] -= m_fixed[u];
+        const float r = (mb - mn == mb - mn) ? mb - mn : INFINITY;
+        range = fmaxf(range, r);
     }
-    const float m_fixed = mb + scale2;
-#pragma unroll
-    for (int kt = 0; kt < NT; kt++)
-#pragma unroll
-        for (int i = 0; i < 4; i++) acc0[kt][i] -= m_fixed;
-    float range = (mb - mn == mb - mn) ? mb - mn : INFINITY;
 #pragma unroll
     for (int off = 8; off >= 1; off >>= 1) range = fmaxf(range, __shfl_xor(range, off));
     // w = 2^(m - lse2) may be folded into dO when it cannot leave the bf16 range
@@ -161,10 +178,9 @@ __global__ void __launch_bounds__(64 * NT) bwd_dq_resident_kernel(const BwdParam
         return total;
     };
 
-    // ---- per-unit fetch: K / V rows by DMA, this lane's share of its query row in registers ----
-    const int frow = wave * 16 + (lane >> 2);
-    const int fc8 = (lane & 3) * 8;
-    struct Row { float lse, delta; };
+    // ---- per-unit fetch: the wavefront's WR rows of k, v (which it will stage) and of q, dO (its own
+    // queries) by DMA, 16 rows per instruction; lse and delta of its queries in registers ----
+    struct Row { float lse[SUB], delta[SUB]; };
     auto dma16 = [&](const E* src, E* lds_wave_base) __attribute__((always_inline)) {
         __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
                                          (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
@@ -174,48 +190,57 @@ __global__ void __launch_bounds__(64 * NT) bwd_dq_resident_kernel(const BwdParam
         // a dozen registers for the whole kernel
         int ln = lane;
         asm volatile("" : "+v"(ln));
-        const int frow = wave * 16 + (ln >> 2);
         const int fc8 = (ln & 3) * 8;
-        const int qi = wave * 16 + (ln & 15);
-        const bool qv = qi < N;
-        if (frow < N) {   // rows wave*16 .. +15 of k, v (to be staged by this wavefront) and of q, dO (its own queries)
-            dma16(reinterpret_cast<const E*>(p.k.ptr) + b * p.k.sb + h * p.k.sh + (int64_t)frow * p.k.sn + fc8,
-                  lds_rawK + wave * 16 * 32);
-            dma16(reinterpret_cast<const E*>(p.v.ptr) + b * p.v.sb + h * p.v.sh + (int64_t)frow * p.v.sn + fc8,
-                  lds_rawV + wave * 16 * 32);
-            dma16(reinterpret_cast<const E*>(p.q.ptr) + b * p.q.sb + h * p.q.sh + (int64_t)frow * p.q.sn + fc8,
-                  lds_rawQ + wave * 16 * 32);
-            dma16(reinterpret_cast<const E*>(p.d_o.ptr) + b * p.d_o.sb + h * p.d_o.sh + (int64_t)frow * p.d_o.sn + fc8,
-                  lds_rawDO + wave * 16 * 32);
-        }
-        r.lse = -INFINITY; r.delta = 0.f;
-        if (qv) {
-            r.lse = p.lse[b * p.lse_sb + h * p.lse_sh + qi];
-            r.delta = p.delta[((int64_t)b * p.heads + h) * p.delta_stride + qi];
+#pragma unroll
+        for (int u = 0; u < SUB; u++) {
+            const int row0 = wave * WR + 16 * u;
+            const int frow = row0 + (ln >> 2);
+            if (frow < N) {
+                dma16(reinterpret_cast<const E*>(p.k.ptr) + b * p.k.sb + h * p.k.sh + (int64_t)frow * p.k.sn + fc8,
+                      lds_rawK + row0 * 32);
+                dma16(reinterpret_cast<const E*>(p.v.ptr) + b * p.v.sb + h * p.v.sh + (int64_t)frow * p.v.sn + fc8,
+                      lds_rawV + row0 * 32);
+                dma16(reinterpret_cast<const E*>(p.q.ptr) + b * p.q.sb + h * p.q.sh + (int64_t)frow * p.q.sn + fc8,
+                      lds_rawQ + row0 * 32);
+                dma16(reinterpret_cast<const E*>(p.d_o.ptr) + b * p.d_o.sb + h * p.d_o.sh + (int64_t)frow * p.d_o.sn + fc8,
+                      lds_rawDO + row0 * 32);
+            }
+            const int q = row0 + (ln & 15);
+            r.lse[u] = -INFINITY; r.delta[u] = 0.f;
+            if (q < N) {
+                r.lse[u] = p.lse[b * p.lse_sb + h * p.lse_sh + q];
+                r.delta[u] = p.delta[((int64_t)b * p.heads + h) * p.delta_stride + q];
+            }
         }
     };
     auto stage = [&](int buf) __attribute__((always_inline)) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        const V8 kk = ld8<V8>(lds_rawK + frow * 32 + fc8);
-        const V8 vv = ld8<V8>(lds_rawV + frow * 32 + fc8);
-        float x[8];
-        unpack8(kk, x);
-        float ss = 0.f;
+        const int fc8 = (lane & 3) * 8;
 #pragma unroll
-        for (int j = 0; j < 8; j++) ss += x[j] * x[j];
-        ss = quad_add(ss);
-        const float inv = inv_norm(ss);
-        SV8 kn;
+        for (int u = 0; u < SUB; u++) {
+            const int frow = wave * WR + 16 * u + (lane >> 2);
+            const V8 kk = ld8<V8>(lds_rawK + frow * 32 + fc8);
+            const V8 vv = ld8<V8>(lds_rawV + frow * 32 + fc8);
+            float x[8];
+            unpack8(kk, x);
+            float ss = 0.f;
 #pragma unroll
-        for (int j = 0; j < 8; j++) kn[j] = (SE)(x[j] * inv);
-        st8<SV8>(&lds_K[buf][frow * S + fc8], kn);
-        st8<V8>(&lds_V[buf][frow * S + fc8], vv);
+            for (int j = 0; j < 8; j++) ss += x[j] * x[j];
+            ss = quad_add(ss);
+            const float inv = inv_norm(ss);
+            SV8 kn;
+#pragma unroll
+            for (int j = 0; j < 8; j++) kn[j] = (SE)(x[j] * inv);
+            st8<SV8>(&lds_K[buf][frow * S + fc8], kn);
+            st8<V8>(&lds_V[buf][frow * S + fc8], vv);
+        }
     };
 
     __syncthreads();
     int t = rank_from(grp);
     Row row;
-    row.lse = -INFINITY; row.delta = 0.f;
+#pragma unroll
+    for (int u = 0; u < SUB; u++) { row.lse[u] = -INFINITY; row.delta[u] = 0.f; }
     if (t < total) {
         fetch(unit_of(t), row);
         stage(0);
@@ -229,68 +254,77 @@ __global__ void __launch_bounds__(64 * NT) bwd_dq_resident_kernel(const BwdParam
         const int tn = rank_from(t + groups);
         const int bn = tn < total ? unit_of(tn) : p.bw;
 
-        const ME* mrow = nullptr;
+        const ME* mrow[SUB];
         bool safe = false;
+#pragma unroll
+        for (int u = 0; u < SUB; u++) mrow[u] = nullptr;
         if (MASKED) {
             const int w = b % p.n_windows;
             safe = p.mask_live ? (flags_of(b) & 2) != 0 : false;
-            mrow = reinterpret_cast<const ME*>(p.mask) + w * p.mask_sw + (int64_t)qc * p.mask_sn;
+#pragma unroll
+            for (int u = 0; u < SUB; u++)
+                mrow[u] = reinterpret_cast<const ME*>(p.mask) + w * p.mask_sw + (int64_t)qc[u] * p.mask_sn;
         }
         const bool fold = wave_fold && (!MASKED || safe);
 
-        // ---- this unit's operands out of the prefetched row ----
-        SV8 bq;
-        V8 bd;
-        float nl, nd, inv, nrm;
-        {
+        // ---- this unit's operands out of the landed rows ----
+        SV8 bq[SUB];
+        V8 bd[SUB];
+        f32x4 ndv[SUB], dqacc[SUB][2];
+        float nl[SUB], inv[SUB];
+#pragma unroll
+        for (int u = 0; u < SUB; u++) {
             // the rows landed before the previous unit's barrier (the first unit's before the one above)
-            const V8 qcur = ld8<V8>(lds_rawQ + (wave * 16 + l16) * 32 + 8 * g);
-            const V8 docur = ld8<V8>(lds_rawDO + (wave * 16 + l16) * 32 + 8 * g);
+            const V8 qcur = ld8<V8>(lds_rawQ + (wave * WR + 16 * u + l16) * 32 + 8 * g);
+            const V8 docur = ld8<V8>(lds_rawDO + (wave * WR + 16 * u + l16) * 32 + 8 * g);
             float x[8];
             unpack8(qcur, x);
             float ss = 0.f;
 #pragma unroll
             for (int j = 0; j < 8; j++) ss += x[j] * x[j];
             ss = col_add(ss);
-            nrm = sqrtf(ss);
-            inv = 1.0f / fmaxf(nrm, kNormEps);
-            const float sc = scale2 * inv;
+            inv[u] = 1.0f / fmaxf(sqrtf(ss), kNormEps);
+            const float sc = scale2 * inv[u];
 #pragma unroll
-            for (int j = 0; j < 8; j++) bq[j] = (SE)(x[j] * sc);
-            nl = (row.lse == -INFINITY) ? -INFINITY : m_fixed - row.lse * kLog2e;   // fully masked row: P = 0
+            for (int j = 0; j < 8; j++) bq[u][j] = (SE)(x[j] * sc);
+            // fully masked row (lse = -inf): P = 0
+            nl[u] = (row.lse[u] == -INFINITY) ? -INFINITY : m_fixed[u] - row.lse[u] * kLog2e;
+            float nd;
             if (fold) {
-                const float w = fast_exp2(nl);
+                const float w = fast_exp2(nl[u]);
 #pragma unroll
-                for (int j = 0; j < 8; j++) bd[j] = (E)((float)docur[j] * w);
-                nd = -row.delta * w;
-                nl = 0.f;
+                for (int j = 0; j < 8; j++) bd[u][j] = (E)((float)docur[j] * w);
+                nd = -row.delta[u] * w;
+                nl[u] = 0.f;
             } else {
-                bd = docur;
-                nd = -row.delta;
+                bd[u] = docur;
+                nd = -row.delta[u];
             }
+#pragma unroll
+            for (int i = 0; i < 4; i++) { dqacc[u][0][i] = 0.f; dqacc[u][1][i] = 0.f; ndv[u][i] = nd; }
         }
         if (bn < p.bw) fetch(bn, row);      // in flight while this unit is computed
 
         const SE* Kb = &lds_K[cur][0];
         const E* Vb = &lds_V[cur][0];
-        f32x4 dqacc[2], ndv;
-#pragma unroll
-        for (int i = 0; i < 4; i++) { dqacc[0][i] = 0.f; dqacc[1][i] = 0.f; ndv[i] = nd; }
 
-        auto group = [&](int kp, bool with_mask, bool folded, const MV8& mk) __attribute__((always_inline)) {
+        auto group = [&](int kp, bool folded, const MV8* mk) __attribute__((always_inline)) {
             const int krow = 32 * kp + 8 * (l16 >> 2) + (l16 & 3);
-            SV8 bz;
+            SV8 bz[SUB];
 #pragma unroll
             for (int half = 0; half < 2; half++) {
                 const SV8 ak = ld8<SV8>(Kb + (krow + 4 * half) * S + 8 * g);
                 const V8 av = ld8<V8>(Vb + (krow + 4 * half) * S + 8 * g);
-                f32x4 s = Elem<kScoreDT>::mfma16(ak, bq, acc0[2 * kp + half]);
-                const f32x4 dp = Elem<DT>::mfma16(av, bd, ndv);
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    if (MASK_DT >= 0 && with_mask) s[i] = fmaf((float)mk[4 * half + i], kLog2e, s[i]);
-                    const float e = folded ? fast_exp2(s[i]) : fast_exp2(s[i] + nl);
-                    bz[4 * half + i] = (SE)(e * dp[i]);
+                for (int u = 0; u < SUB; u++) {
+                    f32x4 s = Elem<kScoreDT>::mfma16(ak, bq[u], acc0[u][2 * kp + half]);
+                    const f32x4 dp = Elem<DT>::mfma16(av, bd[u], ndv[u]);
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        if (MASKED) s[i] = fmaf((float)mk[u][4 * half + i], kLog2e, s[i]);
+                        const float e = folded ? fast_exp2(s[i]) : fast_exp2(s[i] + nl[u]);
+                        bz[u][4 * half + i] = (SE)(e * dp[i]);
+                    }
                 }
             }
 #pragma unroll
@@ -298,21 +332,28 @@ __global__ void __launch_bounds__(64 * NT) bwd_dq_resident_kernel(const BwdParam
                 // A row m <-> d = 8 (m / 4) + 4 dt + m % 4, so that this lane's accumulators hold d = 8g + 4dt + i
                 const SE* klo = Kb + (32 * kp + 8 * g + (l16 >> 2)) * S + 8 * (l16 & 3) + 4 * dt;
                 const SV8 akt = lds_tr8<kScoreDT>(klo, klo + 4 * S);
-                dqacc[dt] = Elem<kScoreDT>::mfma16(akt, bz, dqacc[dt]);
+#pragma unroll
+                for (int u = 0; u < SUB; u++) dqacc[u][dt] = Elem<kScoreDT>::mfma16(akt, bz[u], dqacc[u][dt]);
             }
         };
         auto body = [&](bool folded) __attribute__((always_inline)) {
-            MV8 mq[2];
+            MV8 mq[2][SUB];      // mask rows travel two key groups ahead of their use
             if (MASKED) {
-                mq[0] = load_raw8<VEC, ME>(mrow, 8 * g, N, 0.f);
-                mq[1] = load_raw8<VEC, ME>(mrow, 32 + 8 * g, N, 0.f);
+#pragma unroll
+                for (int u = 0; u < SUB; u++) {
+                    mq[0][u] = load_raw8<VEC, ME>(mrow[u], 8 * g, N, 0.f);
+                    mq[1][u] = load_raw8<VEC, ME>(mrow[u], 32 + 8 * g, N, 0.f);
+                }
             }
 #pragma unroll
             for (int kp = 0; kp < NT / 2; kp++) {
                 if (32 * kp < N) {
-                    group(kp, MASKED, folded, mq[kp & 1]);
-                    __builtin_amdgcn_sched_barrier(0);   // keep the groups apart: their temporaries must not pile up
-                    if (MASKED && kp + 2 < NT / 2) mq[kp & 1] = load_raw8<VEC, ME>(mrow, 32 * (kp + 2) + 8 * g, N, 0.f);
+                    group(kp, folded, mq[kp & 1]);
+                    if (MASKED && kp + 2 < NT / 2) {
+#pragma unroll
+                        for (int u = 0; u < SUB; u++)
+                            mq[kp & 1][u] = load_raw8<VEC, ME>(mrow[u], 32 * (kp + 2) + 8 * g, N, 0.f);
+                    }
                 }
             }
         };
@@ -322,27 +363,30 @@ __global__ void __launch_bounds__(64 * NT) bwd_dq_resident_kernel(const BwdParam
 
         // ---- back through q / max(|q|, eps); q_hat . dq_hat is this row's share of dlogit_scale ----
         // q_hat is taken back from the fp16 score operand (q_hat s log2e), which is live anyway
-        float qh[8];
-        float dot = 0.f;
         const float unscale = 1.0f / scale2;
-#pragma unroll
-        for (int j = 0; j < 8; j++) {
-            qh[j] = (float)bq[j] * unscale;
-            dot += dqacc[j >> 2][j & 3] * qh[j];
-        }
-        dot = col_add(dot);
-        const float proj = nrm > kNormEps ? dot : 0.f;
-        const float f = s_true * inv;
         int ln2 = lane;
         asm volatile("" : "+v"(ln2));
-        const int qi2 = wave * 16 + (ln2 & 15);
-        if (qv) {
-            E* dqrow = reinterpret_cast<E*>(const_cast<void*>(p.dq.ptr)) + b * p.dq.sb + h * p.dq.sh + (int64_t)qi2 * p.dq.sn;
-            V8 o8;
 #pragma unroll
-            for (int j = 0; j < 8; j++) o8[j] = (E)(f * (dqacc[j >> 2][j & 3] - qh[j] * proj));
-            st8<V8>(dqrow + 8 * (ln2 >> 4), o8);
-            if (g == 0) ds_acc += dot;
+        for (int u = 0; u < SUB; u++) {
+            float qh[8];
+            float dot = 0.f;
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                qh[j] = (float)bq[u][j] * unscale;
+                dot += dqacc[u][j >> 2][j & 3] * qh[j];
+            }
+            dot = col_add(dot);
+            const float proj = inv[u] < 0.5f / kNormEps ? dot : 0.f;      // |q| <= eps: no projection
+            const float f = s_true * inv[u];
+            const int q = wave * WR + 16 * u + (ln2 & 15);
+            if (q < N) {
+                E* dqrow = reinterpret_cast<E*>(const_cast<void*>(p.dq.ptr)) + b * p.dq.sb + h * p.dq.sh + (int64_t)q * p.dq.sn;
+                V8 o8;
+#pragma unroll
+                for (int j = 0; j < 8; j++) o8[j] = (E)(f * (dqacc[u][j >> 2][j & 3] - qh[j] * proj));
+                st8<V8>(dqrow + 8 * (ln2 >> 4), o8);
+                if (g == 0) ds_acc += dot;
+            }
         }
 
         __syncthreads();
@@ -376,10 +420,12 @@ static int resident_fit(K kern, int threads) {
 // Launches the kernel(s) and reports how many dscale partials per head they wrote.
 template <int DT, bool HAS_BIAS, int MASK_DT, int NT, bool VEC>
 static hipError_t launch_nt(BwdParams p, hipStream_t st, int max_groups, int* ds_parts_out) {
-    const int waves = (p.n + 15) / 16;
-    static const int fit_plain = resident_fit(bwd_dq_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, false>, 64 * NT);
+    constexpr int SUB = kDqSub;
+    const int waves = (p.n + 16 * SUB - 1) / (16 * SUB);
+    static const int fit_plain =
+        resident_fit(bwd_dq_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, false, SUB>, 64 * NT / SUB);
     static const int fit_masked =
-        MASK_DT >= 0 ? resident_fit(bwd_dq_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, true>, 64 * NT) : 1;
+        MASK_DT >= 0 ? resident_fit(bwd_dq_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, true, SUB>, 64 * NT / SUB) : 1;
     auto groups_for = [&](int fit) {
         int groups = (p.cus * fit) / p.heads;
         if (groups < 1) groups = 1;
@@ -394,13 +440,13 @@ static hipError_t launch_nt(BwdParams p, hipStream_t st, int max_groups, int* ds
     if (g_plain) {
         p.dq_groups = g_plain;
         p.ds_slot0 = 0;
-        hipLaunchKernelGGL((bwd_dq_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, false>), dim3(p.heads * g_plain),
+        hipLaunchKernelGGL((bwd_dq_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, false, SUB>), dim3(p.heads * g_plain),
                            dim3(64 * waves), 0, st, p);
     }
     if (g_masked) {
         p.dq_groups = g_masked;
         p.ds_slot0 = g_plain;
-        hipLaunchKernelGGL((bwd_dq_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, true>), dim3(p.heads * g_masked),
+        hipLaunchKernelGGL((bwd_dq_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, true, SUB>), dim3(p.heads * g_masked),
                            dim3(64 * waves), 0, st, p);
     }
     *ds_parts_out = p.ds_parts;

@@ -250,6 +250,11 @@ struct BwdParams {
     int dq_groups;       // workgroups per head of the current launch of the resident dq kernel
     float* delta;        // [BW * H, delta_stride] fp32 rowsum(o * dO), written by the key-side kernel
     int delta_stride;
+    // windows of more than 256 tokens: 256 x 256 super-tiles of the score matrix
+    int n_chunks;        // chunks of 256 rows per side
+    int r_tot, npk_tot;  // padded query / key extents of the key-major side tables and partial tiles
+    float* part_dk;      // [n_chunks, BW, H, npk_tot, 32] fp32 partials over the query chunks
+    float* part_dv;
     int dq_waves;        // wavefronts per workgroup of the dq kernel
     int dq_chunks;       // dq workgroups per (bw, head)
     bool side_vec;       // rows of bias and mask (query-major) may be read with 16-byte loads, n % 8 == 0

@@ -45,7 +45,27 @@ def classic_fwd_bwd(q, k, v, logit_scale, bias, mask, do, dtype=torch.float32):
     ml = None if mask is None else mask.detach().to(dtype)
     o = win_attention_classic(ql, kl, vl, sl, bl, ml)
     o.backward(do.detach().to(dtype))
+    # Conditioning of dlogit_scale: it is the signed sum over all (bw, i, j) of s dZ_ij c_ij, which
+    # can cancel almost completely; dscale_l1[h] is the sum of the absolute terms.  The cosine scores
+    # are recovered from the gradient identity d(o.dO)/dC = dZ, i.e. from autograd of the same graph.
+    dscale_l1 = None
+    if sl is not None:
+        with torch.enable_grad():
+            qh = F.normalize(ql.detach(), dim=-1)
+            kh = F.normalize(kl.detach(), dim=-1)
+            cos = (qh @ kh.transpose(-1, -2)).requires_grad_(True)
+            s = torch.exp(torch.clamp(sl.detach(), max=math.log(100.0)))
+            scores = cos * s
+            if bl is not None:
+                scores = scores + bl.detach()[None]
+            if ml is not None:
+                n_w = ml.shape[0]
+                bw_, h_, n_q, n_k = scores.shape
+                scores = (scores.reshape(bw_ // n_w, n_w, h_, n_q, n_k) + ml[None, :, None]).reshape(bw_, h_, n_q, n_k)
+            (torch.softmax(scores, dim=-1) @ vl.detach() * do.detach().to(dtype)).sum().backward()
+        dscale_l1 = (cos.grad * cos.detach()).abs().sum(dim=(0, 2, 3))
     return {
+        "dscale_l1": dscale_l1,
         "o": o.detach(),
         "dq": ql.grad,
         "dk": kl.grad,
