@@ -159,7 +159,8 @@ int fwa2_forward(const fwa2_problem* p) {
     k.logit_scale = p->logit_scale;
     k.bias = p->bias.ptr; k.bias_sh = p->bias.stride_a; k.bias_sn = p->bias.stride_n;
     k.mask = p->mask.ptr; k.mask_sw = p->mask.stride_a; k.mask_sn = p->mask.stride_n;
-    k.mask_live = p->mask.ptr ? p->mask_live : nullptr;
+    // the kernels keep the per-window flags in LDS; beyond that many windows they go without
+    k.mask_live = (p->mask.ptr && p->n_windows <= fwa2::kLiveCache) ? p->mask_live : nullptr;
     k.lse = p->lse; k.lse_sb = p->lse_stride_bw; k.lse_sh = p->lse_stride_h;
     k.bw = p->bw; k.heads = p->heads; k.n = p->n; k.n_windows = p->mask.ptr ? p->n_windows : 1;
     k.scale_kind = p->scale_kind;
@@ -184,7 +185,8 @@ int fwa2_backward(const fwa2_problem* p) {
     k.logit_scale = p->logit_scale;
     k.bias = p->bias.ptr; k.bias_sh = p->bias.stride_a; k.bias_sn = p->bias.stride_n;
     k.mask = p->mask.ptr; k.mask_sw = p->mask.stride_a; k.mask_sn = p->mask.stride_n;
-    k.mask_live = p->mask.ptr ? p->mask_live : nullptr;
+    // the kernels keep the per-window flags in LDS; beyond that many windows they go without
+    k.mask_live = (p->mask.ptr && p->n_windows <= fwa2::kLiveCache) ? p->mask_live : nullptr;
     k.lse = p->lse; k.lse_sb = p->lse_stride_bw; k.lse_sh = p->lse_stride_h;
     k.bw = p->bw; k.heads = p->heads; k.n = p->n; k.n_windows = p->mask.ptr ? p->n_windows : 1;
     k.scale_kind = p->scale_kind;
