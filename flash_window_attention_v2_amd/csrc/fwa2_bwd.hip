@@ -503,27 +503,29 @@ __global__ void __launch_bounds__(256) transpose_pad_kernel(const T* src, int64_
 }
 
 // dbias[h][q][k] = sum_g part[h][g][k][q]; dscale[h] = gate * sum_g part_dscale[h][g].
+// One workgroup per (32 queries, key row, head): 8 groups of 32 threads each sum every 8th partial
+// tile, then the 8 sums are added in a fixed order, so results are bit-reproducible.
 template <int DT>
 __global__ void __launch_bounds__(256) reduce_kernel(const BwdParams p, int npk, int r, bool has_bias) {
     typedef typename Elem<DT>::E E;
-    __shared__ float tile[8][33];
+    __shared__ float part[8][32];
     const int h = blockIdx.z;
     const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
     if (has_bias) {
-        const int q0 = blockIdx.x * 32, k0 = blockIdx.y * 8;
+        const int q = blockIdx.x * 32 + tx, k = blockIdx.y;
         float acc = 0.f;
-        if (k0 + ty < npk) {
-            const float* src = p.part_dbias + (((int64_t)h * p.db_parts) * npk + k0 + ty) * r + q0 + tx;
-            const int64_t gs = (int64_t)npk * r;
+        const float* src = p.part_dbias + (((int64_t)h * p.db_parts) * npk + k) * r + q;
+        const int64_t gs = (int64_t)npk * r;
 #pragma unroll 4
-            for (int gi = 0; gi < p.db_parts; gi++) acc += src[gi * gs];
-        }
-        tile[ty][tx] = acc;
+        for (int gi = ty; gi < p.db_parts; gi += 8) acc += src[gi * gs];
+        part[ty][tx] = acc;
         __syncthreads();
-        // thread (ty, tx) -> query q0 + (4*ty + tx/8), key k0 + tx%8
-        const int qq = 4 * ty + (tx >> 3), kk = tx & 7;
-        const int q = q0 + qq, k = k0 + kk;
-        if (q < p.n && k < p.n) reinterpret_cast<E*>(p.dbias)[((int64_t)h * p.n + q) * p.n + k] = (E)tile[kk][qq];
+        if (ty == 0 && q < p.n && k < p.n) {
+            float tot = 0.f;
+#pragma unroll
+            for (int j = 0; j < 8; j++) tot += part[j][tx];
+            reinterpret_cast<E*>(p.dbias)[((int64_t)h * p.n + q) * p.n + k] = (E)tot;
+        }
     }
     if (p.scale_kind == FWA2_SCALE_TENSOR && blockIdx.x == 0 && blockIdx.y == 0) {
         float v = 0.f;
@@ -769,7 +771,7 @@ static hipError_t launch_bwd_dt(BwdParams p, bool has_bias, int mask_dt, hipStre
     }
     if (e != hipSuccess) return e;
     if (has_bias || p.scale_kind == FWA2_SCALE_TENSOR) {
-        dim3 gr(has_bias ? pl.r / 32 : 1, has_bias ? (pl.npk + 7) / 8 : 1, p.heads);
+        dim3 gr(has_bias ? pl.r / 32 : 1, has_bias ? pl.npk : 1, p.heads);
         hipLaunchKernelGGL(reduce_kernel<DT>, gr, dim3(256), 0, st, p, pl.npk, pl.r, has_bias);
         e = hipGetLastError();
     }
