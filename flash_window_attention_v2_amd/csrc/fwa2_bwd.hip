@@ -68,7 +68,7 @@ struct BwdLds {
 template <class E>
 __device__ __forceinline__ void async_row_chunk(const E* gsrc, E* lds_wave_base) {
     __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gsrc,
-                                     (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
+                                     (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, kStreamPolicy);
 }
 
 // All query blocks of one unit.  MASKED is uniform per unit (the window's mask is live or not),
@@ -155,7 +155,8 @@ __device__ __forceinline__ void unit_blocks(BwdLds<DT, NQB>& L, WaveRegs<DT, NQB
                 }
 #pragma unroll
                 for (int dt = 0; dt < 2; dt++) {
-                    const int off = (q8 + (l16 >> 2)) * kRow + 16 * dt + 4 * (l16 & 3);
+                    // A row m <-> d = 8 (m / 4) + 4 dt + m % 4: the lane's dk / dv values are d = 8g + 4dt + i
+                    const int off = (q8 + (l16 >> 2)) * kRow + 8 * (l16 & 3) + 4 * dt;
                     const V8 a_do = lds_tr8<DT>(L.dOs + off, L.dOs + off + 4 * kRow);
                     w.dvacc[kt][dt] = Elem<DT>::mfma16(a_do, p8, w.dvacc[kt][dt]);
                     const V8 a_q = lds_tr8<DT>(L.Qs + off, L.Qs + off + 4 * kRow);
@@ -325,7 +326,7 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
         for (int r0 = wave * 64; r0 < N; r0 += 64 * p.waves) {
             if (r0 + lane < N)
                 __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(lseptr + r0 + lane),
-                                                 (__attribute__((address_space(3))) void*)(L.rawLse + r0), 4, 0, 0);
+                                                 (__attribute__((address_space(3))) void*)(L.rawLse + r0), 4, 0, kStreamPolicy);
         }
     };
 
@@ -407,7 +408,7 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
             if (qb == fetch_at && b_next < p.bw) fetch_unit(b_next);
         });
 
-        // ---- epilogue dk, dv: lane (key, g) holds d = 16dt + 4g + i; k_hat and 1/|k| come from LDS ----
+        // ---- epilogue dk, dv: lane (key, g) holds d = 8g + 4dt + i (16 bytes of a row); k_hat and 1/|k| come from LDS ----
 #pragma unroll
         for (int kt = 0; kt < KT; kt++) {
             const int key = key0 + 16 * kt;
@@ -416,7 +417,7 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
             float dot = 0.f;
 #pragma unroll
             for (int dt = 0; dt < 2; dt++) {
-                const V4 k4 = *reinterpret_cast<const V4*>(L.Ks + key * kRow + 16 * dt + 4 * g);
+                const V4 k4 = *reinterpret_cast<const V4*>(L.Ks + key * kRow + 8 * g + 4 * dt);
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     x[4 * dt + i] = (float)k4[i];
@@ -440,23 +441,20 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
                             o4[i] = inv * (a[4 * dt + i] - x[4 * dt + i] * proj);
                             v4[i] = w.dvacc[kt][dt][i];
                         }
-                        *reinterpret_cast<f32x4*>(p.part_dk + row * 32 + 16 * dt + 4 * g) = o4;
-                        *reinterpret_cast<f32x4*>(p.part_dv + row * 32 + 16 * dt + 4 * g) = v4;
+                        *reinterpret_cast<f32x4*>(p.part_dk + row * 32 + 8 * g + 4 * dt) = o4;
+                        *reinterpret_cast<f32x4*>(p.part_dv + row * 32 + 8 * g + 4 * dt) = v4;
                     }
                 } else {
                     E* dkp = reinterpret_cast<E*>(const_cast<void*>(p.dk.ptr)) + b * p.dk.sb + h * p.dk.sh + (int64_t)key * p.dk.sn;
                     E* dvp = reinterpret_cast<E*>(const_cast<void*>(p.dv.ptr)) + b * p.dv.sb + h * p.dv.sh + (int64_t)key * p.dv.sn;
+                    V8 o8, v8;
 #pragma unroll
-                    for (int dt = 0; dt < 2; dt++) {
-                        V4 o4, v4;
-#pragma unroll
-                        for (int i = 0; i < 4; i++) {
-                            o4[i] = (E)(inv * (a[4 * dt + i] - x[4 * dt + i] * proj));
-                            v4[i] = (E)w.dvacc[kt][dt][i];
-                        }
-                        *reinterpret_cast<V4*>(dkp + 16 * dt + 4 * g) = o4;
-                        *reinterpret_cast<V4*>(dvp + 16 * dt + 4 * g) = v4;
+                    for (int j = 0; j < 8; j++) {
+                        o8[j] = (E)(inv * (a[j] - x[j] * proj));
+                        v8[j] = (E)w.dvacc[kt][j >> 2][j & 3];
                     }
+                    st8_stream<V8>(dkp + 8 * g, o8);
+                    st8_stream<V8>(dvp + 8 * g, v8);
                 }
             }
         }
@@ -474,8 +472,8 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
                     f32x4 a, c;
 #pragma unroll
                     for (int j = 0; j < 4; j++) { a[j] = w.dbacc[qb][kt][j]; c[j] = w.dbacc[qb][kt][4 + j]; }
-                    *reinterpret_cast<f32x4*>(dst + 32 * qb + 8 * g) = a;
-                    *reinterpret_cast<f32x4*>(dst + 32 * qb + 8 * g + 4) = c;
+                    __builtin_nontemporal_store(a, reinterpret_cast<f32x4*>(dst + 32 * qb + 8 * g));
+                    __builtin_nontemporal_store(c, reinterpret_cast<f32x4*>(dst + 32 * qb + 8 * g + 4));
                 }
             }
         }

@@ -183,7 +183,7 @@ __global__ void __launch_bounds__(64 * NT / SUB) bwd_dq_resident_kernel(const Bw
     struct Row { float lse[SUB], delta[SUB]; };
     auto dma16 = [&](const E* src, E* lds_wave_base) __attribute__((always_inline)) {
         __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                         (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
+                                         (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, kStreamPolicy);
     };
     auto fetch = [&](int b, Row& r) __attribute__((always_inline)) {
         // lane-derived offsets are re-materialised here: hoisted out of the unit loop they would occupy
@@ -384,7 +384,7 @@ __global__ void __launch_bounds__(64 * NT / SUB) bwd_dq_resident_kernel(const Bw
                 V8 o8;
 #pragma unroll
                 for (int j = 0; j < 8; j++) o8[j] = (E)(f * (dqacc[u][j >> 2][j & 3] - qh[j] * proj));
-                st8<V8>(dqrow + 8 * (ln2 >> 4), o8);
+                st8_stream<V8>(dqrow + 8 * (ln2 >> 4), o8);
                 if (g == 0) ds_acc += dot;
             }
         }

@@ -65,6 +65,10 @@ __device__ __forceinline__ V8 ld8(const E* p) { return *reinterpret_cast<const V
 template <class V8, class E>
 __device__ __forceinline__ void st8(E* p, V8 v) { *reinterpret_cast<V8*>(p) = v; }
 
+// 16-byte store of an output row chunk that nobody re-reads soon: non-temporal, like the row fetches.
+template <class V8, class E>
+__device__ __forceinline__ void st8_stream(E* p, V8 v) { __builtin_nontemporal_store(v, reinterpret_cast<V8*>(p)); }
+
 template <class V8>
 __device__ __forceinline__ V8 zero8() {
     V8 z;
@@ -189,6 +193,10 @@ __device__ __forceinline__ auto load_raw8(const T* row, int c0, int n, float pad
     }
     return v;
 }
+
+// Cache policy of the streaming q / k / v / dO / o row fetches: non-temporal, so that rows read once do
+// not push the bias / mask tables (re-read by every unit) out of the L2.
+constexpr int kStreamPolicy = 2;
 
 constexpr int kKeyChunk = 256;   // keys staged in LDS at a time by the query-owning kernels
 constexpr int kLdsStride = 40;   // elements per staged row (32 + 8 pad): 80-byte rows

@@ -179,9 +179,9 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
             const E* kp = reinterpret_cast<const E*>(p.k.ptr) + b * p.k.sb + h * p.k.sh + (int64_t)frow * p.k.sn + fc8;
             const E* vp = reinterpret_cast<const E*>(p.v.ptr) + b * p.v.sb + h * p.v.sh + (int64_t)frow * p.v.sn + fc8;
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)kp,
-                                             (__attribute__((address_space(3))) void*)(lds_rawK + wave * 16 * 32), 16, 0, 0);
+                                             (__attribute__((address_space(3))) void*)(lds_rawK + wave * 16 * 32), 16, 0, kStreamPolicy);
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)vp,
-                                             (__attribute__((address_space(3))) void*)(lds_rawV + wave * 16 * 32), 16, 0, 0);
+                                             (__attribute__((address_space(3))) void*)(lds_rawV + wave * 16 * 32), 16, 0, kStreamPolicy);
         }
         qq = zero8<V8>();
         if (qv) qq = ld8<V8>(reinterpret_cast<const E*>(p.q.ptr) + b * p.q.sb + h * p.q.sh + (int64_t)qi * p.q.sn + 8 * g);
@@ -287,7 +287,8 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
             if (sum_by_mfma) lacc = Elem<DT>::mfma16(ones, bp, lacc);
 #pragma unroll
             for (int dt = 0; dt < 2; dt++) {
-                const E* vlo = Vb + (32 * kp + 8 * g + (l16 >> 2)) * S + 16 * dt + 4 * (l16 & 3);
+                // A row m <-> d = 8 (m / 4) + 4 dt + m % 4: this lane's accumulators hold d = 8g + 4dt + i
+                const E* vlo = Vb + (32 * kp + 8 * g + (l16 >> 2)) * S + 8 * (l16 & 3) + 4 * dt;
                 const V8 av = lds_tr8<DT>(vlo, vlo + 4 * S);
                 oacc[dt] = Elem<DT>::mfma16(av, bp, oacc[dt]);
             }
@@ -358,13 +359,10 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
         const float inv_l = l_tot > 0.f ? 1.0f / l_tot : 0.f;
         if (qv) {
             E* orow = reinterpret_cast<E*>(const_cast<void*>(p.o.ptr)) + b * p.o.sb + h * p.o.sh + (int64_t)qi * p.o.sn;
+            V8 ov;
 #pragma unroll
-            for (int dt = 0; dt < 2; dt++) {
-                V4 ov;
-#pragma unroll
-                for (int i = 0; i < 4; i++) ov[i] = (E)(oacc[dt][i] * inv_l);
-                *reinterpret_cast<V4*>(orow + 16 * dt + 4 * g) = ov;
-            }
+            for (int j = 0; j < 8; j++) ov[j] = (E)(oacc[j >> 2][j & 3] * inv_l);
+            st8_stream<V8>(orow + 8 * g, ov);
             if (g == 0) {
                 const float lse = l_tot > 0.f ? (m_fixed + m_run + fast_log2(l_tot)) * kLn2 : -INFINITY;
                 p.lse[b * p.lse_sb + h * p.lse_sh + qi] = lse;
