@@ -87,94 +87,129 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
     const bool qv = qi < N;
     const int qc = min(qi, N - 1);
 
-    // ---- resident bias, log2 domain.  Keys are taken 32 at a time; of such a group this lane holds
+    // ---- resident tile, log2 domain.  Keys are taken 32 at a time; of such a group this lane holds
     // keys 8g .. 8g+7: acc0[2kp][i] <-> key 32kp + 8g + i, acc0[2kp+1][i] <-> key 32kp + 8g + 4 + i
-    // (so bias and mask rows are read 8 consecutive entries at a time) ----
+    // (so bias and mask rows are read 8 consecutive entries at a time).  The tile holds
+    // (bias + mask) * log2e - m_fixed, m_fixed = s log2e + max_j (bias2 + mask2)[j] being an upper bound
+    // of every logit of the row; the key that attains the maximum scores at least m_fixed - 2 s log2e. ----
     f32x4 acc0[NT];
-    float mb = 0.f, mn = 0.f;
-    if (HAS_BIAS) {
-        const E* brow = reinterpret_cast<const E*>(p.bias) + h * p.bias_sh + (int64_t)qc * p.bias_sn;
-        mb = -INFINITY;
-        mn = INFINITY;
+    float m_fixed = 0.f;
+    auto build_tile = [&](int w) __attribute__((always_inline)) {
+        const E* brow = nullptr;
+        const ME* mrow = nullptr;
+        if (HAS_BIAS) brow = reinterpret_cast<const E*>(p.bias) + h * p.bias_sh + (int64_t)qc * p.bias_sn;
+        if (MASKED) mrow = reinterpret_cast<const ME*>(p.mask) + w * p.mask_sw + (int64_t)qc * p.mask_sn;
+        float mb = -INFINITY;
 #pragma unroll
         for (int kp = 0; kp < NT / 2; kp++) {
-            const auto raw = load_raw8<VEC, E>(brow, 32 * kp + 8 * g, N, -INFINITY);
+            float v[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) v[j] = (32 * kp + 8 * g + j < N) ? 0.f : -INFINITY;
+            if (HAS_BIAS) {
+                const auto raw = load_raw8<VEC, E>(brow, 32 * kp + 8 * g, N, 0.f);
+#pragma unroll
+                for (int j = 0; j < 8; j++) v[j] += (float)raw[j] * kLog2e;
+            }
+            if (MASKED) {
+                const auto raw = load_raw8<VEC, ME>(mrow, 32 * kp + 8 * g, N, 0.f);
+#pragma unroll
+                for (int j = 0; j < 8; j++) v[j] = fmaf((float)raw[j], kLog2e, v[j]);
+            }
 #pragma unroll
             for (int j = 0; j < 8; j++) {
-                const float v = (float)raw[j] * kLog2e;      // -inf stays -inf
-                acc0[2 * kp + (j >> 2)][j & 3] = v;
-                mb = fmaxf(mb, v);
-                mn = fminf(mn, (32 * kp + 8 * g + j < N) ? v : INFINITY);
+                acc0[2 * kp + (j >> 2)][j & 3] = v[j];
+                mb = fmaxf(mb, v[j]);
             }
         }
         mb = col_max(mb);
-        mn = -col_max(-mn);
-        if (!(mb > -INFINITY)) { mb = 0.f; mn = 0.f; }   // a row of -inf bias: nothing to bound
-    } else {
+        if (!(mb > -INFINITY)) mb = 0.f;        // every key of the row removed: nothing to bound
+        m_fixed = mb + scale2;
 #pragma unroll
         for (int kt = 0; kt < NT; kt++)
 #pragma unroll
-            for (int i = 0; i < 4; i++)
-                acc0[kt][i] = (32 * (kt >> 1) + 8 * g + 4 * (kt & 1) + i < N) ? 0.f : -INFINITY;
-    }
-    const float m_fixed = mb + scale2;     // upper bound of every logit of this row (mask <= 0)
-#pragma unroll
-    for (int kt = 0; kt < NT; kt++)
-#pragma unroll
-        for (int i = 0; i < 4; i++) acc0[kt][i] -= m_fixed;
-    // the wavefront takes the maximum-free path if the bound is tight enough for all its rows
-    float range = (mb - mn == mb - mn) ? mb - mn : INFINITY;   // NaN / inf ranges disable it
-#pragma unroll
-    for (int off = 8; off >= 1; off >>= 1) range = fmaxf(range, __shfl_xor(range, off));
-    const bool wave_fast = (DT == FWA2_BF16) && (2.f * scale2 + range <= kGapLimit);
+            for (int i = 0; i < 4; i++) acc0[kt][i] -= m_fixed;
+    };
+    // the maximum-free softmax is used when the row bound cannot be further than this from the
+    // largest logit (the same for every row of the head)
+    const bool fast = (DT == FWA2_BF16) && (2.f * scale2 <= kGapLimit);
 
-    // ---- which units belong to this launch.  With cached flags the windows of this launch's class
-    // (mask live or not) are listed once, and the units are dealt out by their rank within the
-    // class, so every workgroup of the head gets the same number of them whatever the pattern of
-    // masked windows. ----
-    const bool listed = MASK_DT >= 0 && p.mask_live && p.n_windows <= kLiveCache;
+    // ---- which units belong to this launch.  With the mask flags at hand the windows of this
+    // launch's class (mask live or not) are listed once.
+    //   plain launch: the units of the listed windows (all units without a mask) are dealt out by
+    //     their rank, so every workgroup of the head gets the same number of them;
+    //   MASKED launch: the head's workgroups are dealt out over the listed windows (several per
+    //     window, which then share its images, or several windows per workgroup in turn), and the
+    //     tile is rebuilt with the window's mask whenever a workgroup moves on to another window. ----
+    const int nw = MASK_DT >= 0 ? p.n_windows : 1;
+    const bool listed = MASK_DT >= 0 && p.mask_live != nullptr;      // the host drops the flags beyond kLiveCache
     if (listed) {
-        for (int i = tid; i < p.n_windows; i += nthreads) lds_live[i] = p.mask_live[i];
+        for (int i = tid; i < nw; i += nthreads) lds_live[i] = p.mask_live[i];
         __syncthreads();
         if (wave == 0) {
-            int cnt = 0;
-            for (int base = 0; base < p.n_windows; base += 64) {
+            int c = 0;
+            for (int base = 0; base < nw; base += 64) {
                 const int w = base + lane;
-                const bool in = w < p.n_windows && ((lds_live[w] != 0) == MASKED);
+                const bool in = w < nw && ((lds_live[w] != 0) == MASKED);
                 const unsigned long long bal = __ballot(in);
-                if (in) lds_list[cnt + __popcll(bal & ((1ull << lane) - 1ull))] = (uint16_t)w;
-                cnt += __popcll(bal);
+                if (in) lds_list[c + __popcll(bal & ((1ull << lane) - 1ull))] = (uint16_t)w;
+                c += __popcll(bal);
             }
-            if (lane == 0) lds_count = cnt;
+            if (lane == 0) lds_count = c;
         }
         __syncthreads();
     }
-    const int cnt = listed ? lds_count : 0;
-    const int total = listed ? ((p.bw + p.n_windows - 1) / p.n_windows) * cnt : p.bw;   // ranks to deal out
-    auto unit_of = [&](int t) -> int {
-        if (!listed) return t;
-        const int img = t / cnt;
-        // the same for every lane: keep it (and the addresses derived from it) in scalar registers
-        return __builtin_amdgcn_readfirstlane(img * p.n_windows + (int)lds_list[t - img * cnt]);
+    const int cnt = listed ? __builtin_amdgcn_readfirstlane(lds_count) : nw;    // windows of this class
+    const int n_img = p.bw / nw;
+    auto window_at = [&](int wi) -> int {
+        return listed ? __builtin_amdgcn_readfirstlane((int)lds_list[wi]) : wi;
     };
-    auto flags_of = [&](int b) -> int {
-        const int w = b % p.n_windows;
-        return __builtin_amdgcn_readfirstlane(listed ? (int)lds_live[w] : (int)p.mask_live[w]);
-    };
-    // first rank >= t (in steps of the group count) that names an existing unit of this launch
-    auto rank_from = [&](int t) -> int {
-        for (; t < total; t += p.groups) {
-            const int b = unit_of(t);
-            if (b >= p.bw) continue;
-            if (listed || MASK_DT < 0 || !p.mask_live || ((flags_of(b) != 0) == MASKED)) return t;
+    // A cursor names one unit: (wi, img) = (index into the class's windows, image).
+    //   plain:  rank t = img * cnt + wi walks t = grp, grp + groups, ...
+    //   MASKED: wi = wi0, wi0 + wi_step, ... and for each, img = img0, img0 + img_step, ...
+    int wi_step = 1, img0 = 0, img_step = 1, wi0 = grp;
+    if (MASKED) {
+        if (p.groups >= cnt && cnt > 0) {
+            const int per = p.groups / cnt;       // workgroups per window
+            wi0 = grp / per;                      // (>= cnt for the few left over: they idle)
+            img0 = grp - wi0 * per;
+            img_step = per;
+            wi_step = cnt;                        // one window only
+        } else {
+            wi_step = p.groups;
         }
-        return total;
+    }
+    struct Cursor { int wi, img; };
+    auto valid = [&](const Cursor& c) -> bool { return MASKED ? c.wi < cnt : c.img < n_img; };
+    auto first = [&]() -> Cursor {
+        Cursor c;
+        if (MASKED) { c.wi = wi0; c.img = img0; if (img0 >= n_img) c.wi = cnt; }
+        else { c.img = cnt > 0 ? grp / cnt : n_img; c.wi = cnt > 0 ? grp - c.img * cnt : 0; }
+        return c;
     };
+    auto next = [&](Cursor c) -> Cursor {
+        if (MASKED) {
+            c.img += img_step;
+            if (c.img >= n_img) { c.img = img0; c.wi += wi_step; }
+        } else {
+            const int t = c.img * cnt + c.wi + p.groups;
+            c.img = t / cnt;
+            c.wi = t - c.img * cnt;
+        }
+        return c;
+    };
+    auto unit_of = [&](const Cursor& c) -> int { return c.img * nw + window_at(c.wi); };
+
     // ---- per-unit fetch: every wavefront brings in the 16 K and V rows it will stage (lane i lands
     // at 16 i bytes from the wavefront's base) and its own 16 query rows ----
     const int frow = wave * 16 + (lane >> 2);      // K / V row of this lane
     const int fc8 = (lane & 3) * 8;
     auto fetch = [&](int b, V8& qq) __attribute__((always_inline)) {
+        // lane-derived offsets are re-materialised here: hoisted out of the unit loop they would be
+        // spilled, and the reload would sit in front of every fetch
+        int ln = lane;
+        asm volatile("" : "+v"(ln));
+        const int frow = wave * 16 + (ln >> 2);
+        const int fc8 = (ln & 3) * 8;
         if (frow < N) {
             const E* kp = reinterpret_cast<const E*>(p.k.ptr) + b * p.k.sb + h * p.k.sh + (int64_t)frow * p.k.sn + fc8;
             const E* vp = reinterpret_cast<const E*>(p.v.ptr) + b * p.v.sb + h * p.v.sh + (int64_t)frow * p.v.sn + fc8;
@@ -184,7 +219,8 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
                                              (__attribute__((address_space(3))) void*)(lds_rawV + wave * 16 * 32), 16, 0, kStreamPolicy);
         }
         qq = zero8<V8>();
-        if (qv) qq = ld8<V8>(reinterpret_cast<const E*>(p.q.ptr) + b * p.q.sb + h * p.q.sh + (int64_t)qi * p.q.sn + 8 * g);
+        const int fq = wave * 16 + (ln & 15);
+        if (fq < N) qq = ld8<V8>(reinterpret_cast<const E*>(p.q.ptr) + b * p.q.sb + h * p.q.sh + (int64_t)fq * p.q.sn + 8 * (ln >> 4));
     };
     // landing area -> tiles: K normalised and rounded to fp16, V as is (rows >= n stay zero)
     auto stage = [&](int buf) __attribute__((always_inline)) {
@@ -206,19 +242,25 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
     };
 
     __syncthreads();                       // zero fill done
-    int t = rank_from(grp);
+    Cursor c = first();
     V8 qq = zero8<V8>();
-    if (t < total) {
-        fetch(unit_of(t), qq);
+    int tile_wi = -1;                      // window index the resident tile was built for
+    if (!MASKED) build_tile(0);
+    if (valid(c)) {
+        fetch(unit_of(c), qq);
         stage(0);
     }
     __syncthreads();
     int cur = 0;
 
-    while (t < total) {
-        const int b = unit_of(t);
-        const int tn = rank_from(t + p.groups);
-        const int bn = tn < total ? unit_of(tn) : p.bw;
+    while (valid(c)) {
+        const int b = unit_of(c);
+        const Cursor cn = next(c);
+        const bool more = valid(cn);
+        if (MASKED && c.wi != tile_wi) {
+            build_tile(window_at(c.wi));
+            tile_wi = c.wi;
+        }
         // ---- Q operand: normalise, fold s log2e, round to fp16 ----
         SV8 bq;
         {
@@ -232,16 +274,7 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
 #pragma unroll
             for (int j = 0; j < 8; j++) bq[j] = (SE)(x[j] * sc);
         }
-        if (bn < p.bw) fetch(bn, qq);      // in flight while this unit is computed
-
-        const ME* mrow = nullptr;
-        constexpr bool masked = MASKED;
-        bool safe = false;
-        if (MASKED) {
-            const int w = b % p.n_windows;
-            safe = p.mask_live ? (flags_of(b) & 2) != 0 : false;
-            mrow = reinterpret_cast<const ME*>(p.mask) + w * p.mask_sw + (int64_t)qc * p.mask_sn;
-        }
+        if (more) fetch(unit_of(cn), qq);      // in flight while this unit is computed
 
         const SE* Kb = &lds_K[cur][0];
         const E* Vb = &lds_V[cur][0];
@@ -252,24 +285,15 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
             for (int i = 0; i < 4; i++) oacc[dt][i] = 0.f;
         float l_run = 0.f;     // online path: this lane's share of the running row sum
         float m_run = 0.f;     // online path: running maximum relative to m_fixed
-        bool fast_unit = false;
 
-        typedef ME MV8 __attribute__((ext_vector_type(8)));
         // scores of keys 32 kp .. 32 kp + 31: MFMA tile A holds keys 8r/4 + r%4 in its rows r, tile B
         // the keys 4 further on, so that this lane's 8 values are keys 8g .. 8g+7 of the group
-        auto scores = [&](int kp, bool with_mask, const MV8& mk, f32x4& s0, f32x4& s1) __attribute__((always_inline)) {
+        auto scores = [&](int kp, f32x4& s0, f32x4& s1) __attribute__((always_inline)) {
             const int krow = 32 * kp + 8 * (l16 >> 2) + (l16 & 3);
             const SV8 a0 = ld8<SV8>(Kb + krow * S + 8 * g);
             const SV8 a1 = ld8<SV8>(Kb + (krow + 4) * S + 8 * g);
             s0 = Elem<kScoreDT>::mfma16(a0, bq, acc0[2 * kp]);
             s1 = Elem<kScoreDT>::mfma16(a1, bq, acc0[2 * kp + 1]);
-            if (MASK_DT >= 0 && with_mask) {
-#pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    s0[i] = fmaf((float)mk[i], kLog2e, s0[i]);
-                    s1[i] = fmaf((float)mk[4 + i], kLog2e, s1[i]);
-                }
-            }
         };
         // FAST: the row sum comes out of a third MFMA against a tile of ones, i.e. it sums the
         // ROUNDED P~ values that also enter the product with V: o is then an exact convex
@@ -294,41 +318,27 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
             }
         };
 
-        if (wave_fast && (!masked || safe)) {
-            fast_unit = true;
-            auto body = [&](bool with_mask) __attribute__((always_inline)) {
-                // mask rows travel two key groups ahead of their use
-                MV8 mq[2];
-                if (MASK_DT >= 0 && with_mask) {
-                    mq[0] = load_raw8<VEC, ME>(mrow, 8 * g, N, 0.f);
-                    mq[1] = load_raw8<VEC, ME>(mrow, 32 + 8 * g, N, 0.f);
-                }
+        if (fast) {
 #pragma unroll
-                for (int kp = 0; kp < NT / 2; kp++) {
-                    if (32 * kp < N) {
-                        f32x4 s0, s1;
-                        scores(kp, with_mask, mq[kp & 1], s0, s1);
-                        if (MASK_DT >= 0 && with_mask && kp + 2 < NT / 2)
-                            mq[kp & 1] = load_raw8<VEC, ME>(mrow, 32 * (kp + 2) + 8 * g, N, 0.f);
+            for (int kp = 0; kp < NT / 2; kp++) {
+                if (32 * kp < N) {
+                    f32x4 s0, s1;
+                    scores(kp, s0, s1);
 #pragma unroll
-                        for (int i = 0; i < 4; i++) {
-                            s0[i] = fast_exp2(s0[i]);
-                            s1[i] = fast_exp2(s1[i]);
-                        }
-                        pv(kp, s0, s1, true);
+                    for (int i = 0; i < 4; i++) {
+                        s0[i] = fast_exp2(s0[i]);
+                        s1[i] = fast_exp2(s1[i]);
                     }
+                    pv(kp, s0, s1, true);
                 }
-            };
-            body(MASKED);
+            }
         } else {
             m_run = -INFINITY;
 #pragma unroll
             for (int kp = 0; kp < NT / 2; kp++) {
                 if (32 * kp < N) {
                     f32x4 s0, s1;
-                    MV8 mk;
-                    if (MASK_DT >= 0 && masked) mk = load_raw8<VEC, ME>(mrow, 32 * kp + 8 * g, N, 0.f);
-                    scores(kp, masked, mk, s0, s1);
+                    scores(kp, s0, s1);
                     float bm = fmaxf(fmaxf(s0[0], s0[1]), fmaxf(s0[2], s0[3]));
                     bm = fmaxf(bm, fmaxf(fmaxf(s1[0], s1[1]), fmaxf(s1[2], s1[3])));
                     bm = col_max(bm);
@@ -353,25 +363,28 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
             }
         }
 
-        if (bn < p.bw) stage(cur ^ 1);     // before the stores below, so the wait covers only the fetch
+        if (more) stage(cur ^ 1);     // before the stores below, so the wait covers only the fetch
         // ---- normalise, write o (input dtype) and lse (natural log, fp32) ----
-        const float l_tot = fast_unit ? lacc[0] : col_add(l_run);
+        const float l_tot = fast ? lacc[0] : col_add(l_run);
         const float inv_l = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+        int ln2 = lane;
+        asm volatile("" : "+v"(ln2));
+        const int oq = wave * 16 + (ln2 & 15);
         if (qv) {
-            E* orow = reinterpret_cast<E*>(const_cast<void*>(p.o.ptr)) + b * p.o.sb + h * p.o.sh + (int64_t)qi * p.o.sn;
+            E* orow = reinterpret_cast<E*>(const_cast<void*>(p.o.ptr)) + b * p.o.sb + h * p.o.sh + (int64_t)oq * p.o.sn;
             V8 ov;
 #pragma unroll
             for (int j = 0; j < 8; j++) ov[j] = (E)(oacc[j >> 2][j & 3] * inv_l);
             st8_stream<V8>(orow + 8 * g, ov);
             if (g == 0) {
                 const float lse = l_tot > 0.f ? (m_fixed + m_run + fast_log2(l_tot)) * kLn2 : -INFINITY;
-                p.lse[b * p.lse_sb + h * p.lse_sh + qi] = lse;
+                p.lse[b * p.lse_sb + h * p.lse_sh + oq] = lse;
             }
         }
 
         __syncthreads();       // next unit staged; everybody is done with the current buffers
         cur ^= 1;
-        t = tn;
+        c = cn;
     }
 }
 
