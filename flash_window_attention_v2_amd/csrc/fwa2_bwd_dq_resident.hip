@@ -94,89 +94,111 @@ __global__ void __launch_bounds__(64 * NT / SUB) bwd_dq_resident_kernel(const Bw
         qc[u] = min(qi[u], N - 1);
     }
 
-    // ---- resident bias (see fwa2_fwd_resident.hip): acc0[2kp][i] <-> key 32kp + 8g + i,
-    // acc0[2kp+1][i] <-> key 32kp + 8g + 4 + i, log2 domain, minus the row bound ----
+    // ---- resident tile (see fwa2_fwd_resident.hip): acc0[u][2kp][i] <-> key 32kp + 8g + i,
+    // acc0[u][2kp+1][i] <-> key 32kp + 8g + 4 + i of query tile u; (bias + mask) * log2e minus the
+    // row bound m_fixed = s log2e + max_j (bias2 + mask2)[j] ----
     f32x4 acc0[SUB][NT];
     float m_fixed[SUB];
-    float range = 0.f;
+    auto build_tile = [&](int w) __attribute__((always_inline)) {
 #pragma unroll
-    for (int u = 0; u < SUB; u++) {
-        float mb = 0.f, mn = 0.f;
-        if (HAS_BIAS) {
-            const E* brow = reinterpret_cast<const E*>(p.bias) + h * p.bias_sh + (int64_t)qc[u] * p.bias_sn;
-            mb = -INFINITY;
-            mn = INFINITY;
+        for (int u = 0; u < SUB; u++) {
+            const E* brow = nullptr;
+            const ME* mrow = nullptr;
+            if (HAS_BIAS) brow = reinterpret_cast<const E*>(p.bias) + h * p.bias_sh + (int64_t)qc[u] * p.bias_sn;
+            if (MASKED) mrow = reinterpret_cast<const ME*>(p.mask) + w * p.mask_sw + (int64_t)qc[u] * p.mask_sn;
+            float mb = -INFINITY;
 #pragma unroll
             for (int kp = 0; kp < NT / 2; kp++) {
-                const auto raw = load_raw8<VEC, E>(brow, 32 * kp + 8 * g, N, -INFINITY);
+                float v[8];
+#pragma unroll
+                for (int j = 0; j < 8; j++) v[j] = (32 * kp + 8 * g + j < N) ? 0.f : -INFINITY;
+                if (HAS_BIAS) {
+                    const auto raw = load_raw8<VEC, E>(brow, 32 * kp + 8 * g, N, 0.f);
+#pragma unroll
+                    for (int j = 0; j < 8; j++) v[j] += (float)raw[j] * kLog2e;
+                }
+                if (MASKED) {
+                    const auto raw = load_raw8<VEC, ME>(mrow, 32 * kp + 8 * g, N, 0.f);
+#pragma unroll
+                    for (int j = 0; j < 8; j++) v[j] = fmaf((float)raw[j], kLog2e, v[j]);
+                }
 #pragma unroll
                 for (int j = 0; j < 8; j++) {
-                    const float v = (float)raw[j] * kLog2e;
-                    acc0[u][2 * kp + (j >> 2)][j & 3] = v;
-                    mb = fmaxf(mb, v);
-                    mn = fminf(mn, (32 * kp + 8 * g + j < N) ? v : INFINITY);
+                    acc0[u][2 * kp + (j >> 2)][j & 3] = v[j];
+                    mb = fmaxf(mb, v[j]);
                 }
             }
             mb = col_max(mb);
-            mn = -col_max(-mn);
-            if (!(mb > -INFINITY)) { mb = 0.f; mn = 0.f; }
-        } else {
+            if (!(mb > -INFINITY)) mb = 0.f;        // every key of the row removed: nothing to bound
+            m_fixed[u] = mb + scale2;
 #pragma unroll
             for (int kt = 0; kt < NT; kt++)
 #pragma unroll
-                for (int i = 0; i < 4; i++)
-                    acc0[u][kt][i] = (32 * (kt >> 1) + 8 * g + 4 * (kt & 1) + i < N) ? 0.f : -INFINITY;
+                for (int i = 0; i < 4; i++) acc0[u][kt][i] -= m_fixed[u];
         }
-        m_fixed[u] = mb + scale2;
-#pragma unroll
-        for (int kt = 0; kt < NT; kt++)
-#pragma unroll
-            for (int i = 0; i < 4; i++) acc0[u][kt][i] -= m_fixed[u];
-        const float r = (mb - mn == mb - mn) ? mb - mn : INFINITY;
-        range = fmaxf(range, r);
-    }
-#pragma unroll
-    for (int off = 8; off >= 1; off >>= 1) range = fmaxf(range, __shfl_xor(range, off));
-    // w = 2^(m - lse2) may be folded into dO when it cannot leave the bf16 range
-    const bool wave_fold = (DT == FWA2_BF16) && (2.f * scale2 + range <= kGapLimit);
+    };
+    // w = 2^(m - lse2) lies in [1/N, 2^(2 s log2e)]: it may be folded into dO when that cannot leave
+    // the bf16 range
+    const bool fold = (DT == FWA2_BF16) && (2.f * scale2 <= kGapLimit);
 
-    // ---- units of this launch, dealt out by rank within their mask class ----
-    const bool listed = MASK_DT >= 0 && p.mask_live && p.n_windows <= kLiveCache;
+    // ---- which units belong to this launch (same dealing as in fwa2_fwd_resident.hip): the plain
+    // launch deals the units of the unmasked windows out by rank; the MASKED launch deals the head's
+    // workgroups out over the masked windows and rebuilds the tile per window ----
+    const int nw = MASK_DT >= 0 ? p.n_windows : 1;
+    const bool listed = MASK_DT >= 0 && p.mask_live != nullptr;      // the host drops the flags beyond kLiveCache
     if (listed) {
-        for (int i = tid; i < p.n_windows; i += nthreads) lds_live[i] = p.mask_live[i];
+        for (int i = tid; i < nw; i += nthreads) lds_live[i] = p.mask_live[i];
         __syncthreads();
         if (wave == 0) {
-            int cnt = 0;
-            for (int base = 0; base < p.n_windows; base += 64) {
+            int c = 0;
+            for (int base = 0; base < nw; base += 64) {
                 const int w = base + lane;
-                const bool in = w < p.n_windows && ((lds_live[w] != 0) == MASKED);
+                const bool in = w < nw && ((lds_live[w] != 0) == MASKED);
                 const unsigned long long bal = __ballot(in);
-                if (in) lds_list[cnt + __popcll(bal & ((1ull << lane) - 1ull))] = (uint16_t)w;
-                cnt += __popcll(bal);
+                if (in) lds_list[c + __popcll(bal & ((1ull << lane) - 1ull))] = (uint16_t)w;
+                c += __popcll(bal);
             }
-            if (lane == 0) lds_count = cnt;
+            if (lane == 0) lds_count = c;
         }
         __syncthreads();
     }
-    const int cnt = listed ? lds_count : 0;
-    const int total = listed ? ((p.bw + p.n_windows - 1) / p.n_windows) * cnt : p.bw;
-    auto unit_of = [&](int t) -> int {
-        if (!listed) return t;
-        const int img = t / cnt;
-        return __builtin_amdgcn_readfirstlane(img * p.n_windows + (int)lds_list[t - img * cnt]);
+    const int cnt = listed ? __builtin_amdgcn_readfirstlane(lds_count) : nw;    // windows of this class
+    const int n_img = p.bw / nw;
+    auto window_at = [&](int wi) -> int {
+        return listed ? __builtin_amdgcn_readfirstlane((int)lds_list[wi]) : wi;
     };
-    auto flags_of = [&](int b) -> int {
-        const int w = b % p.n_windows;
-        return __builtin_amdgcn_readfirstlane(listed ? (int)lds_live[w] : (int)p.mask_live[w]);
-    };
-    auto rank_from = [&](int t) -> int {
-        for (; t < total; t += groups) {
-            const int b = unit_of(t);
-            if (b >= p.bw) continue;
-            if (listed || MASK_DT < 0 || !p.mask_live || ((flags_of(b) != 0) == MASKED)) return t;
+    int wi_step = 1, img0 = 0, img_step = 1, wi0 = grp;
+    if (MASKED) {
+        if (groups >= cnt && cnt > 0) {
+            const int per = groups / cnt;         // workgroups per window
+            wi0 = grp / per;                      // (>= cnt for the few left over: they idle)
+            img0 = grp - wi0 * per;
+            img_step = per;
+            wi_step = cnt;                        // one window only
+        } else {
+            wi_step = groups;
         }
-        return total;
+    }
+    struct Cursor { int wi, img; };
+    auto valid = [&](const Cursor& c) -> bool { return MASKED ? c.wi < cnt : c.img < n_img; };
+    auto first = [&]() -> Cursor {
+        Cursor c;
+        if (MASKED) { c.wi = wi0; c.img = img0; if (img0 >= n_img) c.wi = cnt; }
+        else { c.img = cnt > 0 ? grp / cnt : n_img; c.wi = cnt > 0 ? grp - c.img * cnt : 0; }
+        return c;
     };
+    auto next = [&](Cursor c) -> Cursor {
+        if (MASKED) {
+            c.img += img_step;
+            if (c.img >= n_img) { c.img = img0; c.wi += wi_step; }
+        } else {
+            const int t = c.img * cnt + c.wi + groups;
+            c.img = t / cnt;
+            c.wi = t - c.img * cnt;
+        }
+        return c;
+    };
+    auto unit_of = [&](const Cursor& c) -> int { return c.img * nw + window_at(c.wi); };
 
     // ---- per-unit fetch: the wavefront's WR rows of k, v (which it will stage) and of q, dO (its own
     // queries) by DMA, 16 rows per instruction; lse and delta of its queries in registers ----
@@ -237,35 +259,28 @@ __global__ void __launch_bounds__(64 * NT / SUB) bwd_dq_resident_kernel(const Bw
     };
 
     __syncthreads();
-    int t = rank_from(grp);
+    Cursor c = first();
+    int tile_wi = -1;                      // window index the resident tile was built for
+    if (!MASKED) build_tile(0);
     Row row;
 #pragma unroll
     for (int u = 0; u < SUB; u++) { row.lse[u] = -INFINITY; row.delta[u] = 0.f; }
-    if (t < total) {
-        fetch(unit_of(t), row);
+    if (valid(c)) {
+        fetch(unit_of(c), row);
         stage(0);
     }
     __syncthreads();
     int cur = 0;
     float ds_acc = 0.f;        // sum over this lane's queries of q_hat . dq_hat
 
-    while (t < total) {
-        const int b = unit_of(t);
-        const int tn = rank_from(t + groups);
-        const int bn = tn < total ? unit_of(tn) : p.bw;
-
-        const ME* mrow[SUB];
-        bool safe = false;
-#pragma unroll
-        for (int u = 0; u < SUB; u++) mrow[u] = nullptr;
-        if (MASKED) {
-            const int w = b % p.n_windows;
-            safe = p.mask_live ? (flags_of(b) & 2) != 0 : false;
-#pragma unroll
-            for (int u = 0; u < SUB; u++)
-                mrow[u] = reinterpret_cast<const ME*>(p.mask) + w * p.mask_sw + (int64_t)qc[u] * p.mask_sn;
+    while (valid(c)) {
+        const int b = unit_of(c);
+        const Cursor cn = next(c);
+        const bool more = valid(cn);
+        if (MASKED && c.wi != tile_wi) {
+            build_tile(window_at(c.wi));
+            tile_wi = c.wi;
         }
-        const bool fold = wave_fold && (!MASKED || safe);
 
         // ---- this unit's operands out of the landed rows ----
         SV8 bq[SUB];
@@ -303,12 +318,12 @@ __global__ void __launch_bounds__(64 * NT / SUB) bwd_dq_resident_kernel(const Bw
 #pragma unroll
             for (int i = 0; i < 4; i++) { dqacc[u][0][i] = 0.f; dqacc[u][1][i] = 0.f; ndv[u][i] = nd; }
         }
-        if (bn < p.bw) fetch(bn, row);      // in flight while this unit is computed
+        if (more) fetch(unit_of(cn), row);      // in flight while this unit is computed
 
         const SE* Kb = &lds_K[cur][0];
         const E* Vb = &lds_V[cur][0];
 
-        auto group = [&](int kp, bool folded, const MV8* mk) __attribute__((always_inline)) {
+        auto group = [&](int kp, bool folded) __attribute__((always_inline)) {
             const int krow = 32 * kp + 8 * (l16 >> 2) + (l16 & 3);
             SV8 bz[SUB];
 #pragma unroll
@@ -321,7 +336,6 @@ __global__ void __launch_bounds__(64 * NT / SUB) bwd_dq_resident_kernel(const Bw
                     const f32x4 dp = Elem<DT>::mfma16(av, bd[u], ndv[u]);
 #pragma unroll
                     for (int i = 0; i < 4; i++) {
-                        if (MASKED) s[i] = fmaf((float)mk[u][4 * half + i], kLog2e, s[i]);
                         const float e = folded ? fast_exp2(s[i]) : fast_exp2(s[i] + nl[u]);
                         bz[u][4 * half + i] = (SE)(e * dp[i]);
                     }
@@ -337,29 +351,13 @@ __global__ void __launch_bounds__(64 * NT / SUB) bwd_dq_resident_kernel(const Bw
             }
         };
         auto body = [&](bool folded) __attribute__((always_inline)) {
-            MV8 mq[2][SUB];      // mask rows travel two key groups ahead of their use
-            if (MASKED) {
 #pragma unroll
-                for (int u = 0; u < SUB; u++) {
-                    mq[0][u] = load_raw8<VEC, ME>(mrow[u], 8 * g, N, 0.f);
-                    mq[1][u] = load_raw8<VEC, ME>(mrow[u], 32 + 8 * g, N, 0.f);
-                }
-            }
-#pragma unroll
-            for (int kp = 0; kp < NT / 2; kp++) {
-                if (32 * kp < N) {
-                    group(kp, folded, mq[kp & 1]);
-                    if (MASKED && kp + 2 < NT / 2) {
-#pragma unroll
-                        for (int u = 0; u < SUB; u++)
-                            mq[kp & 1][u] = load_raw8<VEC, ME>(mrow[u], 32 * (kp + 2) + 8 * g, N, 0.f);
-                    }
-                }
-            }
+            for (int kp = 0; kp < NT / 2; kp++)
+                if (32 * kp < N) group(kp, folded);
         };
         if (fold) body(true); else body(false);
 
-        if (bn < p.bw) stage(cur ^ 1);     // before the stores below, so the wait covers only the fetch
+        if (more) stage(cur ^ 1);     // before the stores below, so the wait covers only the fetch
 
         // ---- back through q / max(|q|, eps); q_hat . dq_hat is this row's share of dlogit_scale ----
         // q_hat is taken back from the fp16 score operand (q_hat s log2e), which is live anyway
@@ -391,7 +389,7 @@ __global__ void __launch_bounds__(64 * NT / SUB) bwd_dq_resident_kernel(const Bw
 
         __syncthreads();
         cur ^= 1;
-        t = tn;
+        c = cn;
     }
 
     // ---- dlogit_scale: one partial per workgroup ----
