@@ -406,7 +406,12 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
         const int fetch_at = nqb - 1;
         unit_blocks<DT, HAS_BIAS, ME, NQB, KT, MASKED, BIG>(L, w, bias_t, mask_t, NK, nqb, l16, g, key0, tail_keys, R_tot, [&](int qb) {
             if (qb == fetch_at && b_next < p.bw) fetch_unit(b_next);
+            // The SIMD favours its older wavefront, so the younger one of each pair would finish the
+            // blocks long after it and run the tail alone; raising its priority after the first quarter
+            // lets both reach the end of the unit together.
+            if (qb == NQB / 4 && wave_0 >= (p.waves >> 1)) __builtin_amdgcn_s_setprio(2);
         });
+        __builtin_amdgcn_s_setprio(0);
 
         // ---- epilogue dk, dv: lane (key, g) holds d = 8g + 4dt + i (16 bytes of a row); k_hat and 1/|k| come from LDS ----
 #pragma unroll
