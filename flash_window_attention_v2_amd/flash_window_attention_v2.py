@@ -159,3 +159,76 @@ class FlashWindowAttentionV2(torch.autograd.Function):
             p.stream = torch.cuda.current_stream().cuda_stream
             _abi.check(lib.fwa2_backward(p), "fwa2_backward")
         return dq, dk, dv, dscale, db, None
+
+
+class FlashWindowAttentionV2QKVPacked(torch.autograd.Function):
+    """The same operator fed straight from the qkv projection, for the caller at
+    swin_transformer_v2.py:279-295 of the reference: `qkv` is the GEMM output viewed as
+    [BW, N, 3, H, d]; the result is [BW, N, H, d], so the caller's transpose + reshape to
+    [BW, N, C] is a view.  Backward writes dq, dk and dv into one [BW, N, 3, H, d] buffer,
+    which removes the three zero-fill + strided-copy passes autograd otherwise spends on
+    re-packing separate gradients.  Has no counterpart in the reference, whose kernels
+    take the same strided views but return separate tensors."""
+
+    @staticmethod
+    def forward(ctx, qkv, logit_scale=None, bias=None, mask=None):
+        assert qkv.dim() == 5 and qkv.shape[2] == 3, "qkv must be [BW, N, 3, H, d]"
+        if not (_rows_16b_aligned(qkv) and qkv.is_contiguous()):
+            qkv = qkv.contiguous()
+        q, k, v = (qkv[:, :, i].transpose(1, 2) for i in range(3))       # [BW, H, N, d] views
+        if logit_scale is not None:
+            assert isinstance(logit_scale, torch.Tensor), \
+                "Make sure logit_scale is a tensor if defined in the paramaters."
+            scale_type = "tensor"
+            logit_scale = logit_scale.contiguous()
+        else:
+            scale_type = "scalar"
+            logit_scale = torch.tensor(1.0 / math.sqrt(q.shape[-1]), device=q.device)
+        _check_inputs(q, k, v, logit_scale, bias, mask, scale_type)
+        if bias is not None and bias.stride(-1) != 1:
+            bias = bias.contiguous()
+        if mask is not None and mask.stride(-1) != 1:
+            mask = mask.contiguous()
+
+        bw, heads, n, d = q.shape
+        lib = _abi.load()
+        lse = torch.empty((bw, heads, (n + 63) // 64 * 64), device=q.device, dtype=torch.float32)
+        out = torch.empty((bw, n, heads, d), device=q.device, dtype=q.dtype)
+        mask_live = mask_window_flags(mask) if mask is not None else None
+        p = _describe(q, k, v, out.transpose(1, 2), lse, logit_scale, bias, mask, mask_live, scale_type)
+        with torch.cuda.device(q.device):
+            p.stream = torch.cuda.current_stream().cuda_stream
+            _abi.check(lib.fwa2_forward(p), "fwa2_forward")
+
+        ctx.save_for_backward(qkv, out, lse, logit_scale, bias, mask)
+        ctx.scale_type = scale_type
+        ctx.mask_live = mask_live
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        qkv, out, lse, logit_scale, bias, mask = ctx.saved_tensors
+        scale_type = ctx.scale_type
+        q, k, v = (qkv[:, :, i].transpose(1, 2) for i in range(3))
+        do = dout.transpose(1, 2)                                          # [BW, H, N, d] view
+        if not _rows_16b_aligned(do):
+            do = do.contiguous()
+        dqkv = torch.empty_like(qkv)
+        dq, dk, dv = (dqkv[:, :, i].transpose(1, 2) for i in range(3))
+        dscale = torch.empty_like(logit_scale, memory_format=torch.contiguous_format) if scale_type == "tensor" else None
+        db = torch.empty_like(bias, memory_format=torch.contiguous_format) if bias is not None else None
+
+        lib = _abi.load()
+        p = _describe(q, k, v, out.transpose(1, 2), lse, logit_scale, bias, mask, ctx.mask_live, scale_type)
+        p.d_o, p.dq, p.dk, p.dv = _t4(do), _t4(dq), _t4(dk), _t4(dv)
+        if db is not None:
+            p.dbias = db.data_ptr()
+        if dscale is not None:
+            p.dscale = dscale.data_ptr()
+        with torch.cuda.device(qkv.device):
+            need = lib.fwa2_backward_workspace_bytes(p)
+            ws = torch.empty(max(need, 1), dtype=torch.uint8, device=qkv.device)
+            p.workspace, p.workspace_bytes = ws.data_ptr(), need
+            p.stream = torch.cuda.current_stream().cuda_stream
+            _abi.check(lib.fwa2_backward(p), "fwa2_backward")
+        return dqkv, dscale, db, None

@@ -17,7 +17,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 from torch.utils.checkpoint import checkpoint
 
-from .win_attention_func import flash_win_attn_v2_func, win_attention_torch
+from .win_attention_func import flash_win_attn_v2_func, flash_win_attn_v2_qkvpacked_func, win_attention_torch
 
 
 def _pair(x):
@@ -88,6 +88,10 @@ class WindowAttention(nn.Module):
     """Window multi-head self attention with scaled-cosine scores and a continuous relative
     position bias.  Same arguments as the reference (swin_transformer_v2.py:188-266)."""
 
+    #: feed the fused operator from the packed projection (flash path only); False selects the
+    #: reference's call with three strided views
+    packed_qkv = True
+
     def __init__(self, dim, window_size, num_heads, is_flash=True, qkv_bias=True, attn_drop=0., proj_drop=0.,
                  pretrained_window_size=[0, 0]):
         super().__init__()
@@ -143,15 +147,19 @@ class WindowAttention(nn.Module):
         bias = None
         if self.q_bias is not None:
             bias = torch.cat((self.q_bias, torch.zeros_like(self.v_bias, requires_grad=False), self.v_bias))
-        qkv = F.linear(x, self.qkv.weight, bias).reshape(b_, n, 3, self.num_heads, -1).permute(2, 0, 3, 1, 4)
-        q, k, v = qkv[0], qkv[1], qkv[2]          # strided views, unit inner stride: no copies
-
+        qkv = F.linear(x, self.qkv.weight, bias).reshape(b_, n, 3, self.num_heads, -1)
         rel_bias = self.relative_position_bias()
-        if self.is_flash:
-            out = flash_win_attn_v2_func(q, k, v, self.logit_scale, rel_bias, mask)
+        if self.is_flash and self.packed_qkv:
+            # the kernels read q, k, v out of the GEMM output and write [B_, N, H, d]: no copies either
+            # side, and one packed gradient instead of three that autograd would have to re-pack
+            out = flash_win_attn_v2_qkvpacked_func(qkv, self.logit_scale, rel_bias, mask).reshape(b_, n, c)
         else:
-            out = win_attention_torch(q, k, v, self.logit_scale, rel_bias, mask)
-        out = out.transpose(1, 2).reshape(b_, n, c)
+            q, k, v = qkv.permute(2, 0, 3, 1, 4).unbind(0)      # strided views, unit inner stride
+            if self.is_flash:
+                out = flash_win_attn_v2_func(q, k, v, self.logit_scale, rel_bias, mask)
+            else:
+                out = win_attention_torch(q, k, v, self.logit_scale, rel_bias, mask)
+            out = out.transpose(1, 2).reshape(b_, n, c)
         return self.proj_drop(self.proj(out))
 
     def extra_repr(self):

@@ -6,10 +6,13 @@ import math
 import torch
 import torch.nn.functional as F
 
-from .flash_window_attention_v2 import FlashWindowAttentionV2
+from .flash_window_attention_v2 import FlashWindowAttentionV2, FlashWindowAttentionV2QKVPacked
 
 #: fused forward/backward: (q, k, v, logit_scale=None, bias=None, mask=None) -> o
 flash_win_attn_v2_func = FlashWindowAttentionV2.apply
+#: the same fed from the packed projection: (qkv [BW, N, 3, H, d], logit_scale=None, bias=None, mask=None)
+#: -> o [BW, N, H, d]; the gradient comes back as one packed tensor
+flash_win_attn_v2_qkvpacked_func = FlashWindowAttentionV2QKVPacked.apply
 
 
 def win_attention_torch(q, k, v, logit_scale=None, bias=None, mask=None):

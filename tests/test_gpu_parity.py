@@ -203,6 +203,52 @@ def test_strided_qkv_views_like_swin():
         assert _rel(got[i], ref[name]) <= 5e-2, name
 
 
+def test_packed_qkv_entry_point():
+    """`flash_win_attn_v2_qkvpacked_func` on the [B_, N, 3, H, d] projection output: the same kernels as
+    the three-view call, so o and the packed gradient must be bit-identical to it; both are also held
+    against the classic definition."""
+    from flash_window_attention_v2_amd import flash_win_attn_v2_qkvpacked_func
+    dtype = torch.bfloat16
+    bw, n, h, d = 8, 64, 3, 32
+    g = torch.Generator().manual_seed(5)
+    qkv = torch.randn(bw, n, 3, h, d, generator=g).to(dtype)
+    inp = make_inputs(batch=2, n_windows=4, heads=h, n=n, dtype=dtype, seed=5, resolution=16, window=8, shift=4)
+    q, k, v = qkv.permute(2, 0, 3, 1, 4)
+    ref = classic_fwd_bwd(q, k, v, inp["logit_scale"], inp["bias"], inp["mask"], inp["do"])
+    dev = _to_dev(inp)
+
+    a = qkv.cuda().requires_grad_(True)
+    scale_a = dev["logit_scale"].detach().clone().requires_grad_(True)
+    bias_a = dev["bias"].detach().clone().requires_grad_(True)
+    o_a = flash_win_attn_v2_qkvpacked_func(a, scale_a, bias_a, dev["mask"])
+    assert o_a.shape == (bw, n, h, d) and o_a.is_contiguous()
+    o_a.backward(dev["do"].transpose(1, 2))
+
+    b = qkv.cuda().requires_grad_(True)
+    scale_b = dev["logit_scale"].detach().clone().requires_grad_(True)
+    bias_b = dev["bias"].detach().clone().requires_grad_(True)
+    o_b = _func()(*b.permute(2, 0, 3, 1, 4), scale_b, bias_b, dev["mask"])
+    o_b.backward(dev["do"])
+
+    assert torch.equal(o_a.transpose(1, 2), o_b)
+    assert a.grad.shape == qkv.shape and torch.equal(a.grad, b.grad)
+    assert torch.equal(bias_a.grad, bias_b.grad) and torch.equal(scale_a.grad, scale_b.grad)
+    assert float((o_a.detach().transpose(1, 2).float().cpu() - ref["o"]).abs().max()) <= 2e-2
+    got = a.grad.permute(2, 0, 3, 1, 4)
+    for i, name in enumerate(("dq", "dk", "dv")):
+        assert _rel(got[i], ref[name]) <= 5e-2, name
+    assert _rel(bias_a.grad, ref["dbias"]) <= 5e-2
+
+    # optional arguments absent: default scale, no bias, no mask
+    c = qkv.cuda().requires_grad_(True)
+    o_c = flash_win_attn_v2_qkvpacked_func(c)
+    o_c.backward(dev["do"].transpose(1, 2))
+    ref2 = classic_fwd_bwd(q, k, v, None, None, None, inp["do"])
+    assert float((o_c.detach().transpose(1, 2).float().cpu() - ref2["o"]).abs().max()) <= 2e-2
+    for i, name in enumerate(("dq", "dk", "dv")):
+        assert _rel(c.grad.permute(2, 0, 3, 1, 4)[i], ref2[name]) <= 5e-2, name
+
+
 def test_backward_is_deterministic_and_reentrant():
     inp = make_inputs(batch=4, n_windows=4, heads=3, n=256, dtype=torch.bfloat16, seed=7, resolution=32, window=16, shift=8)
     outs = []

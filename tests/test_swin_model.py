@@ -20,7 +20,7 @@ def test_alias_package_exports():
     import flash_win_attn_v2 as ref_name
     from flash_win_attn_v2.swin_transformer_v2 import WindowAttention as wa
     for name in ("WindowAttention", "SwinTransformerV2", "flash_win_attn_v2_func", "win_attention_torch",
-                 "win_attention_torch_compile"):
+                 "win_attention_torch_compile", "flash_win_attn_v2_qkvpacked_func"):
         assert getattr(ref_name, name) is getattr(fwa, name)
     assert wa is swin.WindowAttention
 
@@ -211,6 +211,12 @@ def test_window_attention_module_gpu(dtype):
     tol = 3e-2 if dtype == torch.bfloat16 else 1e-2
     assert yf.dtype == dtype
     assert rel(yf, yc) < tol
+    # the three-view call of the reference runs the same kernels on the same bytes
+    flash.packed_qkv = False
+    xv = x.to(dtype).requires_grad_()
+    yv = flash(xv, mask)
+    assert torch.equal(yv, yf)
+    del flash.packed_qkv
     assert rel(xf.grad, xc.grad) < tol
     for name in ("qkv.weight", "q_bias", "v_bias", "logit_scale", "cpb_mlp.0.weight", "cpb_mlp.2.weight",
                  "proj.weight"):
