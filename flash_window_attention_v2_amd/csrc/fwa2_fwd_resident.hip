@@ -95,10 +95,16 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
     f32x4 acc0[NT];
     float m_fixed = 0.f;
     auto build_tile = [&](int w) __attribute__((always_inline)) {
+        // lane-derived offsets are re-materialised per call: hoisted out of the unit loop, the row
+        // addresses of every key group would stay alive (and spilled) across all units
+        int ln = lane;
+        if (MASKED) asm volatile("" : "+v"(ln));
+        const int g = ln >> 4;
+        const int qrow = min(wave * 16 + (ln & 15), N - 1);
         const E* brow = nullptr;
         const ME* mrow = nullptr;
-        if (HAS_BIAS) brow = reinterpret_cast<const E*>(p.bias) + h * p.bias_sh + (int64_t)qc * p.bias_sn;
-        if (MASKED) mrow = reinterpret_cast<const ME*>(p.mask) + w * p.mask_sw + (int64_t)qc * p.mask_sn;
+        if (HAS_BIAS) brow = reinterpret_cast<const E*>(p.bias) + h * p.bias_sh + (int64_t)qrow * p.bias_sn;
+        if (MASKED) mrow = reinterpret_cast<const ME*>(p.mask) + w * p.mask_sw + (int64_t)qrow * p.mask_sn;
         float mb = -INFINITY;
 #pragma unroll
         for (int kp = 0; kp < NT / 2; kp++) {
