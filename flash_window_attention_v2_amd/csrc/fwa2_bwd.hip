@@ -63,6 +63,14 @@ struct BwdLds {
     float* rawLse;
 };
 
+// Lane index recomputed on the spot (two VALU instructions, never hoisted): what is derived from it
+// need not stay in a register, or in scratch, across the phases of a unit.
+__device__ __forceinline__ int lane_now() {
+    int l;
+    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(l));
+    return l;
+}
+
 // 16 bytes per lane straight from global memory into LDS (no registers held while in flight):
 // lane i of the wavefront lands at lds_wave_base + 16 i.
 template <class E>
@@ -120,6 +128,8 @@ __device__ __forceinline__ void unit_blocks(BwdLds<DT, NQB>& L, WaveRegs<DT, NQB
 #pragma unroll
             for (int kt = 0; kt < KT; kt++) {
                 V8 p8, z8;
+                // k_hat of the lane's key is re-read per block: 4 registers less per key tile than keeping it
+                const V8 bk_now = ld8<V8>(L.Ks + (key0 + 16 * kt) * kRow + 8 * g);
 #pragma unroll
                 for (int t = 0; t < 2; t++) {
                     const int rowq = 32 * qb + 8 * (l16 >> 2) + 4 * t + (l16 & 3);
@@ -128,7 +138,7 @@ __device__ __forceinline__ void unit_blocks(BwdLds<DT, NQB>& L, WaveRegs<DT, NQB
                     // accumulator inits: -lse*log2e and -delta of this lane's 4 queries
                     const f32x4 nl = *reinterpret_cast<const f32x4*>(L.nlse2 + q8 + 4 * t);
                     const f32x4 nd = *reinterpret_cast<const f32x4*>(L.ndelta + q8 + 4 * t);
-                    f32x4 sacc = Elem<DT>::mfma16(aq, w.bk[kt], nl);          // (S - lse) * log2e
+                    f32x4 sacc = Elem<DT>::mfma16(aq, bk_now, nl);            // (S - lse) * log2e
                     const f32x4 pacc = Elem<DT>::mfma16(ado, w.bv[kt], nd);   // dP - delta
                     if (HAS_BIAS) {   // padded key rows of bias_t hold -inf
 #pragma unroll
@@ -227,9 +237,6 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
     const int lane_0 = tid & 63;
     const int wave_0 = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lane = lane_0, wave = wave_0;
-    const int l16_0 = lane & 15;
-    const int g_0 = lane >> 4;
-    int l16 = l16_0, g = g_0;
 
     float s_true;
     if (p.scale_kind == FWA2_SCALE_TENSOR) {
@@ -240,7 +247,6 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
     }
     const float scale2 = s_true * kLog2e;
 
-    const int key0 = wave * 16 * KT + l16;  // this lane's key in key tile 0 (tile kt: + 16 kt)
     const bool tail_keys = NPk > NK;        // some key columns are padding
 
     WaveRegs<DT, NQB, KT> w;
@@ -250,8 +256,9 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
         for (int kt = 0; kt < KT; kt++)
 #pragma unroll
             for (int j = 0; j < 8; j++) w.dbacc[a][kt][j] = 0.f;
-    const E* bias_t = nullptr;
-    if (HAS_BIAS) bias_t = reinterpret_cast<const E*>(p.bias_t) + ((int64_t)h * NPk_tot + k_off + key0) * R_tot + q_off;
+    // key-major side tables: uniform base of this workgroup's keys; the lane's row is added per unit
+    const E* bias_base = nullptr;
+    if (HAS_BIAS) bias_base = reinterpret_cast<const E*>(p.bias_t) + ((int64_t)h * NPk_tot + k_off) * R_tot + q_off;
 
     // ---- which units belong to this launch.  With the mask flags at hand the windows of this
     // launch's class (mask live or not) are listed once and the units are dealt out by their rank
@@ -303,8 +310,8 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
         const float* lseptr = p.lse + b * p.lse_sb + h * p.lse_sh + q_off;
         // re-materialised here so that no per-row address is computed ahead of time and spilled
         // (a spill reload would wait for every fetch already in flight)
-        int lane = lane_0, wave = wave_0;
-        asm volatile("" : "+v"(lane));
+        const int lane = lane_now();
+        int wave = wave_0;
         asm volatile("" : "+s"(wave));
         const int dc = (lane & 3) * 8;
         for (int row0 = wave * 16; row0 < R; row0 += 16 * p.waves) {   // 16 rows per wavefront and instruction
@@ -344,22 +351,18 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
         const int b = unit_of(t);
         const int t_next = rank_from(t + p.groups);
         const int b_next = t_next < total ? unit_of(t_next) : p.bw;
-        const ME* mask_t = nullptr;
+        const ME* mask_base = nullptr;
         if (MASK_DT >= 0) {
             const int wnd = b % p.n_windows;
-            mask_t = reinterpret_cast<const ME*>(p.mask_t) + ((int64_t)wnd * NPk_tot + k_off + key0) * R_tot + q_off;
+            mask_base = reinterpret_cast<const ME*>(p.mask_t) + ((int64_t)wnd * NPk_tot + k_off) * R_tot + q_off;
         }
-
-        // lane-derived values are re-materialised per unit so that the compiler does not keep
-        // dozens of per-block addresses alive (and spilled) across the whole unit loop
-        l16 = l16_0; g = g_0;
-        asm volatile("" : "+v"(l16), "+v"(g));
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wavefront's share of the unit has landed
         __syncthreads();   // ... and everybody's; the previous unit is done with the tiles
         // ---- landing area -> MFMA tiles: one 8-element chunk of a row per thread and pass ----
         {
-            const int dc = (tid & 3) * 8;
-            for (int r = tid >> 2; r < R; r += nthreads >> 2) {
+            const int st = wave_0 * 64 + lane_now();
+            const int dc = (st & 3) * 8;
+            for (int r = st >> 2; r < R; r += nthreads >> 2) {
                 float xq[8], xk[8], xd[8], xo[8];
                 const V8 do8 = ld8<V8>(L.rawDO + r * 32 + dc);
                 unpack8(ld8<V8>(L.rawQ + r * 32 + dc), xq);
@@ -377,18 +380,25 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
                 st8<V8>(L.Qs + r * kRow + dc, qn);
                 st8<V8>(L.Ks + r * kRow + dc, kn);
                 st8<V8>(L.dOs + r * kRow + dc, do8);
-                if ((tid & 3) == 0) {
+                if ((st & 3) == 0) {
                     L.ndelta[r] = -dl;
                     if (!BIG && r < N) p.delta[((int64_t)b * p.heads + h) * p.delta_stride + r] = dl;   // for the dq kernel
                 }
-                if ((tid & 3) == 1) {
+                if ((st & 3) == 1) {
                     float l2 = -INFINITY;          // padded / fully masked rows: P = 0
                     if (r < N) { const float l = L.rawLse[r]; l2 = (l == -INFINITY) ? -INFINITY : -l * kLog2e; }
                     L.nlse2[r] = l2;
                 }
-                if ((tid & 3) == 2) L.kinv[r] = (sqrtf(sk) > kNormEps) ? ik : -ik;
+                if ((st & 3) == 2) L.kinv[r] = (sqrtf(sk) > kNormEps) ? ik : -ik;
             }
         }
+        // lane-derived values of the blocks and the epilogue are made here, once per unit, so that
+        // neither they nor the addresses built on them live (or sit in scratch) across units
+        const int ln = lane_now();
+        const int l16 = ln & 15, g = ln >> 4;
+        const int key0 = wave_0 * 16 * KT + l16;        // this lane's key in key tile 0 (tile kt: + 16 kt)
+        const E* bias_t = HAS_BIAS ? bias_base + key0 * R_tot : nullptr;
+        const ME* mask_t = MASK_DT >= 0 ? mask_base + key0 * R_tot : nullptr;
 #pragma unroll
         for (int kt = 0; kt < KT; kt++) w.bv[kt] = ld8<V8>(L.rawV + (key0 + 16 * kt) * 32 + 8 * g);
         __syncthreads();   // tiles complete; the landing area is free again
@@ -468,6 +478,9 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
 
     // ---- flush the per-workgroup partial sums ----
     if (HAS_BIAS) {
+        const int ln = lane_now();
+        const int g = ln >> 4;
+        const int key0 = wave_0 * 16 * KT + (ln & 15);
 #pragma unroll
         for (int kt = 0; kt < KT; kt++) {
             float* dst = p.part_dbias + (((int64_t)h * p.db_parts + p.db_slot0 + grp) * NPk_tot + k_off + key0 + 16 * kt) * R_tot + q_off;
