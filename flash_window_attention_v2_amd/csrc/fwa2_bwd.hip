@@ -179,14 +179,15 @@ __device__ __forceinline__ void unit_blocks(BwdLds<DT, NQB>& L, WaveRegs<DT, NQB
 }
 
 // KT = key tiles of 16 owned by one wavefront, NQB = compile-time bound on query blocks of 32.
-// MASKED: this launch handles the units whose window mask is live (and adds the mask); the units
-// with an all-zero mask go through a second launch of the MASKED = false instantiation, so no
-// block ever branches on the mask and each launch has a single copy of the block sequence.
+// Units whose window mask is live run the MASKED copy of the block sequence, the others the plain
+// one (uniform per unit, so no block ever branches on the mask).  MODE 2: one launch walks both
+// kinds (windows of up to 128 tokens, where both copies fit the register file without scratch);
+// MODE 0 / 1: a launch for the units with an all-zero mask and one for the others.
 // BIG: windows of more than 256 tokens.  The N x N score matrix is cut into 256 x 256 super-tiles;
 // a workgroup then belongs to one (head, query chunk, key chunk), reads only those rows, keeps that
 // tile of dbias in registers and writes its share of dk / dv (already taken back through the
 // normalisation, which is linear) as fp32 partials that dkv_reduce_kernel sums over the query chunks.
-template <int DT, bool HAS_BIAS, int MASK_DT, int NQB, int KT, bool MASKED, bool BIG>
+template <int DT, bool HAS_BIAS, int MASK_DT, int NQB, int KT, int MODE, bool BIG>
 __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) {
     typedef typename Elem<DT>::E E;
     typedef typename Elem<DT>::V8 V8;
@@ -260,10 +261,12 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
     const E* bias_base = nullptr;
     if (HAS_BIAS) bias_base = reinterpret_cast<const E*>(p.bias_t) + ((int64_t)h * NPk_tot + k_off) * R_tot + q_off;
 
-    // ---- which units belong to this launch.  With the mask flags at hand the windows of this
-    // launch's class (mask live or not) are listed once and the units are dealt out by their rank
-    // within the class, so every workgroup of the head gets the same number of them whatever the
-    // pattern of masked windows. ----
+    // ---- the order in which the head's units are dealt out.  With the mask flags at hand the windows
+    // are listed once, those with a live mask first: ranks t < t_live are the units of the live
+    // windows, the rest those of the all-zero windows, each group image by image.  Every workgroup
+    // walks t = grp, grp + groups, ..., so all get the same number of units (to within one) whatever
+    // the pattern of masked windows, and the workgroups running at any moment read neighbouring
+    // units.  Without the flags every unit of a masked call counts as live. ----
     __shared__ uint8_t lds_live[kLiveCache];
     __shared__ uint16_t lds_list[kLiveCache];
     __shared__ int lds_count;
@@ -273,32 +276,45 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
         __syncthreads();
         if (wave_0 == 0) {
             int cnt = 0;
-            for (int base = 0; base < p.n_windows; base += 64) {
-                const int w = base + lane_0;
-                const bool in = w < p.n_windows && ((lds_live[w] != 0) == MASKED);
-                const unsigned long long bal = __ballot(in);
-                if (in) lds_list[cnt + __popcll(bal & ((1ull << lane_0) - 1ull))] = (uint16_t)w;
-                cnt += __popcll(bal);
+#pragma unroll 1
+            for (int cls = 1; cls >= 0; cls--) {
+                for (int base = 0; base < p.n_windows; base += 64) {
+                    const int w = base + lane_0;
+                    const bool in = w < p.n_windows && ((lds_live[w] != 0) == (cls != 0));
+                    const unsigned long long bal = __ballot(in);
+                    if (in) lds_list[cnt + __popcll(bal & ((1ull << lane_0) - 1ull))] = (uint16_t)w;
+                    cnt += __popcll(bal);
+                }
+                if (cls == 1 && lane_0 == 0) lds_count = cnt;
             }
-            if (lane_0 == 0) lds_count = cnt;
         }
         __syncthreads();
     }
-    const int cnt = listed ? __builtin_amdgcn_readfirstlane(lds_count) : 0;
-    const int total = listed ? ((p.bw + p.n_windows - 1) / p.n_windows) * cnt : p.bw;   // ranks to deal out
+    const int n_live = listed ? __builtin_amdgcn_readfirstlane(lds_count) : 0;
+    const int n_img = (p.bw + p.n_windows - 1) / p.n_windows;
+    const int t_live = listed ? n_img * n_live : (MASK_DT >= 0 ? p.bw : 0);
+    const int total = listed ? n_img * p.n_windows : p.bw;
+    const int t_begin = MODE == 0 ? t_live : 0;              // ranks this launch deals out
+    const int t_end = MODE == 1 ? t_live : total;
     auto unit_of = [&](int t) -> int {
         if (!listed) return t;
-        const int img = t / cnt;
-        return __builtin_amdgcn_readfirstlane(img * p.n_windows + (int)lds_list[t - img * cnt]);
-    };
-    // first rank >= t (in steps of the group count) that names an existing unit of this launch
-    auto rank_from = [&](int t) -> int {
-        for (; t < total; t += p.groups) {
-            const int b = unit_of(t);
-            if (b >= p.bw) continue;
-            if (listed || MASK_DT < 0 || !p.mask_live || ((p.mask_live[b % p.n_windows] != 0) == MASKED)) return t;
+        int img, wi;
+        if (t < t_live) {
+            img = t / n_live;
+            wi = t - img * n_live;
+        } else {
+            const int n_rest = p.n_windows - n_live;
+            const int u = t - t_live;
+            img = u / n_rest;
+            wi = n_live + (u - img * n_rest);
         }
-        return total;
+        return __builtin_amdgcn_readfirstlane(img * p.n_windows + (int)lds_list[wi]);
+    };
+    // first rank >= t (in steps of the group count) that names an existing unit
+    auto rank_from = [&](int t) -> int {
+        for (; t < t_end; t += p.groups)
+            if (unit_of(t) < p.bw) return t;
+        return t_end;
     };
     // ---- asynchronous fetch of one unit's rows into the landing area ----
     auto fetch_unit = [&](int b) __attribute__((always_inline)) {
@@ -344,15 +360,16 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
     }
     __syncthreads();
 
-    int t = rank_from(grp);
-    if (t < total) fetch_unit(unit_of(t));
+    int t = rank_from(t_begin + grp);
+    if (t < t_end) fetch_unit(unit_of(t));
 
-    while (t < total) {
+    while (t < t_end) {
         const int b = unit_of(t);
         const int t_next = rank_from(t + p.groups);
-        const int b_next = t_next < total ? unit_of(t_next) : p.bw;
+        const int b_next = t_next < t_end ? unit_of(t_next) : p.bw;
+        const bool live = MODE != 0 && MASK_DT >= 0 && t < t_live;     // this unit's window mask has non-zero entries
         const ME* mask_base = nullptr;
-        if (MASK_DT >= 0) {
+        if (live) {
             const int wnd = b % p.n_windows;
             mask_base = reinterpret_cast<const ME*>(p.mask_t) + ((int64_t)wnd * NPk_tot + k_off) * R_tot + q_off;
         }
@@ -398,7 +415,7 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
         const int l16 = ln & 15, g = ln >> 4;
         const int key0 = wave_0 * 16 * KT + l16;        // this lane's key in key tile 0 (tile kt: + 16 kt)
         const E* bias_t = HAS_BIAS ? bias_base + key0 * R_tot : nullptr;
-        const ME* mask_t = MASK_DT >= 0 ? mask_base + key0 * R_tot : nullptr;
+        const ME* mask_t = live ? mask_base + key0 * R_tot : nullptr;
 #pragma unroll
         for (int kt = 0; kt < KT; kt++) w.bv[kt] = ld8<V8>(L.rawV + (key0 + 16 * kt) * 32 + 8 * g);
         __syncthreads();   // tiles complete; the landing area is free again
@@ -414,13 +431,19 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
         // The next unit's fetch starts at the top of the last block: memory returns in issue order,
         // so an earlier start would make every later wait for bias values also wait for the fetch.
         const int fetch_at = nqb - 1;
-        unit_blocks<DT, HAS_BIAS, ME, NQB, KT, MASKED, BIG>(L, w, bias_t, mask_t, NK, nqb, l16, g, key0, tail_keys, R_tot, [&](int qb) {
+        auto block_start = [&](int qb) __attribute__((always_inline)) {
             if (qb == fetch_at && b_next < p.bw) fetch_unit(b_next);
             // The SIMD favours its older wavefront, so the younger one of each pair would finish the
             // blocks long after it and run the tail alone; raising its priority after the first quarter
             // lets both reach the end of the unit together.
             if (qb == NQB / 4 && wave_0 >= (p.waves >> 1)) __builtin_amdgcn_s_setprio(2);
-        });
+        };
+        if (MODE == 1 || (MODE == 2 && live))
+            unit_blocks<DT, HAS_BIAS, ME, NQB, KT, MASK_DT >= 0, BIG>(L, w, bias_t, mask_t, NK, nqb, l16, g, key0, tail_keys,
+                                                                      R_tot, block_start);
+        else
+            unit_blocks<DT, HAS_BIAS, ME, NQB, KT, false, BIG>(L, w, bias_t, mask_t, NK, nqb, l16, g, key0, tail_keys, R_tot,
+                                                               block_start);
         __builtin_amdgcn_s_setprio(0);
 
         // ---- epilogue dk, dv: lane (key, g) holds d = 8g + 4dt + i (16 bytes of a row); k_hat and 1/|k| come from LDS ----
@@ -678,29 +701,39 @@ static int resident_per_cu(K kern, int threads) {
 
 template <int DT, bool HAS_BIAS, int MASK_DT, int NQB, int KT, bool BIG>
 static hipError_t launch_main(BwdParams p, const BwdPlan& pl, hipStream_t st, int* groups_out) {
+    // Up to 64 tokens one launch walks masked and unmasked units alike; above that the two copies of
+    // the block sequence cost occupancy (128 tokens) or spill (256), and each kind gets a launch.
+    constexpr bool kOneLaunch = MASK_DT >= 0 && NQB <= 2 && !BIG;
     // never more workgroups per head (and super-tile) than the plan sized the workspace for
     static const int fit = [&] {
-        const int a = resident_per_cu(bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, false, BIG>, 64 * pl.waves);
-        const int b = resident_per_cu(bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, true, BIG>, 64 * pl.waves);
-        return a < b ? a : b;
+        if constexpr (kOneLaunch) {
+            return resident_per_cu(bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, 2, BIG>, 64 * pl.waves);
+        } else {
+            const int a = resident_per_cu(bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, 0, BIG>, 64 * pl.waves);
+            const int b = MASK_DT >= 0 ? resident_per_cu(bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, 1, BIG>, 64 * pl.waves) : a;
+            return a < b ? a : b;
+        }
     }();
     const int tiles = pl.n_chunks * pl.n_chunks;
     int groups = (p.cus * fit) / (p.heads * tiles);
     if (groups < 1) groups = 1;
     if (groups > pl.groups) groups = pl.groups;
     p.groups = groups;
-    p.db_parts = (MASK_DT >= 0 && p.mask_live != nullptr) ? 2 * groups : groups;
+    const bool two = !kOneLaunch && MASK_DT >= 0 && p.mask_live != nullptr;
+    p.db_parts = two ? 2 * groups : groups;
+    p.db_slot0 = 0;
     const dim3 grid(p.heads * tiles * groups), block(64 * pl.waves);
     if (p.ev_start) (void)hipEventRecord(p.ev_start, st);
-    // launch for the units whose mask is all zero (or every unit when there is no mask) ...
-    if (MASK_DT < 0 || p.mask_live != nullptr) {
-        p.db_slot0 = 0;
-        hipLaunchKernelGGL((bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, false, BIG>), grid, block, 0, st, p);
-    }
-    // ... and for the units whose mask is live
-    if (MASK_DT >= 0) {
-        p.db_slot0 = p.mask_live != nullptr ? groups : 0;
-        hipLaunchKernelGGL((bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, true, BIG>), grid, block, 0, st, p);
+    if constexpr (kOneLaunch) {
+        hipLaunchKernelGGL((bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, 2, BIG>), grid, block, 0, st, p);
+    } else {
+        // the units whose mask is all zero (or every unit when there is no mask) ...
+        if (MASK_DT < 0 || two) hipLaunchKernelGGL((bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, 0, BIG>), grid, block, 0, st, p);
+        // ... and the units whose mask is live (all of them when the flags are absent)
+        if (MASK_DT >= 0) {
+            p.db_slot0 = two ? groups : 0;
+            hipLaunchKernelGGL((bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, 1, BIG>), grid, block, 0, st, p);
+        }
     }
     if (p.ev_stop) (void)hipEventRecord(p.ev_stop, st);
     hipError_t e = hipGetLastError();
