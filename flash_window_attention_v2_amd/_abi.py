@@ -25,6 +25,8 @@ EXPORTS = (
     "fwa2_backward_workspace_bytes",
     "fwa2_forward",
     "fwa2_backward",
+    "fwa2_cpb_bias_forward",
+    "fwa2_cpb_bias_backward",
     "fwa2_set_kernel_events",
 )
 
@@ -94,6 +96,12 @@ def load():
         lib.fwa2_forward.restype = ctypes.c_int
         lib.fwa2_backward.argtypes = [ctypes.POINTER(Problem)]
         lib.fwa2_backward.restype = ctypes.c_int
+        lib.fwa2_cpb_bias_forward.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                              ctypes.c_void_p, ctypes.c_void_p]
+        lib.fwa2_cpb_bias_forward.restype = ctypes.c_int
+        lib.fwa2_cpb_bias_backward.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                               ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+        lib.fwa2_cpb_bias_backward.restype = ctypes.c_int
         lib.fwa2_set_kernel_events.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
         lib.fwa2_set_kernel_events.restype = None
         if lib.fwa2_abi_version() != ABI_VERSION:

@@ -16,6 +16,9 @@ hipError_t launch_mask_scan(const void* mask, int mask_dt, int64_t sw, int64_t s
 hipError_t launch_backward(const BwdParams& p, int dtype, bool has_bias, int mask_dt, hipStream_t st);
 size_t backward_workspace_bytes(int heads, int n, int bw, bool has_bias, bool has_mask, int n_windows, int cus);
 int backward_supported(int n);
+hipError_t launch_cpb_bias_forward(const void* table, int dtype, int heads, int wh, int ww, void* bias, hipStream_t st);
+hipError_t launch_cpb_bias_backward(const void* table, const void* dbias, int dtype, int heads, int wh, int ww,
+                                    void* dtable, hipStream_t st);
 }  // namespace fwa2
 
 namespace {
@@ -141,6 +144,33 @@ int fwa2_mask_scan(const void* mask, int mask_dtype, int n_windows, int n, int64
         return fail(FWA2_ERR_INVALID_ARGUMENT, "fwa2_mask_scan: bad mask dtype");
     hipError_t e = fwa2::launch_mask_scan(mask, mask_dtype, stride_w, stride_n, n, n_windows, live, (hipStream_t)stream);
     if (e != hipSuccess) return fail(FWA2_ERR_HIP, "mask scan launch: %s", hipGetErrorString(e));
+    return FWA2_OK;
+}
+
+static int check_cpb(const char* what, const void* a, const void* b, const void* c, int dtype, int heads, int wh, int ww) {
+    if (a == nullptr || b == nullptr || c == nullptr) return fail(FWA2_ERR_INVALID_ARGUMENT, "%s: null pointer", what);
+    if (dtype != FWA2_F16 && dtype != FWA2_BF16) return fail(FWA2_ERR_INVALID_ARGUMENT, "%s: dtype must be fp16 or bf16", what);
+    if (heads <= 0 || wh <= 0 || ww <= 0) return fail(FWA2_ERR_INVALID_ARGUMENT, "%s: heads and window extents must be positive", what);
+    if ((int64_t)wh * ww > 46340) return fail(FWA2_ERR_UNSUPPORTED, "%s: window of %d x %d tokens is too large", what, wh, ww);
+    return FWA2_OK;
+}
+
+int fwa2_cpb_bias_forward(const void* table, int dtype, int heads, int wh, int ww, void* bias, void* stream) {
+    g_err[0] = 0;
+    int rc = check_cpb("fwa2_cpb_bias_forward", table, bias, bias, dtype, heads, wh, ww);
+    if (rc) return rc;
+    hipError_t e = fwa2::launch_cpb_bias_forward(table, dtype, heads, wh, ww, bias, (hipStream_t)stream);
+    if (e != hipSuccess) return fail(FWA2_ERR_HIP, "cpb bias forward launch: %s", hipGetErrorString(e));
+    return FWA2_OK;
+}
+
+int fwa2_cpb_bias_backward(const void* table, const void* dbias, int dtype, int heads, int wh, int ww, void* dtable,
+                           void* stream) {
+    g_err[0] = 0;
+    int rc = check_cpb("fwa2_cpb_bias_backward", table, dbias, dtable, dtype, heads, wh, ww);
+    if (rc) return rc;
+    hipError_t e = fwa2::launch_cpb_bias_backward(table, dbias, dtype, heads, wh, ww, dtable, (hipStream_t)stream);
+    if (e != hipSuccess) return fail(FWA2_ERR_HIP, "cpb bias backward launch: %s", hipGetErrorString(e));
     return FWA2_OK;
 }
 

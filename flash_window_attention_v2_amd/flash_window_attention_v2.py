@@ -232,3 +232,40 @@ class FlashWindowAttentionV2QKVPacked(torch.autograd.Function):
             p.stream = torch.cuda.current_stream().cuda_stream
             _abi.check(lib.fwa2_backward(p), "fwa2_backward")
         return dqkv, dscale, db, None
+
+
+class CpbBias(torch.autograd.Function):
+    """bias[H, N, N] = 16 sigmoid(table[index]) for a window of wh x ww tokens, where `table` is the
+    [(2wh-1)(2ww-1), H] output of the continuous-position-bias MLP and `index` the closed form of the
+    reference's relative_position_index buffer (swin_transformer_v2.py:240-254, 283-287).  One small kernel
+    each way instead of gather + permute + sigmoid + scale, and in backward a fixed-order fp32 sum per
+    table entry instead of autograd's sort-based index_put(accumulate)."""
+
+    @staticmethod
+    def forward(ctx, table, wh, ww):
+        assert table.is_cuda and table.dtype in (torch.float16, torch.bfloat16), "fused bias path: fp16 / bf16 on the GPU"
+        assert table.dim() == 2 and table.shape[0] == (2 * wh - 1) * (2 * ww - 1), "table must be [(2wh-1)(2ww-1), H]"
+        table = table.contiguous()
+        heads = table.shape[1]
+        n = wh * ww
+        bias = torch.empty((heads, n, n), device=table.device, dtype=table.dtype)
+        lib = _abi.load()
+        with torch.cuda.device(table.device):
+            _abi.check(lib.fwa2_cpb_bias_forward(table.data_ptr(), _DTYPES[table.dtype], heads, wh, ww, bias.data_ptr(),
+                                                 torch.cuda.current_stream().cuda_stream), "fwa2_cpb_bias_forward")
+        ctx.save_for_backward(table)
+        ctx.window = (wh, ww)
+        return bias
+
+    @staticmethod
+    def backward(ctx, dbias):
+        (table,) = ctx.saved_tensors
+        wh, ww = ctx.window
+        dbias = dbias.contiguous()
+        dtable = torch.empty_like(table)
+        lib = _abi.load()
+        with torch.cuda.device(table.device):
+            _abi.check(lib.fwa2_cpb_bias_backward(table.data_ptr(), dbias.data_ptr(), _DTYPES[table.dtype], table.shape[1],
+                                                  wh, ww, dtable.data_ptr(), torch.cuda.current_stream().cuda_stream),
+                       "fwa2_cpb_bias_backward")
+        return dtable, None, None

@@ -18,6 +18,7 @@ import torch.nn.functional as F
 from torch.utils.checkpoint import checkpoint
 
 from .win_attention_func import flash_win_attn_v2_func, flash_win_attn_v2_qkvpacked_func, win_attention_torch
+from .flash_window_attention_v2 import CpbBias
 
 
 def _pair(x):
@@ -91,6 +92,9 @@ class WindowAttention(nn.Module):
     #: feed the fused operator from the packed projection (flash path only); False selects the
     #: reference's call with three strided views
     packed_qkv = True
+    #: build the bias (and take its gradient back to table space) with the library's two small kernels
+    #: instead of gather / permute / sigmoid and autograd's sort-based scatter (flash path only)
+    fused_bias = True
 
     def __init__(self, dim, window_size, num_heads, is_flash=True, qkv_bias=True, attn_drop=0., proj_drop=0.,
                  pretrained_window_size=[0, 0]):
@@ -134,10 +138,27 @@ class WindowAttention(nn.Module):
         self.proj = nn.Linear(dim, dim)
         self.proj_drop = nn.Dropout(proj_drop)
 
+    def _index_is_closed_form(self):
+        """Whether the relative_position_index buffer (it travels in state_dicts) still holds the closed
+        form the fused bias kernels compute on the fly; checked once per buffer version."""
+        buf = self.relative_position_index
+        seen = getattr(self, "_index_checked", None)
+        if seen is None or seen[0] != buf._version or seen[1] != buf.data_ptr():
+            wh, ww = self.window_size
+            rows = torch.arange(wh, device=buf.device).repeat_interleave(ww)
+            cols = torch.arange(ww, device=buf.device).repeat(wh)
+            want = (rows[:, None] - rows[None, :] + wh - 1) * (2 * ww - 1) + (cols[:, None] - cols[None, :] + ww - 1)
+            seen = (buf._version, buf.data_ptr(), bool(torch.equal(buf, want)))
+            self._index_checked = seen
+        return seen[2]
+
     def relative_position_bias(self):
         """[H, N, N] bias = 16 sigmoid(cpb_mlp(table)[index]) (swin_transformer_v2.py:283-287)."""
         n = self.window_size[0] * self.window_size[1]
         per_offset = self.cpb_mlp(self.relative_coords_table).view(-1, self.num_heads)
+        if (self.is_flash and self.fused_bias and per_offset.is_cuda
+                and per_offset.dtype in (torch.float16, torch.bfloat16) and self._index_is_closed_form()):
+            return CpbBias.apply(per_offset, self.window_size[0], self.window_size[1])
         bias = per_offset[self.relative_position_index.view(-1)].view(n, n, self.num_heads)
         return 16 * torch.sigmoid(bias.permute(2, 0, 1).contiguous())
 

@@ -163,6 +163,26 @@ int fwa2_forward(const fwa2_problem* p);
 int fwa2_backward(const fwa2_problem* p);
 
 /*
+ * Relative position bias of a window of wh x ww tokens (N = wh ww) from its table, for the caller of the
+ * operator: replaces the gather by relative_position_index, the permute to [H, N, N] and 16 * sigmoid of
+ * flash_win_attn_v2/swin_transformer_v2.py:283-287 (the table is the output of the module's cpb_mlp).
+ *   table [(2wh-1)(2ww-1), H], bias [H, N, N], both contiguous and of `dtype` (F16 or BF16);
+ *   bias[h][q][k] = 16 sigmoid(table[idx(q,k)][h]),
+ *   idx(q,k) = (r_q - r_k + wh - 1)(2ww - 1) + (c_q - c_k + ww - 1) with token = r ww + c
+ *   (the closed form of the reference's relative_position_index buffer, swin_transformer_v2.py:240-254).
+ */
+int fwa2_cpb_bias_forward(const void* table, int dtype, int heads, int wh, int ww, void* bias, void* stream);
+
+/*
+ * Gradient of the above with respect to the table: dtable[i][h] = 16 s (1 - s) * sum of dbias[h][q][k] over
+ * the pairs with idx(q,k) = i, s = sigmoid(table[i][h]); summed in fp32 in a fixed order.  Replaces what
+ * autograd derives for swin_transformer_v2.py:283-287 (sigmoid backward, permute, index_put with accumulate).
+ *   dbias [H, N, N] contiguous, dtable [(2wh-1)(2ww-1), H] contiguous, both of `dtype`.
+ */
+int fwa2_cpb_bias_backward(const void* table, const void* dbias, int dtype, int heads, int wh, int ww, void* dtable,
+                           void* stream);
+
+/*
  * Measurement hook, no counterpart in the reference: when both are non-NULL the
  * next fwa2_backward calls (from any thread of the process) record the two hipEvent_t on the
  * problem's stream immediately before and after the main backward kernel (the

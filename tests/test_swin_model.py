@@ -226,6 +226,39 @@ def test_window_attention_module_gpu(dtype):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("window", [(8, 8), (7, 7), (4, 8), (16, 16)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_fused_position_bias_gpu(window, dtype):
+    """CpbBias (bias from the table and the gradient back into table space) against the module's own
+    framework expression evaluated in fp32 (swin_transformer_v2.py:283-287 of the reference)."""
+    from flash_window_attention_v2_amd.flash_window_attention_v2 import CpbBias
+    torch.manual_seed(1)
+    dev = torch.device("cuda")
+    wh, ww = window
+    n, heads = wh * ww, 3
+    table = (2.0 * torch.randn((2 * wh - 1) * (2 * ww - 1), heads, device=dev)).to(dtype)
+    grad = torch.randn(heads, n, n, device=dev).to(dtype)
+    index = swin.WindowAttention(32 * heads, window, heads, is_flash=False).relative_position_index.to(dev)
+
+    t_ref = table.float().requires_grad_()
+    bias_ref = 16 * torch.sigmoid(t_ref[index.view(-1)].view(n, n, heads).permute(2, 0, 1))
+    bias_ref.backward(grad.float())
+
+    t = table.clone().requires_grad_()
+    bias = CpbBias.apply(t, wh, ww)
+    bias.backward(grad)
+    assert bias.shape == (heads, n, n) and bias.dtype == dtype and bias.is_contiguous()
+    ulp = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+    assert float((bias.float() - bias_ref).abs().max()) <= 16 * ulp          # one rounding of sigmoid, then exact x16
+    scale = float(t_ref.grad.abs().max())
+    assert float((t.grad.float() - t_ref.grad).abs().max()) <= 4 * ulp * scale + 1e-6
+    # same call twice: bit-identical (fixed summation order)
+    t2 = table.clone().requires_grad_()
+    CpbBias.apply(t2, wh, ww).backward(grad)
+    assert torch.equal(t.grad, t2.grad)
+
+
+@pytest.mark.gpu
 def test_model_flash_matches_classic_gpu():
     """Whole-model step at a reduced width: bf16 model on the fused kernels against the same weights
     on the classic path in fp32, LayerNorms away from their zero initialisation and no stochastic
