@@ -103,6 +103,28 @@ def test_fp32_mask_and_odd_group_counts():
     _run_and_check(inp, torch.bfloat16, tag="fp32mask")
 
 
+def test_more_windows_than_the_flag_cache_and_no_flags(monkeypatch):
+    """The kernels keep the per-window mask flags in LDS for up to 1024 windows; beyond that, and when a
+    caller passes no flags at all, every window is treated as masked.  Both paths, forward and backward."""
+    # (a) 1040 windows of 16 tokens, a third of them with a live mask
+    n_w, n, heads = 1040, 16, 2
+    inp = make_inputs(batch=1, n_windows=n_w, heads=heads, n=n, dtype=torch.bfloat16, seed=21, with_mask=False)
+    g = torch.Generator().manual_seed(22)
+    mask = torch.where(torch.rand(n_w, n, n, generator=g) < 0.3, -100.0, 0.0)
+    mask[torch.arange(n_w) % 3 != 0] = 0.0
+    mask[:, torch.arange(n), torch.arange(n)] = 0.0
+    inp["mask"] = mask.to(torch.bfloat16)
+    _run_and_check(inp, torch.bfloat16, tag="1040 windows")
+
+    # (b) a caller that never scanned the mask: the flag pointer stays NULL
+    import flash_window_attention_v2_amd.flash_window_attention_v2 as fw
+    monkeypatch.setattr(fw, "mask_window_flags", lambda mask: None)
+    for n_, res, win, shift in ((64, 32, 8, 4), (256, 64, 16, 8)):
+        inp = make_inputs(batch=2, n_windows=(res // win) ** 2, heads=3, n=n_, dtype=torch.bfloat16, seed=23,
+                          resolution=res, window=win, shift=shift)
+        _run_and_check(inp, torch.bfloat16, tag=f"no flags N={n_}")
+
+
 def test_random_inf_mask_and_random_scale():
     """The reference's own check protocol: randn bias and logit_scale, ~half the mask entries -inf
     (benchmark/check.py:23-33), here with every row keeping at least one open key."""
