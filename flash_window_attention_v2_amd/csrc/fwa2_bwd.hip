@@ -624,6 +624,9 @@ int backward_supported(int n) { return n >= 1; }
 void dq_geometry(int n, int* waves, int* chunks);
 hipError_t launch_backward_dq(const BwdParams& p, int dtype, bool has_bias, int mask_dt, hipStream_t st);
 int backward_dq_resident_supported(int n);
+int backward_fused_supported(int n);
+hipError_t launch_backward_fused(const BwdParams& p, int dtype, bool has_bias, int mask_dt, hipStream_t st,
+                                 int max_groups, int* parts_out);
 hipError_t launch_backward_dq_resident(const BwdParams& p, int dtype, bool has_bias, int mask_dt, hipStream_t st,
                                        int max_groups, int* ds_parts_out);
 
@@ -772,6 +775,21 @@ static hipError_t launch_bwd_dt(BwdParams p, bool has_bias, int mask_dt, hipStre
     p.npk_tot = pl.npk;
     p.part_dk = reinterpret_cast<float*>(ws + pl.off_dk);
     p.part_dv = reinterpret_cast<float*>(ws + pl.off_dv);
+    if (backward_fused_supported(p.n)) {
+        // one pass over q, k, v, o, dO; no key-major side tables, no delta buffer
+        int parts = 0;
+        const int mg = pl.groups < pl.dq_max_groups ? pl.groups : pl.dq_max_groups;
+        hipError_t ef = launch_backward_fused(p, DT, has_bias, mask_dt, st, mg, &parts);
+        if (ef != hipSuccess) return ef;
+        p.db_parts = parts;
+        p.ds_parts = parts;
+        if (has_bias || p.scale_kind == FWA2_SCALE_TENSOR) {
+            dim3 gr(has_bias ? pl.r / 32 : 1, has_bias ? pl.npk : 1, p.heads);
+            hipLaunchKernelGGL(reduce_kernel<DT>, gr, dim3(256), 0, st, p, pl.npk, pl.r, has_bias);
+            ef = hipGetLastError();
+        }
+        return ef;
+    }
     const dim3 tgrid(pl.r / 32, (pl.npk + 31) / 32, 1);
     if (has_bias) {
         dim3 gr(tgrid.x, tgrid.y, p.heads);
