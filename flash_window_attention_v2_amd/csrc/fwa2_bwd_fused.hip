@@ -9,8 +9,9 @@
 //
 // Skeleton of the resident query-side kernel: a workgroup belongs to one head, every
 // wavefront owns 16 query rows and holds (bias [+ mask]) * log2e - m for them in the register
-// layout of the score accumulators; K_hat (fp16) and V of the next unit land in LDS by DMA while
-// the current unit is computed.  Per unit:
+// layout of the score accumulators.  The rows of the next unit travel in registers while the
+// current unit is computed (21 registers per lane; no landing area, so three workgroups fit a CU).
+// Per unit:
 //   phase A (wavefront = 16 queries, lane = query, registers = keys)
 //     S^T - m = K_hat Q_hat^T,  dP^T - delta = V dO^T,  e = 2^(S^T - lse2),  dZ^T = e (dP^T - delta)
 //     dQ_hat^T += K_hat^T dZ^T;  dbias tile += dZ (registers, for the whole launch)
@@ -37,18 +38,13 @@ __global__ void __launch_bounds__(64 * NT) bwd_fused_kernel(const BwdParams p) {
     constexpr int S = kLdsStride;         // row stride of the 32-column tiles
     constexpr int PS = ROWS + 8;          // row stride of the [query][key] tiles
 
-    __shared__ __attribute__((aligned(16))) SE lds_K[2][ROWS * S];     // k_hat, staged one unit ahead
-    __shared__ __attribute__((aligned(16))) E lds_V[2][ROWS * S];
-    __shared__ __attribute__((aligned(16))) float lds_kinv[2][ROWS];   // 1 / max(|k|, eps), negated when |k| <= eps
+    __shared__ __attribute__((aligned(16))) SE lds_K[ROWS * S];        // k_hat of the current unit
+    __shared__ __attribute__((aligned(16))) E lds_V[ROWS * S];
+    __shared__ __attribute__((aligned(16))) float lds_kinv[ROWS];      // 1 / max(|k|, eps), negated when |k| <= eps
     __shared__ __attribute__((aligned(16))) SE lds_Qs[ROWS * S];       // q_hat s log2e of the current unit
     __shared__ __attribute__((aligned(16))) E lds_dOs[ROWS * S];       // dO (times w when folded) of the current unit
     __shared__ __attribute__((aligned(16))) E lds_Pt[ROWS * PS];       // e,  [query][key]
     __shared__ __attribute__((aligned(16))) SE lds_Zt[ROWS * PS];      // dZ, [query][key]
-    __shared__ __attribute__((aligned(16))) E lds_rawK[ROWS * 32];     // landing areas: unpadded 64-byte rows
-    __shared__ __attribute__((aligned(16))) E lds_rawV[ROWS * 32];
-    __shared__ __attribute__((aligned(16))) E lds_rawQ[ROWS * 32];
-    __shared__ __attribute__((aligned(16))) E lds_rawDO[ROWS * 32];
-    __shared__ __attribute__((aligned(16))) E lds_rawO[ROWS * 32];
     __shared__ uint8_t lds_live[kLiveCache];
     __shared__ uint16_t lds_list[kLiveCache];
     __shared__ int lds_count;
@@ -75,27 +71,7 @@ __global__ void __launch_bounds__(64 * NT) bwd_fused_kernel(const BwdParams p) {
     }
     const float scale2 = s_true * kLog2e;
 
-    // rows that no unit ever writes (rows >= n) must read as zeros for the whole kernel
-    for (int i = tid; i < 2 * ROWS * S / 8; i += nthreads) {
-        st8<SV8>(&lds_K[0][0] + i * 8, zero8<SV8>());
-        st8<V8>(&lds_V[0][0] + i * 8, zero8<V8>());
-    }
-    for (int i = tid; i < ROWS * S / 8; i += nthreads) {
-        st8<SV8>(lds_Qs + i * 8, zero8<SV8>());
-        st8<V8>(lds_dOs + i * 8, zero8<V8>());
-    }
-    for (int i = tid; i < ROWS * PS / 8; i += nthreads) {
-        st8<V8>(lds_Pt + i * 8, zero8<V8>());
-        st8<SV8>(lds_Zt + i * 8, zero8<SV8>());
-    }
-    for (int i = tid; i < ROWS * 32 / 8; i += nthreads) {
-        st8<V8>(lds_rawK + i * 8, zero8<V8>());
-        st8<V8>(lds_rawV + i * 8, zero8<V8>());
-        st8<V8>(lds_rawQ + i * 8, zero8<V8>());
-        st8<V8>(lds_rawDO + i * 8, zero8<V8>());
-        st8<V8>(lds_rawO + i * 8, zero8<V8>());
-    }
-    for (int i = tid; i < 2 * ROWS; i += nthreads) (&lds_kinv[0][0])[i] = 0.f;
+    // every tile row is rewritten for every unit (rows >= n with zeros), nothing to clear up front
 
     const int qrow = wave * 16 + l16;       // this lane's query in phase A
 
@@ -204,45 +180,34 @@ __global__ void __launch_bounds__(64 * NT) bwd_fused_kernel(const BwdParams p) {
     };
     auto unit_of = [&](const Cursor& c) -> int { return c.img * nw + window_at(c.wi); };
 
-    // ---- per-unit fetch: the wavefront's 16 rows of k, v (which it will stage) and of q, dO, o (its
-    // own queries) by DMA; lse of its queries in a register ----
-    auto dma16 = [&](const E* src, E* lds_wave_base) __attribute__((always_inline)) {
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                         (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, kStreamPolicy);
+    // ---- per-unit fetch, one unit ahead, into registers: 16 bytes of a k and a v row (the 16 rows
+    // this wavefront stages, 4 lanes per row) and 16 bytes of the q, dO and o rows of this lane's
+    // query in the operand layout (lane (query, g) takes columns 8g .. 8g+7); rows >= n read as zeros ----
+    struct Rows { V8 k, v, q, dO, o; float lse; };
+    auto ldrow = [&](const T4& t, int b, int row, int col) -> V8 {
+        return ld8<V8>(reinterpret_cast<const E*>(t.ptr) + b * t.sb + h * t.sh + (int64_t)row * t.sn + col);
     };
-    auto fetch = [&](int b, float& lse) __attribute__((always_inline)) {
-        int ln = lane;
+    auto fetch = [&](int b, Rows& r) __attribute__((always_inline)) {
+        int ln = lane;                     // re-derived per call: no address lives across the unit loop
         asm volatile("" : "+v"(ln));
-        const int fc8 = (ln & 3) * 8;
-        const int row0 = wave * 16;
-        const int frow = row0 + (ln >> 2);
-        if (frow < N) {
-            dma16(reinterpret_cast<const E*>(p.k.ptr) + b * p.k.sb + h * p.k.sh + (int64_t)frow * p.k.sn + fc8,
-                  lds_rawK + row0 * 32);
-            dma16(reinterpret_cast<const E*>(p.v.ptr) + b * p.v.sb + h * p.v.sh + (int64_t)frow * p.v.sn + fc8,
-                  lds_rawV + row0 * 32);
-            dma16(reinterpret_cast<const E*>(p.q.ptr) + b * p.q.sb + h * p.q.sh + (int64_t)frow * p.q.sn + fc8,
-                  lds_rawQ + row0 * 32);
-            dma16(reinterpret_cast<const E*>(p.d_o.ptr) + b * p.d_o.sb + h * p.d_o.sh + (int64_t)frow * p.d_o.sn + fc8,
-                  lds_rawDO + row0 * 32);
-            dma16(reinterpret_cast<const E*>(p.o.ptr) + b * p.o.sb + h * p.o.sh + (int64_t)frow * p.o.sn + fc8,
-                  lds_rawO + row0 * 32);
+        const int frow = wave * 16 + (ln >> 2), fc8 = (ln & 3) * 8;
+        r.k = zero8<V8>(); r.v = zero8<V8>();
+        if (frow < N) { r.k = ldrow(p.k, b, frow, fc8); r.v = ldrow(p.v, b, frow, fc8); }
+        const int q = wave * 16 + (ln & 15), c8 = (ln >> 4) * 8;
+        r.q = zero8<V8>(); r.dO = zero8<V8>(); r.o = zero8<V8>();
+        r.lse = -INFINITY;
+        if (q < N) {
+            r.q = ldrow(p.q, b, q, c8); r.dO = ldrow(p.d_o, b, q, c8); r.o = ldrow(p.o, b, q, c8);
+            r.lse = p.lse[b * p.lse_sb + h * p.lse_sh + q];
         }
-        const int q = row0 + (ln & 15);
-        lse = -INFINITY;
-        if (q < N) lse = p.lse[b * p.lse_sb + h * p.lse_sh + q];
     };
-    // landing area -> tiles of the unit after the current one: K normalised and rounded to fp16, V as is
-    auto stage = [&](int buf) __attribute__((always_inline)) {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // k, v rows -> tiles: K normalised and rounded to fp16, V as is
+    auto stage = [&](const Rows& r) __attribute__((always_inline)) {
         int ln = lane;
         asm volatile("" : "+v"(ln));
-        const int fc8 = (ln & 3) * 8;
-        const int frow = wave * 16 + (ln >> 2);
-        const V8 kk = ld8<V8>(lds_rawK + frow * 32 + fc8);
-        const V8 vv = ld8<V8>(lds_rawV + frow * 32 + fc8);
+        const int frow = wave * 16 + (ln >> 2), fc8 = (ln & 3) * 8;
         float x[8];
-        unpack8(kk, x);
+        unpack8(r.k, x);
         float ss = 0.f;
 #pragma unroll
         for (int j = 0; j < 8; j++) ss += x[j] * x[j];
@@ -251,9 +216,9 @@ __global__ void __launch_bounds__(64 * NT) bwd_fused_kernel(const BwdParams p) {
         SV8 kn;
 #pragma unroll
         for (int j = 0; j < 8; j++) kn[j] = (SE)(x[j] * inv);
-        st8<SV8>(&lds_K[buf][frow * S + fc8], kn);
-        st8<V8>(&lds_V[buf][frow * S + fc8], vv);
-        if ((ln & 3) == 0) lds_kinv[buf][frow] = (sqrtf(ss) > kNormEps) ? inv : -inv;
+        st8<SV8>(lds_K + frow * S + fc8, kn);
+        st8<V8>(lds_V + frow * S + fc8, r.v);
+        if ((ln & 3) == 0) lds_kinv[frow] = (sqrtf(ss) > kNormEps) ? inv : -inv;
     };
 
     // ---- dbias tile of this wavefront's queries, in the layout of the resident tile ----
@@ -267,17 +232,17 @@ __global__ void __launch_bounds__(64 * NT) bwd_fused_kernel(const BwdParams p) {
     // 32-column group, wavefront pairs share a group and take its two interleaved halves
     const int kcol0 = 32 * (wave >> 1) + 4 * (wave & 1);
 
-    __syncthreads();
     Cursor c = first();
     int tile_wi = -1;                      // window index the resident tile was built for
     if (!MASKED) build_tile(0);
-    float lse_next = -INFINITY;
+    Rows nx;
+    nx.k = zero8<V8>(); nx.v = zero8<V8>(); nx.q = zero8<V8>(); nx.dO = zero8<V8>(); nx.o = zero8<V8>();
+    nx.lse = -INFINITY;
     if (valid(c)) {
-        fetch(unit_of(c), lse_next);
-        stage(0);
+        fetch(unit_of(c), nx);
+        stage(nx);
     }
     __syncthreads();
-    int cur = 0;
     float ds_acc = 0.f;        // sum over this lane's queries of q_hat . dq_hat
 
     while (valid(c)) {
@@ -295,9 +260,7 @@ __global__ void __launch_bounds__(64 * NT) bwd_fused_kernel(const BwdParams p) {
         f32x4 ndv, dqacc[2];
         float nl, inv;
         {
-            const V8 qcur = ld8<V8>(lds_rawQ + qrow * 32 + 8 * g);
-            const V8 docur = ld8<V8>(lds_rawDO + qrow * 32 + 8 * g);
-            const V8 ocur = ld8<V8>(lds_rawO + qrow * 32 + 8 * g);
+            const V8 qcur = nx.q, docur = nx.dO, ocur = nx.o;
             float x[8];
             unpack8(qcur, x);
             float ss = 0.f, dl = 0.f;
@@ -309,7 +272,7 @@ __global__ void __launch_bounds__(64 * NT) bwd_fused_kernel(const BwdParams p) {
             const float sc = scale2 * inv;
 #pragma unroll
             for (int j = 0; j < 8; j++) bq[j] = (SE)(x[j] * sc);
-            const float lse = lse_next;
+            const float lse = nx.lse;
             // fully masked row (lse = -inf): P = 0
             nl = (lse == -INFINITY) ? -INFINITY : m_fixed - lse * kLog2e;
             float nd;
@@ -329,10 +292,10 @@ __global__ void __launch_bounds__(64 * NT) bwd_fused_kernel(const BwdParams p) {
             st8<SV8>(lds_Qs + qrow * S + 8 * g, bq);
             st8<V8>(lds_dOs + qrow * S + 8 * g, bd);
         }
-        if (more) fetch(unit_of(cn), lse_next);      // in flight while this unit is computed
+        if (more) fetch(unit_of(cn), nx);      // in flight while this unit is computed
 
-        const SE* Kb = &lds_K[cur][0];
-        const E* Vb = &lds_V[cur][0];
+        const SE* Kb = lds_K;
+        const E* Vb = lds_V;
 
         // ---- phase A ----
         auto group = [&](int kp, bool folded) __attribute__((always_inline)) {
@@ -398,7 +361,16 @@ __global__ void __launch_bounds__(64 * NT) bwd_fused_kernel(const BwdParams p) {
             }
         }
 
-        __syncthreads();       // e, dZ, q_hat and dO tiles of every wavefront are complete
+        // k_hat row and 1/|k| of this lane's phase-B key, taken while the K tile is still this unit's
+        int ln3 = lane;
+        asm volatile("" : "+v"(ln3));
+        const int n16 = ln3 & 15, g3 = ln3 >> 4;
+        const int key = kcol0 + 8 * (n16 >> 2) + (n16 & 3);
+        const SV8 krow8 = ld8<SV8>(Kb + key * S + 8 * g3);
+        const float ki = lds_kinv[key];
+
+        __syncthreads();       // e, dZ, q_hat and dO tiles of every wavefront are complete; K / V tiles are free
+        if (more) stage(nx);   // the next unit's k, v rows have had phase A to arrive
 
         // ---- phase B: this wavefront's 16 keys against all queries ----
         {
@@ -425,24 +397,15 @@ __global__ void __launch_bounds__(64 * NT) bwd_fused_kernel(const BwdParams p) {
                 }
             }
             // epilogue dk, dv: lane (key, g) holds d = 8g + 4dt + i (16 bytes of a row)
-            int ln3 = lane;
-            asm volatile("" : "+v"(ln3));
-            const int n16 = ln3 & 15, g3 = ln3 >> 4;
-            const int key = kcol0 + 8 * (n16 >> 2) + (n16 & 3);
             float x[8], a[8];
             float dot = 0.f;
 #pragma unroll
-            for (int dt = 0; dt < 2; dt++) {
-                const SV4 k4 = *reinterpret_cast<const SV4*>(Kb + key * S + 8 * g3 + 4 * dt);
-#pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    x[4 * dt + i] = (float)k4[i];
-                    a[4 * dt + i] = dkacc[dt][i] * kLn2;      // undo the log2e folded into q_hat
-                    dot += a[4 * dt + i] * x[4 * dt + i];
-                }
+            for (int j = 0; j < 8; j++) {
+                x[j] = (float)krow8[j];
+                a[j] = dkacc[j >> 2][j & 3] * kLn2;      // undo the log2e folded into q_hat
+                dot += a[j] * x[j];
             }
             dot = xor32_add(xor16_add(dot));
-            const float ki = lds_kinv[cur][key];
             const float kinv = fabsf(ki);
             const float proj = ki > 0.f ? dot : 0.f;
             if (key < N) {
@@ -459,9 +422,7 @@ __global__ void __launch_bounds__(64 * NT) bwd_fused_kernel(const BwdParams p) {
             }
         }
 
-        if (more) stage(cur ^ 1);
         __syncthreads();       // next unit staged; everybody is done with this unit's tiles
-        cur ^= 1;
         c = cn;
     }
 
