@@ -26,7 +26,7 @@
 namespace fwa2 {
 
 template <int DT, bool HAS_BIAS, int MASK_DT, int NT, bool VEC, bool MASKED>
-__global__ void __launch_bounds__(64 * NT) bwd_fused_kernel(const BwdParams p) {
+__global__ void __launch_bounds__(64 * NT, 3) bwd_fused_kernel(const BwdParams p) {
     typedef typename Elem<DT>::E E;
     typedef typename Elem<DT>::V8 V8;
     typedef typename Elem<DT>::V4 V4;
