@@ -20,6 +20,40 @@ def _t4(t):
     return _abi.Tensor4(t.data_ptr(), t.stride(0), t.stride(1), t.stride(2))
 
 
+def _set_t4(dst, t):
+    st = t.stride()
+    dst.ptr, dst.stride_bw, dst.stride_h, dst.stride_n = t.data_ptr(), st[0], st[1], st[2]
+
+
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_get_device = getattr(torch._C, "_cuda_getDevice", None)
+
+
+class _on_device:
+    """Make `device` current for the duration of a library call and hand back the raw handle of its
+    current stream.  The common case (the device is current already) costs two C calls; only a
+    different device goes through torch's device guard."""
+
+    __slots__ = ("index", "guard")
+
+    def __init__(self, device):
+        self.index = device.index if device.index is not None else torch.cuda.current_device()
+        self.guard = None
+
+    def __enter__(self):
+        if _get_device is None or _get_device() != self.index:
+            self.guard = torch.cuda.device(self.index)
+            self.guard.__enter__()
+        if _raw_stream is not None:
+            return _raw_stream(self.index)
+        return torch.cuda.current_stream(self.index).cuda_stream
+
+    def __exit__(self, *exc):
+        if self.guard is not None:
+            self.guard.__exit__(*exc)
+        return False
+
+
 def _rows_16b_aligned(t):
     return t.stride(-1) == 1 and t.data_ptr() % 16 == 0 and all(s % 8 == 0 for s in t.stride()[:-1])
 
@@ -38,9 +72,9 @@ def mask_window_flags(mask):
         return cached[1]
     lib = _abi.load()
     live = torch.empty(mask.shape[0], dtype=torch.uint8, device=mask.device)
-    with torch.cuda.device(mask.device):
+    with _on_device(mask.device) as stream:
         st = lib.fwa2_mask_scan(mask.data_ptr(), _DTYPES[mask.dtype], mask.shape[0], mask.shape[1], mask.stride(0),
-                                mask.stride(1), live.data_ptr(), torch.cuda.current_stream().cuda_stream)
+                                mask.stride(1), live.data_ptr(), stream)
     _abi.check(st, "fwa2_mask_scan")
     try:
         mask._fwa2_live = (mask._version, live)
@@ -56,13 +90,13 @@ def _describe(q, k, v, o, lse, logit_scale, bias, mask, mask_live, scale_type):
     p.scale_kind = _abi.SCALE_TENSOR if scale_type == "tensor" else _abi.SCALE_DEFAULT
     p.bw, p.heads, p.n, p.head_dim = bw, heads, n, d
     p.n_windows = mask.shape[0] if mask is not None else 1
-    p.q, p.k, p.v, p.o = _t4(q), _t4(k), _t4(v), _t4(o)
+    _set_t4(p.q, q); _set_t4(p.k, k); _set_t4(p.v, v); _set_t4(p.o, o)
     if scale_type == "tensor":
         p.logit_scale = logit_scale.data_ptr()
     if bias is not None:
-        p.bias = _abi.Tensor3(bias.data_ptr(), bias.stride(0), bias.stride(1))
+        p.bias.ptr, p.bias.stride_a, p.bias.stride_n = bias.data_ptr(), bias.stride(0), bias.stride(1)
     if mask is not None:
-        p.mask = _abi.Tensor3(mask.data_ptr(), mask.stride(0), mask.stride(1))
+        p.mask.ptr, p.mask.stride_a, p.mask.stride_n = mask.data_ptr(), mask.stride(0), mask.stride(1)
         p.mask_dtype = _DTYPES[mask.dtype]
         if mask_live is not None:
             p.mask_live = mask_live.data_ptr()
@@ -125,8 +159,8 @@ class FlashWindowAttentionV2(torch.autograd.Function):
             o = torch.empty(q.shape, device=q.device, dtype=q.dtype)
         mask_live = mask_window_flags(mask) if mask is not None else None
         p = _describe(q, k, v, o, lse, logit_scale, bias, mask, mask_live, scale_type)
-        with torch.cuda.device(q.device):
-            p.stream = torch.cuda.current_stream().cuda_stream
+        with _on_device(q.device) as stream:
+            p.stream = stream
             _abi.check(lib.fwa2_forward(p), "fwa2_forward")
 
         ctx.save_for_backward(q, k, v, o, lse, logit_scale, bias, mask)
@@ -147,16 +181,16 @@ class FlashWindowAttentionV2(torch.autograd.Function):
 
         lib = _abi.load()
         p = _describe(q, k, v, o, lse, logit_scale, bias, mask, ctx.mask_live, scale_type)
-        p.d_o, p.dq, p.dk, p.dv = _t4(do), _t4(dq), _t4(dk), _t4(dv)
+        _set_t4(p.d_o, do); _set_t4(p.dq, dq); _set_t4(p.dk, dk); _set_t4(p.dv, dv)
         if db is not None:
             p.dbias = db.data_ptr()
         if dscale is not None:
             p.dscale = dscale.data_ptr()
-        with torch.cuda.device(q.device):
+        with _on_device(q.device) as stream:
             need = lib.fwa2_backward_workspace_bytes(p)
             ws = torch.empty(max(need, 1), dtype=torch.uint8, device=q.device)
             p.workspace, p.workspace_bytes = ws.data_ptr(), need
-            p.stream = torch.cuda.current_stream().cuda_stream
+            p.stream = stream
             _abi.check(lib.fwa2_backward(p), "fwa2_backward")
         return dq, dk, dv, dscale, db, None
 
@@ -196,8 +230,8 @@ class FlashWindowAttentionV2QKVPacked(torch.autograd.Function):
         out = torch.empty((bw, n, heads, d), device=q.device, dtype=q.dtype)
         mask_live = mask_window_flags(mask) if mask is not None else None
         p = _describe(q, k, v, out.transpose(1, 2), lse, logit_scale, bias, mask, mask_live, scale_type)
-        with torch.cuda.device(q.device):
-            p.stream = torch.cuda.current_stream().cuda_stream
+        with _on_device(q.device) as stream:
+            p.stream = stream
             _abi.check(lib.fwa2_forward(p), "fwa2_forward")
 
         ctx.save_for_backward(qkv, out, lse, logit_scale, bias, mask)
@@ -220,16 +254,16 @@ class FlashWindowAttentionV2QKVPacked(torch.autograd.Function):
 
         lib = _abi.load()
         p = _describe(q, k, v, out.transpose(1, 2), lse, logit_scale, bias, mask, ctx.mask_live, scale_type)
-        p.d_o, p.dq, p.dk, p.dv = _t4(do), _t4(dq), _t4(dk), _t4(dv)
+        _set_t4(p.d_o, do); _set_t4(p.dq, dq); _set_t4(p.dk, dk); _set_t4(p.dv, dv)
         if db is not None:
             p.dbias = db.data_ptr()
         if dscale is not None:
             p.dscale = dscale.data_ptr()
-        with torch.cuda.device(qkv.device):
+        with _on_device(qkv.device) as stream:
             need = lib.fwa2_backward_workspace_bytes(p)
             ws = torch.empty(max(need, 1), dtype=torch.uint8, device=qkv.device)
             p.workspace, p.workspace_bytes = ws.data_ptr(), need
-            p.stream = torch.cuda.current_stream().cuda_stream
+            p.stream = stream
             _abi.check(lib.fwa2_backward(p), "fwa2_backward")
         return dqkv, dscale, db, None
 
@@ -250,9 +284,9 @@ class CpbBias(torch.autograd.Function):
         n = wh * ww
         bias = torch.empty((heads, n, n), device=table.device, dtype=table.dtype)
         lib = _abi.load()
-        with torch.cuda.device(table.device):
+        with _on_device(table.device) as stream:
             _abi.check(lib.fwa2_cpb_bias_forward(table.data_ptr(), _DTYPES[table.dtype], heads, wh, ww, bias.data_ptr(),
-                                                 torch.cuda.current_stream().cuda_stream), "fwa2_cpb_bias_forward")
+                                                 stream), "fwa2_cpb_bias_forward")
         ctx.save_for_backward(table)
         ctx.window = (wh, ww)
         return bias
@@ -264,8 +298,8 @@ class CpbBias(torch.autograd.Function):
         dbias = dbias.contiguous()
         dtable = torch.empty_like(table)
         lib = _abi.load()
-        with torch.cuda.device(table.device):
+        with _on_device(table.device) as stream:
             _abi.check(lib.fwa2_cpb_bias_backward(table.data_ptr(), dbias.data_ptr(), _DTYPES[table.dtype], table.shape[1],
-                                                  wh, ww, dtable.data_ptr(), torch.cuda.current_stream().cuda_stream),
+                                                  wh, ww, dtable.data_ptr(), stream),
                        "fwa2_cpb_bias_backward")
         return dtable, None, None
