@@ -63,14 +63,6 @@ struct BwdLds {
     float* rawLse;
 };
 
-// Lane index recomputed on the spot (two VALU instructions, never hoisted): what is derived from it
-// need not stay in a register, or in scratch, across the phases of a unit.
-__device__ __forceinline__ int lane_now() {
-    int l;
-    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(l));
-    return l;
-}
-
 // 16 bytes per lane straight from global memory into LDS (no registers held while in flight):
 // lane i of the wavefront lands at lds_wave_base + 16 i.
 template <class E>
@@ -625,6 +617,7 @@ void dq_geometry(int n, int* waves, int* chunks);
 hipError_t launch_backward_dq(const BwdParams& p, int dtype, bool has_bias, int mask_dt, hipStream_t st);
 int backward_dq_resident_supported(int n);
 int backward_fused_supported(int n);
+
 hipError_t launch_backward_fused(const BwdParams& p, int dtype, bool has_bias, int mask_dt, hipStream_t st,
                                  int max_groups, int* parts_out);
 hipError_t launch_backward_dq_resident(const BwdParams& p, int dtype, bool has_bias, int mask_dt, hipStream_t st,

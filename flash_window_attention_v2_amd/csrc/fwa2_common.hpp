@@ -111,6 +111,14 @@ __device__ __forceinline__ float quad_add(float x) {
     return x + y;
 }
 
+// Lane index recomputed on the spot (two VALU instructions, never hoisted): what is derived from it
+// need not stay in a register, or in scratch, across the phases of a unit.
+__device__ __forceinline__ int lane_now() {
+    int l;
+    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(l));
+    return l;
+}
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
