@@ -422,14 +422,15 @@ static int resident_fit(K kern, int threads) {
 }
 
 // Launches the kernel(s) and reports how many dscale partials per head they wrote.
-template <int DT, bool HAS_BIAS, int MASK_DT, int NT, bool VEC>
+// SUBP: 16-row query tiles per wavefront in the launch over the unmasked units; the masked launch always
+// uses kDqSub (its tile rebuilds leave no room in 128 registers).
+template <int DT, bool HAS_BIAS, int MASK_DT, int NT, bool VEC, int SUBP = kDqSub>
 static hipError_t launch_nt(BwdParams p, hipStream_t st, int max_groups, int* ds_parts_out) {
-    constexpr int SUB = kDqSub;
-    const int waves = (p.n + 16 * SUB - 1) / (16 * SUB);
+    constexpr int SUBM = kDqSub;
     static const int fit_plain =
-        resident_fit(bwd_dq_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, false, SUB>, 64 * NT / SUB);
+        resident_fit(bwd_dq_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, false, SUBP>, 64 * NT / SUBP);
     static const int fit_masked =
-        MASK_DT >= 0 ? resident_fit(bwd_dq_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, true, SUB>, 64 * NT / SUB) : 1;
+        MASK_DT >= 0 ? resident_fit(bwd_dq_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, true, SUBM>, 64 * NT / SUBM) : 1;
     auto groups_for = [&](int fit) {
         int groups = (p.cus * fit) / p.heads;
         if (groups < 1) groups = 1;
@@ -444,14 +445,14 @@ static hipError_t launch_nt(BwdParams p, hipStream_t st, int max_groups, int* ds
     if (g_plain) {
         p.dq_groups = g_plain;
         p.ds_slot0 = 0;
-        hipLaunchKernelGGL((bwd_dq_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, false, SUB>), dim3(p.heads * g_plain),
-                           dim3(64 * waves), 0, st, p);
+        hipLaunchKernelGGL((bwd_dq_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, false, SUBP>), dim3(p.heads * g_plain),
+                           dim3(64 * ((p.n + 16 * SUBP - 1) / (16 * SUBP))), 0, st, p);
     }
     if (g_masked) {
         p.dq_groups = g_masked;
         p.ds_slot0 = g_plain;
-        hipLaunchKernelGGL((bwd_dq_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, true, SUB>), dim3(p.heads * g_masked),
-                           dim3(64 * waves), 0, st, p);
+        hipLaunchKernelGGL((bwd_dq_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, true, SUBM>), dim3(p.heads * g_masked),
+                           dim3(64 * ((p.n + 16 * SUBM - 1) / (16 * SUBM))), 0, st, p);
     }
     *ds_parts_out = p.ds_parts;
     return hipGetLastError();
@@ -463,10 +464,13 @@ static hipError_t launch_mask(const BwdParams& p, hipStream_t st, int mg, int* o
     if (p.side_vec) {
         if (nt == 4) return launch_nt<DT, HAS_BIAS, MASK_DT, 4, true>(p, st, mg, out);
         if (nt == 8) return launch_nt<DT, HAS_BIAS, MASK_DT, 8, true>(p, st, mg, out);
+        // 129 .. 160 tokens: 16 rows per wavefront give nine or ten wavefronts instead of five
+        if (p.n <= 160) return launch_nt<DT, HAS_BIAS, MASK_DT, 16, true, 1>(p, st, mg, out);
         return launch_nt<DT, HAS_BIAS, MASK_DT, 16, true>(p, st, mg, out);
     }
     if (nt == 4) return launch_nt<DT, HAS_BIAS, MASK_DT, 4, false>(p, st, mg, out);
     if (nt == 8) return launch_nt<DT, HAS_BIAS, MASK_DT, 8, false>(p, st, mg, out);
+    if (p.n <= 160) return launch_nt<DT, HAS_BIAS, MASK_DT, 16, false, 1>(p, st, mg, out);
     return launch_nt<DT, HAS_BIAS, MASK_DT, 16, false>(p, st, mg, out);
 }
 
