@@ -126,3 +126,25 @@ def test_function_rejects_bad_arguments_on_cpu():
         flash_win_attn_v2_func(q, q.half(), q)
     with pytest.raises(AssertionError):            # logit_scale must be a tensor
         flash_win_attn_v2_func(q, q, q, 1.0)
+
+
+def test_header_compiles_as_c_and_cxx(tmp_path):
+    """include/fwa2.h is the boundary a C or C++ host binds: it must be self-contained in both languages
+    and lay the problem struct out exactly as the ctypes mirror does."""
+    import shutil
+    import subprocess
+    if shutil.which("gcc") is None or shutil.which("g++") is None:
+        pytest.skip("no host compiler")
+    src = tmp_path / "use_header.c"
+    src.write_text(
+        '#include "fwa2.h"\n#include <stdio.h>\n'
+        'int main(void) { fwa2_problem p; (void)p; printf("%zu %zu %zu\\n", sizeof(fwa2_problem), '
+        'sizeof(fwa2_tensor4), sizeof(fwa2_tensor3)); return 0; }\n')
+    inc = os.path.join(ROOT, "include")
+    exe = tmp_path / "use_header"
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-pedantic", "-I", inc, str(src), "-o", str(exe)], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()
+    assert [int(x) for x in out] == [ctypes.sizeof(_abi.Problem), ctypes.sizeof(_abi.Tensor4), ctypes.sizeof(_abi.Tensor3)]
+    cxx = tmp_path / "use_header.cpp"
+    cxx.write_text('#include "fwa2.h"\nint main() { fwa2_problem p{}; return p.n; }\n')
+    subprocess.run(["g++", "-std=c++17", "-Wall", "-Werror", "-I", inc, "-fsyntax-only", str(cxx)], check=True)
