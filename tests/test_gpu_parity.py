@@ -245,6 +245,35 @@ def test_strided_qkv_views_like_swin():
         assert _rel(got[i], ref[name]) <= 5e-2, name
 
 
+@pytest.mark.parametrize("n,res,win,shift", [(64, 16, 8, 4), (256, 32, 16, 8)])
+def test_every_tensor_with_its_own_strides(n, res, win, shift):
+    """q in [BW, N, H, d] order, k in [BW, H, N, d] with padded rows, v as a slice of a wider tensor, dO
+    transposed: the kernels take each tensor's own element strides (flash_window_attention_v2.py:20)."""
+    dtype = torch.bfloat16
+    heads, n_w = 3, (res // win) ** 2
+    inp = make_inputs(batch=2, n_windows=n_w, heads=heads, n=n, dtype=dtype, seed=31, resolution=res, window=win, shift=shift)
+    ref = classic_fwd_bwd(inp["q"], inp["k"], inp["v"], inp["logit_scale"], inp["bias"], inp["mask"], inp["do"])
+    dev = _to_dev(inp)
+    bw = inp["q"].shape[0]
+    q_store = dev["q"].detach().transpose(1, 2).contiguous().requires_grad_(True)            # [BW, N, H, d]
+    k_store = torch.zeros(bw, heads, n, 40, device="cuda", dtype=dtype)
+    k_store[..., :32] = dev["k"].detach()
+    k_store.requires_grad_(True)
+    v_store = torch.zeros(bw, heads + 1, n, 32, device="cuda", dtype=dtype)
+    v_store[:, 1:] = dev["v"].detach()
+    v_store.requires_grad_(True)
+    q, k, v = q_store.transpose(1, 2), k_store[..., :32], v_store[:, 1:]
+    assert not q.is_contiguous() and not k.is_contiguous() and not v.is_contiguous()
+    o = _func()(q, k, v, dev["logit_scale"], dev["bias"], dev["mask"])
+    do = dev["do"].transpose(1, 2).contiguous().transpose(1, 2)                                # non-contiguous dO
+    o.backward(do)
+    assert float((o.detach().float().cpu() - ref["o"]).abs().max()) <= 2e-2
+    assert _rel(q_store.grad.transpose(1, 2), ref["dq"]) <= 5e-2
+    assert _rel(k_store.grad[..., :32], ref["dk"]) <= 5e-2 and float(k_store.grad[..., 32:].abs().max()) == 0.0
+    assert _rel(v_store.grad[:, 1:], ref["dv"]) <= 5e-2 and float(v_store.grad[:, 0].abs().max()) == 0.0
+    assert _rel(dev["bias"].grad, ref["dbias"]) <= 5e-2
+
+
 def test_packed_qkv_entry_point():
     """`flash_win_attn_v2_qkvpacked_func` on the [B_, N, 3, H, d] projection output: the same kernels as
     the three-view call, so o and the packed gradient must be bit-identical to it; both are also held
