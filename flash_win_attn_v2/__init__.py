@@ -4,8 +4,9 @@ The submodule names of the reference are aliased too."""
 import sys
 
 import flash_window_attention_v2_amd as _impl
-from flash_window_attention_v2_amd import (FlashWindowAttentionV2, FlashWindowAttentionV2QKVPacked,
-                                           SwinTransformerV2, WindowAttention, flash_win_attn_v2_func,
+from flash_window_attention_v2_amd import (FlashWindowAttentionV2, FlashWindowAttentionV2Grid,
+                                           FlashWindowAttentionV2QKVPacked, SwinTransformerV2, WindowAttention,
+                                           flash_win_attn_v2_func, flash_win_attn_v2_grid_func,
                                            flash_win_attn_v2_qkvpacked_func, win_attention_torch,
                                            win_attention_torch_compile)
 from flash_window_attention_v2_amd import flash_window_attention_v2, swin_transformer_v2, win_attention_func

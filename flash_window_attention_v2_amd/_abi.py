@@ -9,7 +9,7 @@ import ctypes
 import os
 import threading
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 OK, ERR_INVALID_ARGUMENT, ERR_UNSUPPORTED, ERR_HIP, ERR_NO_DEVICE = range(5)
 F16, BF16, F32 = 0, 1, 2
@@ -55,6 +55,9 @@ class Problem(ctypes.Structure):
         ("dbias", ctypes.c_void_p), ("dscale", ctypes.c_void_p),
         ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
         ("stream", ctypes.c_void_p),
+        ("grid_h", ctypes.c_int32), ("grid_w", ctypes.c_int32),
+        ("win_h", ctypes.c_int32), ("win_w", ctypes.c_int32),
+        ("shift_h", ctypes.c_int32), ("shift_w", ctypes.c_int32),
     ]
 
 

@@ -92,6 +92,23 @@ int validate(const fwa2_problem* p, int backward) {
         if (p->mask.stride_n < p->n)
             return fail(FWA2_ERR_INVALID_ARGUMENT, "mask: row stride %lld < n", (long long)p->mask.stride_n);
     }
+    if (p->grid_h != 0 || p->grid_w != 0 || p->win_h != 0 || p->win_w != 0 || p->shift_h != 0 || p->shift_w != 0) {
+        if (p->grid_h <= 0 || p->grid_w <= 0 || p->win_h <= 0 || p->win_w <= 0 || p->grid_h % p->win_h || p->grid_w % p->win_w)
+            return fail(FWA2_ERR_INVALID_ARGUMENT, "window map: the %d x %d grid is not a whole number of %d x %d windows",
+                        p->grid_h, p->grid_w, p->win_h, p->win_w);
+        if (p->n != p->win_h * p->win_w)
+            return fail(FWA2_ERR_INVALID_ARGUMENT, "window map: n = %d is not win_h * win_w", p->n);
+        if (p->shift_h < 0 || p->shift_h >= p->grid_h || p->shift_w < 0 || p->shift_w >= p->grid_w)
+            return fail(FWA2_ERR_INVALID_ARGUMENT, "window map: shifts must lie in [0, grid extent)");
+        const int nw = (p->grid_h / p->win_h) * (p->grid_w / p->win_w);
+        if (p->bw % nw) return fail(FWA2_ERR_INVALID_ARGUMENT, "window map: bw %d is not a multiple of %d windows per image", p->bw, nw);
+        if (p->mask.ptr && p->n_windows != nw)
+            return fail(FWA2_ERR_INVALID_ARGUMENT, "window map: mask has %d windows, the grid %d", p->n_windows, nw);
+        if (p->win_w > 64 || p->n > 256)
+            return fail(FWA2_ERR_UNSUPPORTED, "window map: windows of more than 256 tokens are not supported");
+        if (backward && p->n > fwa2::kMapBackwardMaxN)
+            return fail(FWA2_ERR_UNSUPPORTED, "window map: backward supports windows of up to %d tokens", fwa2::kMapBackwardMaxN);
+    }
     if (p->lse == nullptr) return fail(FWA2_ERR_INVALID_ARGUMENT, "lse: null pointer");
     if (p->lse_stride_h < p->n) return fail(FWA2_ERR_INVALID_ARGUMENT, "lse: head stride %lld < n", (long long)p->lse_stride_h);
     if (backward) {
@@ -110,6 +127,20 @@ int validate(const fwa2_problem* p, int backward) {
             return fail(FWA2_ERR_INVALID_ARGUMENT, "workspace must be 256-byte aligned");
     }
     return FWA2_OK;
+}
+
+fwa2::WinMap to_map(const fwa2_problem* p) {
+    fwa2::WinMap m;
+    memset(&m, 0, sizeof(m));
+    if (p->grid_h > 0) {
+        m.nwx = p->grid_w / p->win_w;
+        m.nw = (p->grid_h / p->win_h) * m.nwx;
+        m.gh = p->grid_h; m.gw = p->grid_w;
+        m.wh = p->win_h; m.ww = p->win_w;
+        m.sh = p->shift_h; m.sw = p->shift_w;
+        m.inv_ww = 65536 / p->win_w + 1;
+    }
+    return m;
 }
 
 bool row_vec_ok(const void* ptr, int64_t sa, int64_t sn, int n) {
@@ -186,6 +217,7 @@ int fwa2_forward(const fwa2_problem* p) {
     fwa2::FwdParams k;
     memset(&k, 0, sizeof(k));
     k.q = to_t4(p->q); k.k = to_t4(p->k); k.v = to_t4(p->v); k.o = to_t4(p->o);
+    k.map = to_map(p);
     k.logit_scale = p->logit_scale;
     k.bias = p->bias.ptr; k.bias_sh = p->bias.stride_a; k.bias_sn = p->bias.stride_n;
     k.mask = p->mask.ptr; k.mask_sw = p->mask.stride_a; k.mask_sn = p->mask.stride_n;
@@ -212,6 +244,7 @@ int fwa2_backward(const fwa2_problem* p) {
     memset(&k, 0, sizeof(k));
     k.q = to_t4(p->q); k.k = to_t4(p->k); k.v = to_t4(p->v); k.o = to_t4(p->o);
     k.d_o = to_t4(p->d_o); k.dq = to_t4(p->dq); k.dk = to_t4(p->dk); k.dv = to_t4(p->dv);
+    k.map = to_map(p);
     k.logit_scale = p->logit_scale;
     k.bias = p->bias.ptr; k.bias_sh = p->bias.stride_a; k.bias_sn = p->bias.stride_n;
     k.mask = p->mask.ptr; k.mask_sw = p->mask.stride_a; k.mask_sn = p->mask.stride_n;

@@ -25,7 +25,8 @@
 
 namespace fwa2 {
 
-template <int DT, bool HAS_BIAS, int MASK_DT, int NT, bool VEC, bool MASKED>
+// MAPPED: rows are addressed through the window map (cyclic shift + window partition done here).
+template <int DT, bool HAS_BIAS, int MASK_DT, int NT, bool VEC, bool MASKED, bool MAPPED>
 __global__ void __launch_bounds__(64 * NT, 3) bwd_fused_kernel(const BwdParams p) {
     typedef typename Elem<DT>::E E;
     typedef typename Elem<DT>::V8 V8;
@@ -185,7 +186,7 @@ __global__ void __launch_bounds__(64 * NT, 3) bwd_fused_kernel(const BwdParams p
     // query in the operand layout (lane (query, g) takes columns 8g .. 8g+7); rows >= n read as zeros ----
     struct Rows { V8 k, v, q, dO, o; float lse; };
     auto ldrow = [&](const T4& t, int b, int row, int col) -> V8 {
-        return ld8<V8>(reinterpret_cast<const E*>(t.ptr) + b * t.sb + h * t.sh + (int64_t)row * t.sn + col);
+        return ld8<V8>(reinterpret_cast<const E*>(t.ptr) + row_off<MAPPED>(t, p.map, b, h, row) + col);
     };
     auto fetch = [&](int b, Rows& r) __attribute__((always_inline)) {
         int ln = lane;                     // re-derived per call: no address lives across the unit loop
@@ -352,7 +353,7 @@ __global__ void __launch_bounds__(64 * NT, 3) bwd_fused_kernel(const BwdParams p
             const float f = s_true * inv;
             const int q = wave * 16 + (ln2 & 15);
             if (q < N) {
-                E* dqrow = reinterpret_cast<E*>(const_cast<void*>(p.dq.ptr)) + b * p.dq.sb + h * p.dq.sh + (int64_t)q * p.dq.sn;
+                E* dqrow = reinterpret_cast<E*>(const_cast<void*>(p.dq.ptr)) + row_off<MAPPED>(p.dq, p.map, b, h, q);
                 V8 o8;
 #pragma unroll
                 for (int j = 0; j < 8; j++) o8[j] = (E)(f * (dqacc[j >> 2][j & 3] - qh[j] * proj));
@@ -409,8 +410,8 @@ __global__ void __launch_bounds__(64 * NT, 3) bwd_fused_kernel(const BwdParams p
             const float kinv = fabsf(ki);
             const float proj = ki > 0.f ? dot : 0.f;
             if (key < N) {
-                E* dkp = reinterpret_cast<E*>(const_cast<void*>(p.dk.ptr)) + b * p.dk.sb + h * p.dk.sh + (int64_t)key * p.dk.sn;
-                E* dvp = reinterpret_cast<E*>(const_cast<void*>(p.dv.ptr)) + b * p.dv.sb + h * p.dv.sh + (int64_t)key * p.dv.sn;
+                E* dkp = reinterpret_cast<E*>(const_cast<void*>(p.dk.ptr)) + row_off<MAPPED>(p.dk, p.map, b, h, key);
+                E* dvp = reinterpret_cast<E*>(const_cast<void*>(p.dv.ptr)) + row_off<MAPPED>(p.dv, p.map, b, h, key);
                 V8 o8, v8;
 #pragma unroll
                 for (int j = 0; j < 8; j++) {
@@ -463,14 +464,14 @@ static int resident_fit(K kern, int threads) {
 }
 
 // Launches the kernel(s); reports how many partial tiles / dscale partials per head they wrote.
-template <int DT, bool HAS_BIAS, int MASK_DT, bool VEC>
-static hipError_t launch_vec(BwdParams p, hipStream_t st, int max_groups, int* parts_out) {
+template <int DT, bool HAS_BIAS, int MASK_DT, bool VEC, bool MAPPED>
+static hipError_t launch_map(BwdParams p, hipStream_t st, int max_groups, int* parts_out) {
     constexpr int NT = 4;
     // wavefront pairs share a 32-key group in phase B, so there is always an even number of them
     const int waves = 2 * ((p.n + 31) / 32);
-    static const int fit_plain = resident_fit(bwd_fused_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, false>, 64 * NT);
+    static const int fit_plain = resident_fit(bwd_fused_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, false, MAPPED>, 64 * NT);
     static const int fit_masked =
-        MASK_DT >= 0 ? resident_fit(bwd_fused_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, true>, 64 * NT) : 1;
+        MASK_DT >= 0 ? resident_fit(bwd_fused_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, true, MAPPED>, 64 * NT) : 1;
     auto groups_for = [&](int fit) {
         int groups = (p.cus * fit) / p.heads;
         if (groups < 1) groups = 1;
@@ -486,18 +487,24 @@ static hipError_t launch_vec(BwdParams p, hipStream_t st, int max_groups, int* p
     if (g_plain) {
         p.dq_groups = g_plain;
         p.ds_slot0 = p.db_slot0 = 0;
-        hipLaunchKernelGGL((bwd_fused_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, false>), dim3(p.heads * g_plain),
+        hipLaunchKernelGGL((bwd_fused_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, false, MAPPED>), dim3(p.heads * g_plain),
                            dim3(64 * waves), 0, st, p);
     }
     if (g_masked) {
         p.dq_groups = g_masked;
         p.ds_slot0 = p.db_slot0 = g_plain;
-        hipLaunchKernelGGL((bwd_fused_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, true>), dim3(p.heads * g_masked),
+        hipLaunchKernelGGL((bwd_fused_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, true, MAPPED>), dim3(p.heads * g_masked),
                            dim3(64 * waves), 0, st, p);
     }
     if (p.ev_stop) (void)hipEventRecord(p.ev_stop, st);
     *parts_out = p.ds_parts;
     return hipGetLastError();
+}
+
+template <int DT, bool HAS_BIAS, int MASK_DT, bool VEC>
+static hipError_t launch_vec(const BwdParams& p, hipStream_t st, int max_groups, int* parts_out) {
+    if (p.map.nw > 0) return launch_map<DT, HAS_BIAS, MASK_DT, VEC, true>(p, st, max_groups, parts_out);
+    return launch_map<DT, HAS_BIAS, MASK_DT, VEC, false>(p, st, max_groups, parts_out);
 }
 
 template <int DT, bool HAS_BIAS, int MASK_DT>

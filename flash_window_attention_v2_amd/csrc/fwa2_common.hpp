@@ -206,6 +206,7 @@ __device__ __forceinline__ auto load_raw8(const T* row, int c0, int n, float pad
 // not push the bias / mask tables (re-read by every unit) out of the L2.
 constexpr int kStreamPolicy = 2;
 
+constexpr int kMapBackwardMaxN = 64;   // largest window the backward kernels address through a window map
 constexpr int kKeyChunk = 256;   // keys staged in LDS at a time by the query-owning kernels
 constexpr int kLdsStride = 40;   // elements per staged row (32 + 8 pad): 80-byte rows
 
@@ -214,8 +215,34 @@ struct T4 {
     const void* ptr;
     int64_t sb, sh, sn;
 };
+// Window partition and cyclic shift as address arithmetic (nw == 0: off, tensors are [BW, H, N, d]).
+// With a map, q / k / v / o (and the gradients) are token grids [B, gh * gw, ...]: T4::sb is the stride
+// between images, T4::sn the stride between consecutive tokens of the row-major grid, and row n = r ww + c
+// of window w = wy nwx + wx of an image sits at grid position ((wy wh + r + sh) mod gh, (wx ww + c + sw) mod gw).
+struct WinMap {
+    int nw, nwx;        // windows per image, windows per grid row
+    int gh, gw;         // token grid of one image
+    int wh, ww;         // window extents
+    int sh, sw;         // cyclic shift (0 <= sh < gh, 0 <= sw < gw)
+    int inv_ww;         // 65536 / ww + 1: n / ww == (n * inv_ww) >> 16 for n * ww < 65536
+};
+// Element offset of row `row` of unit b, head h.  b is uniform, so the two divisions are scalar work.
+template <bool MAPPED>
+__device__ __forceinline__ int64_t row_off(const T4& t, const WinMap& m, int b, int h, int row) {
+    if (!MAPPED) return b * t.sb + h * t.sh + (int64_t)row * t.sn;
+    const int img = b / m.nw, w = b - img * m.nw;
+    const int wy = w / m.nwx, wx = w - wy * m.nwx;
+    const int r = (row * m.inv_ww) >> 16, c = row - r * m.ww;
+    int y = wy * m.wh + r + m.sh;
+    int x = wx * m.ww + c + m.sw;
+    y -= y >= m.gh ? m.gh : 0;
+    x -= x >= m.gw ? m.gw : 0;
+    return img * t.sb + h * t.sh + (int64_t)(y * m.gw + x) * t.sn;
+}
+
 struct FwdParams {
     T4 q, k, v, o;
+    WinMap map;
     const void* logit_scale;
     const void* bias;
     int64_t bias_sh, bias_sn;
@@ -238,6 +265,7 @@ struct FwdParams {
 
 struct BwdParams {
     T4 q, k, v, o, d_o, dq, dk, dv;
+    WinMap map;
     const void* logit_scale;
     const void* bias;
     int64_t bias_sh, bias_sn;

@@ -35,7 +35,8 @@ namespace fwa2 {
 // ceil(N / 16) wavefronts.
 // MASKED: this launch handles the units whose window mask is live; the other units (or all, when
 // there is no mask) go through the MASKED = false instantiation.
-template <int DT, bool HAS_BIAS, int MASK_DT, int NT, bool VEC, bool MASKED>
+// MAPPED: rows are addressed through the window map (cyclic shift + window partition done here).
+template <int DT, bool HAS_BIAS, int MASK_DT, int NT, bool VEC, bool MASKED, bool MAPPED>
 __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p) {
     typedef typename Elem<DT>::E E;
     typedef typename Elem<DT>::V8 V8;
@@ -217,8 +218,8 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
         const int frow = wave * 16 + (ln >> 2);
         const int fc8 = (ln & 3) * 8;
         if (frow < N) {
-            const E* kp = reinterpret_cast<const E*>(p.k.ptr) + b * p.k.sb + h * p.k.sh + (int64_t)frow * p.k.sn + fc8;
-            const E* vp = reinterpret_cast<const E*>(p.v.ptr) + b * p.v.sb + h * p.v.sh + (int64_t)frow * p.v.sn + fc8;
+            const E* kp = reinterpret_cast<const E*>(p.k.ptr) + row_off<MAPPED>(p.k, p.map, b, h, frow) + fc8;
+            const E* vp = reinterpret_cast<const E*>(p.v.ptr) + row_off<MAPPED>(p.v, p.map, b, h, frow) + fc8;
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)kp,
                                              (__attribute__((address_space(3))) void*)(lds_rawK + wave * 16 * 32), 16, 0, kStreamPolicy);
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)vp,
@@ -226,7 +227,7 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
         }
         qq = zero8<V8>();
         const int fq = wave * 16 + (ln & 15);
-        if (fq < N) qq = ld8<V8>(reinterpret_cast<const E*>(p.q.ptr) + b * p.q.sb + h * p.q.sh + (int64_t)fq * p.q.sn + 8 * (ln >> 4));
+        if (fq < N) qq = ld8<V8>(reinterpret_cast<const E*>(p.q.ptr) + row_off<MAPPED>(p.q, p.map, b, h, fq) + 8 * (ln >> 4));
     };
     // landing area -> tiles: K normalised and rounded to fp16, V as is (rows >= n stay zero)
     auto stage = [&](int buf) __attribute__((always_inline)) {
@@ -377,7 +378,7 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
         asm volatile("" : "+v"(ln2));
         const int oq = wave * 16 + (ln2 & 15);
         if (qv) {
-            E* orow = reinterpret_cast<E*>(const_cast<void*>(p.o.ptr)) + b * p.o.sb + h * p.o.sh + (int64_t)oq * p.o.sn;
+            E* orow = reinterpret_cast<E*>(const_cast<void*>(p.o.ptr)) + row_off<MAPPED>(p.o, p.map, b, h, oq);
             V8 ov;
 #pragma unroll
             for (int j = 0; j < 8; j++) ov[j] = (E)(oacc[j >> 2][j & 3] * inv_l);
@@ -404,12 +405,13 @@ static int resident_fit(K kern, int threads) {
     return n;
 }
 
-template <int DT, bool HAS_BIAS, int MASK_DT, int NT, bool VEC>
-static hipError_t launch_nt(FwdParams p, hipStream_t st) {
+template <int DT, bool HAS_BIAS, int MASK_DT, int NT, bool VEC, bool MAPPED>
+static hipError_t launch_map(FwdParams p, hipStream_t st) {
     const int waves = (p.n + 15) / 16;
     // the runtime's figure is for full 64 NT-thread groups; smaller groups only fit better
-    static const int fit_plain = resident_fit(fwd_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, false>, 64 * NT);
-    static const int fit_masked = MASK_DT >= 0 ? resident_fit(fwd_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, true>, 64 * NT) : 1;
+    static const int fit_plain = resident_fit(fwd_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, false, MAPPED>, 64 * NT);
+    static const int fit_masked =
+        MASK_DT >= 0 ? resident_fit(fwd_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, true, MAPPED>, 64 * NT) : 1;
     auto groups_for = [&](int fit) {
         int groups = (p.cus * fit) / p.heads;
         if (groups < 1) groups = 1;
@@ -419,16 +421,22 @@ static hipError_t launch_nt(FwdParams p, hipStream_t st) {
     // units with an all-zero mask (or every unit when there is no mask) ...
     if (MASK_DT < 0 || p.mask_live != nullptr) {
         p.groups = groups_for(fit_plain);
-        hipLaunchKernelGGL((fwd_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, false>), dim3(p.heads * p.groups),
+        hipLaunchKernelGGL((fwd_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, false, MAPPED>), dim3(p.heads * p.groups),
                            dim3(64 * waves), 0, st, p);
     }
     // ... and the units whose mask is live
     if (MASK_DT >= 0) {
         p.groups = groups_for(fit_masked);
-        hipLaunchKernelGGL((fwd_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, true>), dim3(p.heads * p.groups),
+        hipLaunchKernelGGL((fwd_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, true, MAPPED>), dim3(p.heads * p.groups),
                            dim3(64 * waves), 0, st, p);
     }
     return hipGetLastError();
+}
+
+template <int DT, bool HAS_BIAS, int MASK_DT, int NT, bool VEC>
+static hipError_t launch_nt(const FwdParams& p, hipStream_t st) {
+    if (p.map.nw > 0) return launch_map<DT, HAS_BIAS, MASK_DT, NT, VEC, true>(p, st);
+    return launch_map<DT, HAS_BIAS, MASK_DT, NT, VEC, false>(p, st);
 }
 
 template <int DT, bool HAS_BIAS, int MASK_DT>

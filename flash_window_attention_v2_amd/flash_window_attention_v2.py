@@ -83,9 +83,14 @@ def mask_window_flags(mask):
     return live
 
 
-def _describe(q, k, v, o, lse, logit_scale, bias, mask, mask_live, scale_type):
+def _describe(q, k, v, o, lse, logit_scale, bias, mask, mask_live, scale_type, window_map=None):
     bw, heads, n, d = q.shape
     p = _abi.new_problem()
+    if window_map is not None:
+        # q, k, v, o are token grids [B, H, gh * gw, d]; the library partitions them into windows
+        (gh, gw), (wh, ww), (sh, sw) = window_map
+        p.grid_h, p.grid_w, p.win_h, p.win_w, p.shift_h, p.shift_w = gh, gw, wh, ww, sh, sw
+        bw, n = bw * (gh // wh) * (gw // ww), wh * ww
     p.dtype = _DTYPES[q.dtype]
     p.scale_kind = _abi.SCALE_TENSOR if scale_type == "tensor" else _abi.SCALE_DEFAULT
     p.bw, p.heads, p.n, p.head_dim = bw, heads, n, d
@@ -266,6 +271,98 @@ class FlashWindowAttentionV2QKVPacked(torch.autograd.Function):
             p.stream = stream
             _abi.check(lib.fwa2_backward(p), "fwa2_backward")
         return dqkv, dscale, db, None
+
+
+MAPPED_BACKWARD_MAX_N = 64      # largest window whose backward the library addresses through a window map
+
+
+class FlashWindowAttentionV2Grid(torch.autograd.Function):
+    """The packed operator applied to the un-partitioned token grid: the cyclic shift, window_partition,
+    window_reverse and the shift back that surround the attention call in the reference's block
+    (swin_transformer_v2.py:419-441) become address arithmetic inside the kernels, so none of the four
+    copies (nor their four backward copies) is made.  `qkv` is the projection output [B, gh * gw, 3, H, d]
+    of the image tokens in row-major order; the result is [B, gh * gw, H, d] in the same order.  The qkv and
+    output projections act on single tokens, so they commute with the permutation and the caller applies
+    them to the grid.  `shift` is the block's shift_size (the reference rolls by -shift before partitioning).
+    Has no counterpart in the reference."""
+
+    @staticmethod
+    def forward(ctx, qkv, grid, window, shift, logit_scale=None, bias=None, mask=None):
+        (gh, gw), (wh, ww), (sh, sw) = grid, window, shift
+        assert qkv.dim() == 5 and qkv.shape[2] == 3 and qkv.shape[1] == gh * gw, "qkv must be [B, gh * gw, 3, H, d]"
+        assert gh % wh == 0 and gw % ww == 0, "the grid must be a whole number of windows"
+        if not (_rows_16b_aligned(qkv) and qkv.is_contiguous()):
+            qkv = qkv.contiguous()
+        q, k, v = (qkv[:, :, i].transpose(1, 2) for i in range(3))       # [B, H, L, d] views
+        if logit_scale is not None:
+            assert isinstance(logit_scale, torch.Tensor), \
+                "Make sure logit_scale is a tensor if defined in the paramaters."
+            scale_type = "tensor"
+            logit_scale = logit_scale.contiguous()
+        else:
+            scale_type = "scalar"
+            logit_scale = torch.tensor(1.0 / math.sqrt(q.shape[-1]), device=q.device)
+        b, heads, length, d = q.shape
+        n, nw = wh * ww, (gh // wh) * (gw // ww)
+        assert d <= 128, "FlashAttention only support head dimensions up to 128"
+        assert q.dtype in (torch.float16, torch.bfloat16), "Only support fp16 and bf16"
+        assert q.is_cuda, "qkv must be on the GPU"
+        if scale_type == "tensor":
+            assert logit_scale.is_cuda and logit_scale.shape == (heads, 1, 1) and logit_scale.dtype == q.dtype
+        if bias is not None:
+            assert bias.is_cuda and bias.dtype == q.dtype and bias.shape == (heads, n, n)
+            if bias.stride(-1) != 1:
+                bias = bias.contiguous()
+        if mask is not None:
+            assert mask.is_cuda and mask.dtype in (q.dtype, torch.float32)
+            assert mask.shape == (nw, n, n), "mask must be [nW, N, N] with nW the windows of one image"
+            if mask.stride(-1) != 1:
+                mask = mask.contiguous()
+
+        lib = _abi.load()
+        lse = torch.empty((b * nw, heads, (n + 63) // 64 * 64), device=q.device, dtype=torch.float32)
+        out = torch.empty((b, length, heads, d), device=q.device, dtype=q.dtype)
+        mask_live = mask_window_flags(mask) if mask is not None else None
+        window_map = ((gh, gw), (wh, ww), (sh % gh, sw % gw))
+        p = _describe(q, k, v, out.transpose(1, 2), lse, logit_scale, bias, mask, mask_live, scale_type, window_map)
+        with _on_device(q.device) as stream:
+            p.stream = stream
+            _abi.check(lib.fwa2_forward(p), "fwa2_forward")
+
+        ctx.save_for_backward(qkv, out, lse, logit_scale, bias, mask)
+        ctx.scale_type = scale_type
+        ctx.mask_live = mask_live
+        ctx.window_map = window_map
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        qkv, out, lse, logit_scale, bias, mask = ctx.saved_tensors
+        scale_type = ctx.scale_type
+        q, k, v = (qkv[:, :, i].transpose(1, 2) for i in range(3))
+        do = dout.transpose(1, 2)                                          # [B, H, L, d] view
+        if not _rows_16b_aligned(do):
+            do = do.contiguous()
+        dqkv = torch.empty_like(qkv)
+        dq, dk, dv = (dqkv[:, :, i].transpose(1, 2) for i in range(3))
+        dscale = torch.empty_like(logit_scale, memory_format=torch.contiguous_format) if scale_type == "tensor" else None
+        db = torch.empty_like(bias, memory_format=torch.contiguous_format) if bias is not None else None
+
+        lib = _abi.load()
+        p = _describe(q, k, v, out.transpose(1, 2), lse, logit_scale, bias, mask, ctx.mask_live, scale_type,
+                      ctx.window_map)
+        _set_t4(p.d_o, do); _set_t4(p.dq, dq); _set_t4(p.dk, dk); _set_t4(p.dv, dv)
+        if db is not None:
+            p.dbias = db.data_ptr()
+        if dscale is not None:
+            p.dscale = dscale.data_ptr()
+        with _on_device(qkv.device) as stream:
+            need = lib.fwa2_backward_workspace_bytes(p)
+            ws = torch.empty(max(need, 1), dtype=torch.uint8, device=qkv.device)
+            p.workspace, p.workspace_bytes = ws.data_ptr(), need
+            p.stream = stream
+            _abi.check(lib.fwa2_backward(p), "fwa2_backward")
+        return dqkv, None, None, None, dscale, db, None
 
 
 class CpbBias(torch.autograd.Function):

@@ -17,8 +17,9 @@ import torch.nn as nn
 import torch.nn.functional as F
 from torch.utils.checkpoint import checkpoint
 
-from .win_attention_func import flash_win_attn_v2_func, flash_win_attn_v2_qkvpacked_func, win_attention_torch
-from .flash_window_attention_v2 import CpbBias
+from .win_attention_func import (flash_win_attn_v2_func, flash_win_attn_v2_grid_func, flash_win_attn_v2_qkvpacked_func,
+                                 win_attention_torch)
+from .flash_window_attention_v2 import CpbBias, MAPPED_BACKWARD_MAX_N
 
 
 def _pair(x):
@@ -95,6 +96,9 @@ class WindowAttention(nn.Module):
     #: build the bias (and take its gradient back to table space) with the library's two small kernels
     #: instead of gather / permute / sigmoid and autograd's sort-based scatter (flash path only)
     fused_bias = True
+    #: let the kernels do the cyclic shift and the window partition / reverse of the enclosing block by
+    #: address arithmetic (flash path only; used by SwinTransformerBlock when `grid_ready` says so)
+    fused_grid = True
 
     def __init__(self, dim, window_size, num_heads, is_flash=True, qkv_bias=True, attn_drop=0., proj_drop=0.,
                  pretrained_window_size=[0, 0]):
@@ -183,6 +187,30 @@ class WindowAttention(nn.Module):
             out = out.transpose(1, 2).reshape(b_, n, c)
         return self.proj_drop(self.proj(out))
 
+    def grid_ready(self, x):
+        """True when `forward_grid` can take `x`: the fused path on the GPU in half precision, and a window the
+        library's backward addresses through a window map whenever a gradient will be asked for."""
+        if not (self.is_flash and self.packed_qkv and self.fused_grid and x.is_cuda):
+            return False
+        if x.dtype not in (torch.float16, torch.bfloat16) and not torch.is_autocast_enabled():
+            return False
+        n = self.window_size[0] * self.window_size[1]
+        return n <= 256 and (n <= MAPPED_BACKWARD_MAX_N or not torch.is_grad_enabled())
+
+    def forward_grid(self, x, grid, shift, mask=None):
+        """The attention of every (shifted) window of the token grid x [B, gh * gw, C], result in the same
+        layout: what the reference's block computes with roll + window_partition around `forward` and
+        window_reverse + roll after it (swin_transformer_v2.py:419-441), with the permutation done by the
+        kernels' addressing.  `shift` = (shift_size, shift_size) of the block."""
+        b, length, c = x.shape
+        bias = None
+        if self.q_bias is not None:
+            bias = torch.cat((self.q_bias, torch.zeros_like(self.v_bias, requires_grad=False), self.v_bias))
+        qkv = F.linear(x, self.qkv.weight, bias).reshape(b, length, 3, self.num_heads, -1)
+        rel_bias = self.relative_position_bias()
+        out = flash_win_attn_v2_grid_func(qkv, grid, self.window_size, shift, self.logit_scale, rel_bias, mask)
+        return self.proj_drop(self.proj(out.reshape(b, length, c)))
+
     def extra_repr(self):
         return (f"dim={self.dim}, window_size={self.window_size}, "
                 f"pretrained_window_size={self.pretrained_window_size}, num_heads={self.num_heads}")
@@ -225,6 +253,11 @@ class SwinTransformerBlock(nn.Module):
         b, length, c = x.shape
         assert length == h * w, "input feature has wrong size"
         shortcut = x
+        if self.attn.grid_ready(x):
+            # roll, window_partition, window_reverse and the roll back happen inside the kernels
+            x = self.attn.forward_grid(x, (h, w), (self.shift_size, self.shift_size), mask=self.attn_mask)
+            x = shortcut + self.drop_path(self.norm1(x))
+            return x + self.drop_path(self.norm2(self.mlp(x)))
         x = x.view(b, h, w, c)
         if self.shift_size > 0:
             x = torch.roll(x, shifts=(-self.shift_size, -self.shift_size), dims=(1, 2))

@@ -6,13 +6,18 @@ import math
 import torch
 import torch.nn.functional as F
 
-from .flash_window_attention_v2 import FlashWindowAttentionV2, FlashWindowAttentionV2QKVPacked
+from .flash_window_attention_v2 import (FlashWindowAttentionV2, FlashWindowAttentionV2Grid,
+                                         FlashWindowAttentionV2QKVPacked)
 
 #: fused forward/backward: (q, k, v, logit_scale=None, bias=None, mask=None) -> o
 flash_win_attn_v2_func = FlashWindowAttentionV2.apply
 #: the same fed from the packed projection: (qkv [BW, N, 3, H, d], logit_scale=None, bias=None, mask=None)
 #: -> o [BW, N, H, d]; the gradient comes back as one packed tensor
 flash_win_attn_v2_qkvpacked_func = FlashWindowAttentionV2QKVPacked.apply
+#: the packed operator on the un-partitioned token grid, with the cyclic shift and the window partition /
+#: reverse done by the kernels: (qkv [B, gh*gw, 3, H, d], (gh, gw), (wh, ww), (shift_h, shift_w),
+#: logit_scale=None, bias=None, mask=None) -> o [B, gh*gw, H, d]
+flash_win_attn_v2_grid_func = FlashWindowAttentionV2Grid.apply
 
 
 def win_attention_torch(q, k, v, logit_scale=None, bias=None, mask=None):

@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define FWA2_ABI_VERSION 1
+#define FWA2_ABI_VERSION 2
 
 typedef enum fwa2_status {
     FWA2_OK = 0,
@@ -113,6 +113,21 @@ typedef struct fwa2_problem {
     size_t  workspace_bytes;
 
     void*   stream;          /* hipStream_t */
+
+    /*
+     * Optional window map, all zero = off.  It does the cyclic shift and the window partition / reverse of
+     * the caller (flash_win_attn_v2/swin_transformer_v2.py:419-441: roll, window_partition, window_reverse,
+     * roll back) by address arithmetic.  With grid_h > 0 the tensors q, k, v, o, d_o, dq, dk, dv are token
+     * grids [B, grid_h * grid_w, ...] instead of [BW, H, N, d]: stride_bw is then the stride between IMAGES
+     * and stride_n the stride between consecutive tokens of the row-major grid.  Unit b = image * nW + window,
+     * nW = (grid_h / win_h) (grid_w / win_w), window = wy (grid_w / win_w) + wx; its row n = r win_w + c is the
+     * token at ((wy win_h + r + shift_h) mod grid_h, (wx win_w + c + shift_w) mod grid_w).  n must equal
+     * win_h win_w and bw must equal B nW; lse, bias, mask, dbias are indexed as without a map (mask: nW == n_windows).
+     * Supported for n <= 256 in forward and n <= 64 in backward (FWA2_ERR_UNSUPPORTED otherwise).
+     */
+    int32_t grid_h, grid_w;
+    int32_t win_h, win_w;
+    int32_t shift_h, shift_w;
 } fwa2_problem;
 
 /* Library / ABI identification.  Returns FWA2_ABI_VERSION. */

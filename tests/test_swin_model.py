@@ -20,7 +20,7 @@ def test_alias_package_exports():
     import flash_win_attn_v2 as ref_name
     from flash_win_attn_v2.swin_transformer_v2 import WindowAttention as wa
     for name in ("WindowAttention", "SwinTransformerV2", "flash_win_attn_v2_func", "win_attention_torch",
-                 "win_attention_torch_compile", "flash_win_attn_v2_qkvpacked_func"):
+                 "win_attention_torch_compile", "flash_win_attn_v2_qkvpacked_func", "flash_win_attn_v2_grid_func"):
         assert getattr(ref_name, name) is getattr(fwa, name)
     assert wa is swin.WindowAttention
 
@@ -256,6 +256,50 @@ def test_fused_position_bias_gpu(window, dtype):
     t2 = table.clone().requires_grad_()
     CpbBias.apply(t2, wh, ww).backward(grad)
     assert torch.equal(t.grad, t2.grad)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shift", [0, 4])
+def test_block_window_map_matches_partition_gpu(shift):
+    """SwinTransformerBlock with the roll / partition / reverse done by the kernels' addressing against the
+    same block doing them as the reference does (swin_transformer_v2.py:419-441).  The attention kernels see
+    the same values either way; the projections run on differently ordered rows, hence a tolerance of a few ulp."""
+    torch.manual_seed(3)
+    dev = torch.device("cuda")
+    blk = swin.SwinTransformerBlock(96, (32, 32), 3, window_size=8, shift_size=shift, is_flash=True).to(dev).bfloat16()
+    x = torch.randn(2, 32 * 32, 96, device=dev).bfloat16()
+    g = torch.randn(2, 32 * 32, 96, device=dev).bfloat16()
+
+    assert blk.attn.grid_ready(x)
+    xa = x.clone().requires_grad_()
+    ya = blk(xa)
+    ya.backward(g)
+    grads_a = {n: p.grad.clone() for n, p in blk.named_parameters()}
+    blk.zero_grad()
+
+    blk.attn.fused_grid = False
+    assert not blk.attn.grid_ready(x)
+    xb = x.clone().requires_grad_()
+    yb = blk(xb)
+    yb.backward(g)
+    del blk.attn.fused_grid
+
+    def rel(a, b):
+        return float((a.float() - b.float()).abs().max() / b.float().abs().max())
+
+    assert rel(ya, yb) < 1e-2
+    assert rel(xa.grad, xb.grad) < 1e-2
+    for n, p in blk.named_parameters():
+        assert rel(grads_a[n], p.grad) < 2e-2, n
+    # windows of 256 tokens: taken under no_grad only, where no mapped backward is needed
+    big = swin.SwinTransformerBlock(96, (32, 32), 3, window_size=16, shift_size=2 * shift, is_flash=True).to(dev).bfloat16()
+    assert not big.attn.grid_ready(x)
+    with torch.no_grad():
+        assert big.attn.grid_ready(x)
+        y1 = big(x)
+        big.attn.fused_grid = False
+        y2 = big(x)
+    assert rel(y1, y2) < 1e-2
 
 
 @pytest.mark.gpu
