@@ -104,10 +104,9 @@ int validate(const fwa2_problem* p, int backward) {
         if (p->bw % nw) return fail(FWA2_ERR_INVALID_ARGUMENT, "window map: bw %d is not a multiple of %d windows per image", p->bw, nw);
         if (p->mask.ptr && p->n_windows != nw)
             return fail(FWA2_ERR_INVALID_ARGUMENT, "window map: mask has %d windows, the grid %d", p->n_windows, nw);
-        if (p->win_w > 64 || p->n > 256)
-            return fail(FWA2_ERR_UNSUPPORTED, "window map: windows of more than 256 tokens are not supported");
-        if (backward && p->n > fwa2::kMapBackwardMaxN)
-            return fail(FWA2_ERR_UNSUPPORTED, "window map: backward supports windows of up to %d tokens", fwa2::kMapBackwardMaxN);
+        if (p->win_w > 64 || p->n > fwa2::kMapMaxN)
+            return fail(FWA2_ERR_UNSUPPORTED, "window map: windows of more than %d tokens (or wider than 64) are not supported",
+                        fwa2::kMapMaxN);
     }
     if (p->lse == nullptr) return fail(FWA2_ERR_INVALID_ARGUMENT, "lse: null pointer");
     if (p->lse_stride_h < p->n) return fail(FWA2_ERR_INVALID_ARGUMENT, "lse: head stride %lld < n", (long long)p->lse_stride_h);

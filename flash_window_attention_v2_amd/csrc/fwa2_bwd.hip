@@ -179,8 +179,10 @@ __device__ __forceinline__ void unit_blocks(BwdLds<DT, NQB>& L, WaveRegs<DT, NQB
 // a workgroup then belongs to one (head, query chunk, key chunk), reads only those rows, keeps that
 // tile of dbias in registers and writes its share of dk / dv (already taken back through the
 // normalisation, which is linear) as fp32 partials that dkv_reduce_kernel sums over the query chunks.
-template <int DT, bool HAS_BIAS, int MASK_DT, int NQB, int KT, int MODE, bool BIG>
+// MAPPED: rows are addressed through the window map (cyclic shift + window partition done here; not with BIG).
+template <int DT, bool HAS_BIAS, int MASK_DT, int NQB, int KT, int MODE, bool BIG, bool MAPPED = false>
 __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) {
+    static_assert(!(MAPPED && BIG), "the window map is limited to windows one workgroup holds");
     typedef typename Elem<DT>::E E;
     typedef typename Elem<DT>::V8 V8;
     typedef typename Elem<DT>::V4 V4;
@@ -324,6 +326,15 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
         const int dc = (lane & 3) * 8;
         for (int row0 = wave * 16; row0 < R; row0 += 16 * p.waves) {   // 16 rows per wavefront and instruction
             const int r = row0 + (lane >> 2);
+            if constexpr (MAPPED) {
+                if (r < N) {
+                    async_row_chunk(reinterpret_cast<const E*>(p.q.ptr) + row_off<true>(p.q, p.map, b, h, r) + dc, L.rawQ + row0 * 32);
+                    async_row_chunk(reinterpret_cast<const E*>(p.d_o.ptr) + row_off<true>(p.d_o, p.map, b, h, r) + dc, L.rawDO + row0 * 32);
+                    async_row_chunk(reinterpret_cast<const E*>(p.o.ptr) + row_off<true>(p.o, p.map, b, h, r) + dc, L.rawO + row0 * 32);
+                    async_row_chunk(reinterpret_cast<const E*>(p.k.ptr) + row_off<true>(p.k, p.map, b, h, r) + dc, L.rawK + row0 * 32);
+                }
+                continue;
+            }
             if (r < N) {
                 async_row_chunk(qptr + (int64_t)r * p.q.sn + dc, L.rawQ + row0 * 32);
                 async_row_chunk(doptr + (int64_t)r * p.d_o.sn + dc, L.rawDO + row0 * 32);
@@ -336,6 +347,10 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
         for (int kt = 0; kt < KT; kt++) {
             const int row0 = (wave * KT + kt) * 16;
             const int r = row0 + (lane >> 2);
+            if constexpr (MAPPED) {
+                if (r < NK) async_row_chunk(reinterpret_cast<const E*>(p.v.ptr) + row_off<true>(p.v, p.map, b, h, r) + dc, L.rawV + row0 * 32);
+                continue;
+            }
             if (r < NK) async_row_chunk(vptr + (int64_t)r * p.v.sn + dc, L.rawV + row0 * 32);
         }
         for (int r0 = wave * 64; r0 < N; r0 += 64 * p.waves) {
@@ -475,8 +490,8 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
                         *reinterpret_cast<f32x4*>(p.part_dv + row * 32 + 8 * g + 4 * dt) = v4;
                     }
                 } else {
-                    E* dkp = reinterpret_cast<E*>(const_cast<void*>(p.dk.ptr)) + b * p.dk.sb + h * p.dk.sh + (int64_t)key * p.dk.sn;
-                    E* dvp = reinterpret_cast<E*>(const_cast<void*>(p.dv.ptr)) + b * p.dv.sb + h * p.dv.sh + (int64_t)key * p.dv.sn;
+                    E* dkp = reinterpret_cast<E*>(const_cast<void*>(p.dk.ptr)) + row_off<MAPPED>(p.dk, p.map, b, h, key);
+                    E* dvp = reinterpret_cast<E*>(const_cast<void*>(p.dv.ptr)) + row_off<MAPPED>(p.dv, p.map, b, h, key);
                     V8 o8, v8;
 #pragma unroll
                     for (int j = 0; j < 8; j++) {
@@ -697,7 +712,7 @@ static int resident_per_cu(K kern, int threads) {
     return n;
 }
 
-template <int DT, bool HAS_BIAS, int MASK_DT, int NQB, int KT, bool BIG>
+template <int DT, bool HAS_BIAS, int MASK_DT, int NQB, int KT, bool BIG, bool MAPPED = false>
 static hipError_t launch_main(BwdParams p, const BwdPlan& pl, hipStream_t st, int* groups_out) {
     // Up to 64 tokens one launch walks masked and unmasked units alike; above that the two copies of
     // the block sequence cost occupancy (128 tokens) or spill (256), and each kind gets a launch.
@@ -705,10 +720,10 @@ static hipError_t launch_main(BwdParams p, const BwdPlan& pl, hipStream_t st, in
     // never more workgroups per head (and super-tile) than the plan sized the workspace for
     static const int fit = [&] {
         if constexpr (kOneLaunch) {
-            return resident_per_cu(bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, 2, BIG>, 64 * pl.waves);
+            return resident_per_cu(bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, 2, BIG, MAPPED>, 64 * pl.waves);
         } else {
-            const int a = resident_per_cu(bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, 0, BIG>, 64 * pl.waves);
-            const int b = MASK_DT >= 0 ? resident_per_cu(bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, 1, BIG>, 64 * pl.waves) : a;
+            const int a = resident_per_cu(bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, 0, BIG, MAPPED>, 64 * pl.waves);
+            const int b = MASK_DT >= 0 ? resident_per_cu(bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, 1, BIG, MAPPED>, 64 * pl.waves) : a;
             return a < b ? a : b;
         }
     }();
@@ -723,14 +738,14 @@ static hipError_t launch_main(BwdParams p, const BwdPlan& pl, hipStream_t st, in
     const dim3 grid(p.heads * tiles * groups), block(64 * pl.waves);
     if (p.ev_start) (void)hipEventRecord(p.ev_start, st);
     if constexpr (kOneLaunch) {
-        hipLaunchKernelGGL((bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, 2, BIG>), grid, block, 0, st, p);
+        hipLaunchKernelGGL((bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, 2, BIG, MAPPED>), grid, block, 0, st, p);
     } else {
         // the units whose mask is all zero (or every unit when there is no mask) ...
-        if (MASK_DT < 0 || two) hipLaunchKernelGGL((bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, 0, BIG>), grid, block, 0, st, p);
+        if (MASK_DT < 0 || two) hipLaunchKernelGGL((bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, 0, BIG, MAPPED>), grid, block, 0, st, p);
         // ... and the units whose mask is live (all of them when the flags are absent)
         if (MASK_DT >= 0) {
             p.db_slot0 = two ? groups : 0;
-            hipLaunchKernelGGL((bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, 1, BIG>), grid, block, 0, st, p);
+            hipLaunchKernelGGL((bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, 1, BIG, MAPPED>), grid, block, 0, st, p);
         }
     }
     if (p.ev_stop) (void)hipEventRecord(p.ev_stop, st);
@@ -743,6 +758,13 @@ static hipError_t launch_main(BwdParams p, const BwdPlan& pl, hipStream_t st, in
 
 template <int DT, bool HAS_BIAS, int MASK_DT>
 static hipError_t launch_nqb(const BwdParams& p, const BwdPlan& pl, hipStream_t st, int* groups_out) {
+    if (p.map.nw > 0) {
+        // windows of up to 64 tokens with a map go to the fused kernel, longer than 256 are refused earlier
+        if (pl.n_chunks > 1 || pl.nqb_t == 2) return hipErrorInvalidValue;
+        if (pl.nqb_t == 4) return launch_main<DT, HAS_BIAS, MASK_DT, 4, 1, false, true>(p, pl, st, groups_out);
+        if (pl.kt == 1) return launch_main<DT, HAS_BIAS, MASK_DT, 8, 1, false, true>(p, pl, st, groups_out);
+        return launch_main<DT, HAS_BIAS, MASK_DT, 8, 2, false, true>(p, pl, st, groups_out);
+    }
     if (pl.n_chunks > 1) return launch_main<DT, HAS_BIAS, MASK_DT, 8, 2, true>(p, pl, st, groups_out);
     if (pl.nqb_t == 2) return launch_main<DT, HAS_BIAS, MASK_DT, 2, 1, false>(p, pl, st, groups_out);
     if (pl.nqb_t == 4) return launch_main<DT, HAS_BIAS, MASK_DT, 4, 1, false>(p, pl, st, groups_out);

@@ -29,7 +29,8 @@ constexpr int kDqSub = 2;    // 16-row query tiles per wavefront (see below)
 // SUB = 16-row query tiles per wavefront.  With SUB = 2 a wavefront owns 32 query rows as two
 // independent tiles that share every K / V operand it reads from LDS; a unit of 256 rows then takes
 // 8 wavefronts of up to 256 registers instead of 16 of up to 128.
-template <int DT, bool HAS_BIAS, int MASK_DT, int NT, bool VEC, bool MASKED, int SUB>
+// MAPPED: rows are addressed through the window map (cyclic shift + window partition done here).
+template <int DT, bool HAS_BIAS, int MASK_DT, int NT, bool VEC, bool MASKED, int SUB, bool MAPPED = false>
 __global__ void __launch_bounds__(64 * NT / SUB) bwd_dq_resident_kernel(const BwdParams p) {
     typedef typename Elem<DT>::E E;
     typedef typename Elem<DT>::V8 V8;
@@ -224,13 +225,10 @@ __global__ void __launch_bounds__(64 * NT / SUB) bwd_dq_resident_kernel(const Bw
             const int row0 = wave * WR + 16 * u;
             const int frow = row0 + (ln >> 2);
             if (frow < N) {
-                dma16(reinterpret_cast<const E*>(p.k.ptr) + b * p.k.sb + h * p.k.sh + (int64_t)frow * p.k.sn + fc8,
-                      lds_rawK + row0 * 32);
-                dma16(reinterpret_cast<const E*>(p.v.ptr) + b * p.v.sb + h * p.v.sh + (int64_t)frow * p.v.sn + fc8,
-                      lds_rawV + row0 * 32);
-                dma16(reinterpret_cast<const E*>(p.q.ptr) + b * p.q.sb + h * p.q.sh + (int64_t)frow * p.q.sn + fc8,
-                      lds_rawQ + row0 * 32);
-                dma16(reinterpret_cast<const E*>(p.d_o.ptr) + b * p.d_o.sb + h * p.d_o.sh + (int64_t)frow * p.d_o.sn + fc8,
+                dma16(reinterpret_cast<const E*>(p.k.ptr) + row_off<MAPPED>(p.k, p.map, b, h, frow) + fc8, lds_rawK + row0 * 32);
+                dma16(reinterpret_cast<const E*>(p.v.ptr) + row_off<MAPPED>(p.v, p.map, b, h, frow) + fc8, lds_rawV + row0 * 32);
+                dma16(reinterpret_cast<const E*>(p.q.ptr) + row_off<MAPPED>(p.q, p.map, b, h, frow) + fc8, lds_rawQ + row0 * 32);
+                dma16(reinterpret_cast<const E*>(p.d_o.ptr) + row_off<MAPPED>(p.d_o, p.map, b, h, frow) + fc8,
                       lds_rawDO + row0 * 32);
             }
             const int q = row0 + (ln & 15);
@@ -384,7 +382,7 @@ __global__ void __launch_bounds__(64 * NT / SUB) bwd_dq_resident_kernel(const Bw
             const float f = s_true * inv[u];
             const int q = wave * WR + 16 * u + (ln2 & 15);
             if (q < N) {
-                E* dqrow = reinterpret_cast<E*>(const_cast<void*>(p.dq.ptr)) + b * p.dq.sb + h * p.dq.sh + (int64_t)q * p.dq.sn;
+                E* dqrow = reinterpret_cast<E*>(const_cast<void*>(p.dq.ptr)) + row_off<MAPPED>(p.dq, p.map, b, h, q);
                 V8 o8;
 #pragma unroll
                 for (int j = 0; j < 8; j++) o8[j] = (E)(f * (dqacc[u][j >> 2][j & 3] - qh[j] * proj));
@@ -424,13 +422,13 @@ static int resident_fit(K kern, int threads) {
 // Launches the kernel(s) and reports how many dscale partials per head they wrote.
 // SUBP: 16-row query tiles per wavefront in the launch over the unmasked units; the masked launch always
 // uses kDqSub (its tile rebuilds leave no room in 128 registers).
-template <int DT, bool HAS_BIAS, int MASK_DT, int NT, bool VEC, int SUBP = kDqSub>
+template <int DT, bool HAS_BIAS, int MASK_DT, int NT, bool VEC, int SUBP = kDqSub, bool MAPPED = false>
 static hipError_t launch_nt(BwdParams p, hipStream_t st, int max_groups, int* ds_parts_out) {
     constexpr int SUBM = kDqSub;
     static const int fit_plain =
-        resident_fit(bwd_dq_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, false, SUBP>, 64 * NT / SUBP);
+        resident_fit(bwd_dq_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, false, SUBP, MAPPED>, 64 * NT / SUBP);
     static const int fit_masked =
-        MASK_DT >= 0 ? resident_fit(bwd_dq_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, true, SUBM>, 64 * NT / SUBM) : 1;
+        MASK_DT >= 0 ? resident_fit(bwd_dq_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, true, SUBM, MAPPED>, 64 * NT / SUBM) : 1;
     auto groups_for = [&](int fit) {
         int groups = (p.cus * fit) / p.heads;
         if (groups < 1) groups = 1;
@@ -445,13 +443,13 @@ static hipError_t launch_nt(BwdParams p, hipStream_t st, int max_groups, int* ds
     if (g_plain) {
         p.dq_groups = g_plain;
         p.ds_slot0 = 0;
-        hipLaunchKernelGGL((bwd_dq_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, false, SUBP>), dim3(p.heads * g_plain),
+        hipLaunchKernelGGL((bwd_dq_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, false, SUBP, MAPPED>), dim3(p.heads * g_plain),
                            dim3(64 * ((p.n + 16 * SUBP - 1) / (16 * SUBP))), 0, st, p);
     }
     if (g_masked) {
         p.dq_groups = g_masked;
         p.ds_slot0 = g_plain;
-        hipLaunchKernelGGL((bwd_dq_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, true, SUBM>), dim3(p.heads * g_masked),
+        hipLaunchKernelGGL((bwd_dq_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, true, SUBM, MAPPED>), dim3(p.heads * g_masked),
                            dim3(64 * ((p.n + 16 * SUBM - 1) / (16 * SUBM))), 0, st, p);
     }
     *ds_parts_out = p.ds_parts;
@@ -461,6 +459,18 @@ static hipError_t launch_nt(BwdParams p, hipStream_t st, int max_groups, int* ds
 template <int DT, bool HAS_BIAS, int MASK_DT>
 static hipError_t launch_mask(const BwdParams& p, hipStream_t st, int mg, int* out) {
     const int nt = p.n <= 64 ? 4 : (p.n <= 128 ? 8 : 16);
+    if (p.map.nw > 0) {
+        // windows of up to 64 tokens with a map go to the fused kernel, never here
+        if (nt == 4) return hipErrorInvalidValue;
+        if (p.side_vec) {
+            if (nt == 8) return launch_nt<DT, HAS_BIAS, MASK_DT, 8, true, kDqSub, true>(p, st, mg, out);
+            if (p.n <= 160) return launch_nt<DT, HAS_BIAS, MASK_DT, 16, true, 1, true>(p, st, mg, out);
+            return launch_nt<DT, HAS_BIAS, MASK_DT, 16, true, kDqSub, true>(p, st, mg, out);
+        }
+        if (nt == 8) return launch_nt<DT, HAS_BIAS, MASK_DT, 8, false, kDqSub, true>(p, st, mg, out);
+        if (p.n <= 160) return launch_nt<DT, HAS_BIAS, MASK_DT, 16, false, 1, true>(p, st, mg, out);
+        return launch_nt<DT, HAS_BIAS, MASK_DT, 16, false, kDqSub, true>(p, st, mg, out);
+    }
     if (p.side_vec) {
         if (nt == 4) return launch_nt<DT, HAS_BIAS, MASK_DT, 4, true>(p, st, mg, out);
         if (nt == 8) return launch_nt<DT, HAS_BIAS, MASK_DT, 8, true>(p, st, mg, out);

@@ -206,7 +206,7 @@ __device__ __forceinline__ auto load_raw8(const T* row, int c0, int n, float pad
 // not push the bias / mask tables (re-read by every unit) out of the L2.
 constexpr int kStreamPolicy = 2;
 
-constexpr int kMapBackwardMaxN = 64;   // largest window the backward kernels address through a window map
+constexpr int kMapMaxN = 256;    // largest window the kernels address through a window map (the resident-tile ones)
 constexpr int kKeyChunk = 256;   // keys staged in LDS at a time by the query-owning kernels
 constexpr int kLdsStride = 40;   // elements per staged row (32 + 8 pad): 80-byte rows
 

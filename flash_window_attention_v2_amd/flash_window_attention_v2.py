@@ -273,7 +273,7 @@ class FlashWindowAttentionV2QKVPacked(torch.autograd.Function):
         return dqkv, dscale, db, None
 
 
-MAPPED_BACKWARD_MAX_N = 64      # largest window whose backward the library addresses through a window map
+MAPPED_MAX_N = 256      # largest window the library addresses through a window map
 
 
 class FlashWindowAttentionV2Grid(torch.autograd.Function):

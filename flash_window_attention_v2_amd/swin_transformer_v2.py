@@ -19,7 +19,7 @@ from torch.utils.checkpoint import checkpoint
 
 from .win_attention_func import (flash_win_attn_v2_func, flash_win_attn_v2_grid_func, flash_win_attn_v2_qkvpacked_func,
                                  win_attention_torch)
-from .flash_window_attention_v2 import CpbBias, MAPPED_BACKWARD_MAX_N
+from .flash_window_attention_v2 import CpbBias, MAPPED_MAX_N
 
 
 def _pair(x):
@@ -189,13 +189,12 @@ class WindowAttention(nn.Module):
 
     def grid_ready(self, x):
         """True when `forward_grid` can take `x`: the fused path on the GPU in half precision, and a window the
-        library's backward addresses through a window map whenever a gradient will be asked for."""
+        library addresses through a window map."""
         if not (self.is_flash and self.packed_qkv and self.fused_grid and x.is_cuda):
             return False
         if x.dtype not in (torch.float16, torch.bfloat16) and not torch.is_autocast_enabled():
             return False
-        n = self.window_size[0] * self.window_size[1]
-        return n <= 256 and (n <= MAPPED_BACKWARD_MAX_N or not torch.is_grad_enabled())
+        return self.window_size[0] * self.window_size[1] <= MAPPED_MAX_N
 
     def forward_grid(self, x, grid, shift, mask=None):
         """The attention of every (shifted) window of the token grid x [B, gh * gw, C], result in the same

@@ -54,6 +54,12 @@ CASES = [
     (1, (12, 8), (4, 4), (1, 3), 4, True),
     (2, (8, 8), (8, 8), (0, 0), 3, False),          # one window covers the grid
     (2, (6, 9), (3, 3), (1, 1), 2, True),           # 9 tokens
+    (2, (32, 32), (16, 16), (8, 8), 3, True),       # 256 tokens: forward, dq and key-side kernels
+    (2, (32, 16), (16, 16), (0, 0), 3, False),
+    (2, (24, 36), (12, 12), (6, 6), 3, True),       # 144 tokens: one 16-key tile per wavefront
+    (1, (20, 40), (10, 20), (5, 10), 2, True),      # 200 tokens, not a multiple of 16
+    (2, (16, 24), (8, 12), (4, 6), 3, True),        # 96 tokens
+    (2, (22, 11), (11, 11), (5, 5), 2, True),       # 121 tokens, odd
 ]
 
 
@@ -82,22 +88,13 @@ def test_grid_matches_partitioned_call(case, dtype):
     assert torch.equal(scale_a.grad, scale_b.grad)
 
 
-@pytest.mark.parametrize("window,grid,shift", [((16, 16), (32, 32), (8, 8)), ((12, 12), (24, 36), (6, 6)),
-                                               ((10, 20), (20, 40), (5, 10))])
-def test_grid_forward_of_larger_windows(window, grid, shift):
-    """Windows of 65 to 256 tokens: the forward kernel takes the map; the backward kernels do not yet and
-    must say so instead of computing on wrong addresses."""
-    from flash_window_attention_v2_amd import _abi, flash_win_attn_v2_grid_func, flash_win_attn_v2_qkvpacked_func
-    qkv, scale, bias, mask, dout = _inputs(2, grid, window, 3, 32, torch.bfloat16, 12, True)
-    with torch.no_grad():
-        o_a = flash_win_attn_v2_grid_func(qkv, grid, window, shift, scale, bias, mask)
-        o_b = _reverse(flash_win_attn_v2_qkvpacked_func(_partition(qkv, grid, window, shift), scale, bias, mask),
-                       grid, window, shift)
-    assert torch.equal(o_a, o_b)
-    a = qkv.clone().requires_grad_(True)
-    o = flash_win_attn_v2_grid_func(a, grid, window, shift, scale, bias, mask)
+def test_grid_rejects_windows_longer_than_256_tokens():
+    """Windows of more than 256 tokens run on the streaming kernels, which take no map: the library must
+    say so instead of computing on wrong addresses."""
+    from flash_window_attention_v2_amd import flash_win_attn_v2_grid_func
+    qkv, scale, bias, mask, _ = _inputs(1, (36, 18), (18, 18), 2, 32, torch.bfloat16, 12, True)
     with pytest.raises(NotImplementedError, match="window map"):
-        o.backward(dout)
+        flash_win_attn_v2_grid_func(qkv, (36, 18), (18, 18), (9, 9), scale, bias, mask)
 
 
 def test_grid_argument_errors():

@@ -259,14 +259,14 @@ def test_fused_position_bias_gpu(window, dtype):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("shift", [0, 4])
-def test_block_window_map_matches_partition_gpu(shift):
+@pytest.mark.parametrize("window,shift", [(8, 0), (8, 4), (16, 8)])
+def test_block_window_map_matches_partition_gpu(window, shift):
     """SwinTransformerBlock with the roll / partition / reverse done by the kernels' addressing against the
     same block doing them as the reference does (swin_transformer_v2.py:419-441).  The attention kernels see
     the same values either way; the projections run on differently ordered rows, hence a tolerance of a few ulp."""
     torch.manual_seed(3)
     dev = torch.device("cuda")
-    blk = swin.SwinTransformerBlock(96, (32, 32), 3, window_size=8, shift_size=shift, is_flash=True).to(dev).bfloat16()
+    blk = swin.SwinTransformerBlock(96, (32, 32), 3, window_size=window, shift_size=shift, is_flash=True).to(dev).bfloat16()
     x = torch.randn(2, 32 * 32, 96, device=dev).bfloat16()
     g = torch.randn(2, 32 * 32, 96, device=dev).bfloat16()
 
@@ -291,15 +291,6 @@ def test_block_window_map_matches_partition_gpu(shift):
     assert rel(xa.grad, xb.grad) < 1e-2
     for n, p in blk.named_parameters():
         assert rel(grads_a[n], p.grad) < 2e-2, n
-    # windows of 256 tokens: taken under no_grad only, where no mapped backward is needed
-    big = swin.SwinTransformerBlock(96, (32, 32), 3, window_size=16, shift_size=2 * shift, is_flash=True).to(dev).bfloat16()
-    assert not big.attn.grid_ready(x)
-    with torch.no_grad():
-        assert big.attn.grid_ready(x)
-        y1 = big(x)
-        big.attn.fused_grid = False
-        y2 = big(x)
-    assert rel(y1, y2) < 1e-2
 
 
 @pytest.mark.gpu
