@@ -15,6 +15,9 @@ hipError_t launch_mask_scan(const void* mask, int mask_dt, int64_t sw, int64_t s
                             uint8_t* live, hipStream_t st);
 hipError_t launch_backward(const BwdParams& p, int dtype, bool has_bias, int mask_dt, hipStream_t st);
 size_t backward_workspace_bytes(int heads, int n, int bw, bool has_bias, bool has_mask, int n_windows, int cus);
+bool generic_head_dim(int d);
+size_t generic_workspace_bytes(int heads, int n, int bw, bool has_bias);
+hipError_t launch_generic(const fwa2_problem* p, bool backward);
 int backward_supported(int n);
 hipError_t launch_cpb_bias_forward(const void* table, int dtype, int heads, int wh, int ww, void* bias, hipStream_t st);
 hipError_t launch_cpb_bias_backward(const void* table, const void* dbias, int dtype, int heads, int wh, int ww,
@@ -37,13 +40,13 @@ int fail(int code, const char* fmt, ...) {
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
-int check_t4(const char* name, const fwa2_tensor4& t) {
+int check_t4(const char* name, const fwa2_tensor4& t, int head_dim) {
     if (t.ptr == nullptr) return fail(FWA2_ERR_INVALID_ARGUMENT, "%s: null pointer", name);
     if (!aligned16(t.ptr) || (t.stride_bw % 8) || (t.stride_h % 8) || (t.stride_n % 8))
         return fail(FWA2_ERR_UNSUPPORTED,
                     "%s: rows must start on 16-byte boundaries (pointer 16-byte aligned, strides multiples of 8 elements)",
                     name);
-    if (t.stride_n < 32) return fail(FWA2_ERR_INVALID_ARGUMENT, "%s: row stride %lld overlaps rows", name, (long long)t.stride_n);
+    if (t.stride_n < head_dim) return fail(FWA2_ERR_INVALID_ARGUMENT, "%s: row stride %lld overlaps rows", name, (long long)t.stride_n);
     return FWA2_OK;
 }
 
@@ -70,12 +73,13 @@ int validate(const fwa2_problem* p, int backward) {
         return fail(FWA2_ERR_INVALID_ARGUMENT, "bw, heads, n and head_dim must be positive");
     if (p->head_dim > 128)
         return fail(FWA2_ERR_INVALID_ARGUMENT, "FlashAttention only support head dimensions up to 128");
-    if (p->head_dim != 32)
-        return fail(FWA2_ERR_UNSUPPORTED, "head_dim %d: this build implements head_dim 32 only", p->head_dim);
+    if (p->head_dim % 8)
+        return fail(FWA2_ERR_UNSUPPORTED, "head_dim %d: head dimensions must be multiples of 8 (16-byte row chunks)", p->head_dim);
     if ((int64_t)p->bw * p->heads * ((p->n + 255) / 256) > 0x7fffffffLL)
         return fail(FWA2_ERR_UNSUPPORTED, "too many (batch*window, head) pairs for one launch");
     int rc;
-    if ((rc = check_t4("q", p->q)) || (rc = check_t4("k", p->k)) || (rc = check_t4("v", p->v)) || (rc = check_t4("o", p->o)))
+    const int hd = p->head_dim;
+    if ((rc = check_t4("q", p->q, hd)) || (rc = check_t4("k", p->k, hd)) || (rc = check_t4("v", p->v, hd)) || (rc = check_t4("o", p->o, hd)))
         return rc;
     if (p->scale_kind == FWA2_SCALE_TENSOR) {
         if (p->logit_scale == nullptr) return fail(FWA2_ERR_INVALID_ARGUMENT, "logit_scale: null with FWA2_SCALE_TENSOR");
@@ -104,6 +108,8 @@ int validate(const fwa2_problem* p, int backward) {
         if (p->bw % nw) return fail(FWA2_ERR_INVALID_ARGUMENT, "window map: bw %d is not a multiple of %d windows per image", p->bw, nw);
         if (p->mask.ptr && p->n_windows != nw)
             return fail(FWA2_ERR_INVALID_ARGUMENT, "window map: mask has %d windows, the grid %d", p->n_windows, nw);
+        if (fwa2::generic_head_dim(p->head_dim))
+            return fail(FWA2_ERR_UNSUPPORTED, "window map: head_dim %d is not supported with a window map (32 only)", p->head_dim);
         if (p->win_w > 64 || p->n > fwa2::kMapMaxN)
             return fail(FWA2_ERR_UNSUPPORTED, "window map: windows of more than %d tokens (or wider than 64) are not supported",
                         fwa2::kMapMaxN);
@@ -111,8 +117,8 @@ int validate(const fwa2_problem* p, int backward) {
     if (p->lse == nullptr) return fail(FWA2_ERR_INVALID_ARGUMENT, "lse: null pointer");
     if (p->lse_stride_h < p->n) return fail(FWA2_ERR_INVALID_ARGUMENT, "lse: head stride %lld < n", (long long)p->lse_stride_h);
     if (backward) {
-        if ((rc = check_t4("do", p->d_o)) || (rc = check_t4("dq", p->dq)) || (rc = check_t4("dk", p->dk)) ||
-            (rc = check_t4("dv", p->dv)))
+        if ((rc = check_t4("do", p->d_o, hd)) || (rc = check_t4("dq", p->dq, hd)) || (rc = check_t4("dk", p->dk, hd)) ||
+            (rc = check_t4("dv", p->dv, hd)))
             return rc;
         if (p->bias.ptr && p->dbias == nullptr) return fail(FWA2_ERR_INVALID_ARGUMENT, "dbias: null although bias is given");
         if (p->scale_kind == FWA2_SCALE_TENSOR && p->dscale == nullptr)
@@ -161,6 +167,8 @@ int fwa2_validate(const fwa2_problem* p, int backward) {
 
 size_t fwa2_backward_workspace_bytes(const fwa2_problem* p) {
     if (p == nullptr) return 0;
+    if (fwa2::generic_head_dim(p->head_dim))
+        return fwa2::generic_workspace_bytes(p->heads, p->n, p->bw, p->bias.ptr != nullptr);
     return fwa2::backward_workspace_bytes(p->heads, p->n, p->bw, p->bias.ptr != nullptr, p->mask.ptr != nullptr,
                                           p->n_windows, cu_count());
 }
@@ -213,6 +221,11 @@ int fwa2_forward(const fwa2_problem* p) {
     g_err[0] = 0;
     int rc = validate(p, 0);
     if (rc) return rc;
+    if (fwa2::generic_head_dim(p->head_dim)) {
+        hipError_t eg = fwa2::launch_generic(p, false);
+        if (eg != hipSuccess) return fail(FWA2_ERR_HIP, "forward launch: %s", hipGetErrorString(eg));
+        return FWA2_OK;
+    }
     fwa2::FwdParams k;
     memset(&k, 0, sizeof(k));
     k.q = to_t4(p->q); k.k = to_t4(p->k); k.v = to_t4(p->v); k.o = to_t4(p->o);
@@ -239,6 +252,11 @@ int fwa2_backward(const fwa2_problem* p) {
     g_err[0] = 0;
     int rc = validate(p, 1);
     if (rc) return rc;
+    if (fwa2::generic_head_dim(p->head_dim)) {
+        hipError_t eg = fwa2::launch_generic(p, true);
+        if (eg != hipSuccess) return fail(FWA2_ERR_HIP, "backward launch: %s", hipGetErrorString(eg));
+        return FWA2_OK;
+    }
     fwa2::BwdParams k;
     memset(&k, 0, sizeof(k));
     k.q = to_t4(p->q); k.k = to_t4(p->k); k.v = to_t4(p->v); k.o = to_t4(p->o);

@@ -1,0 +1,530 @@
+// Head dimensions other than 32 (any multiple of 8 up to 128): forward and backward for gfx950.
+//
+// The reference pads the head dimension to a power of two of at least 16 and supports up to 128
+// (flash_win_attn_v2/kernels/attn_kernel_forward.py:267, 298); every configuration it benchmarks uses 32,
+// which the tuned kernels of this library cover.  The kernels here restore the rest of that contract with
+// one plain skeleton instead of five tuned ones: no register-resident bias, no persistent workgroups, no
+// asynchronous prefetch.
+//
+// One skeleton, four modes.  A workgroup of four wavefronts works on one (batch*window, head) unit and 64
+// "owner" rows, 16 per wavefront, one per lane column (lane % 16); it walks over the "other" rows in steps
+// of 32, which all four wavefronts share through LDS:
+//
+//   FWD    owner = queries, other = keys:     online softmax, O^T += V^T P^T
+//   DQ     owner = queries, other = keys:     delta = rowsum(o * dO), dQ^^T += K^^T dZ^T; per-row dscale terms
+//   DKV    owner = keys,    other = queries:  dK^^T += Q^^T dZ, dV^T += dO^T P
+//   DBIAS  owner = queries, other = 32 keys:  loops over the units of a group, sums dZ per (query, key)
+//
+// Every score tile is v_mfma_f32_16x16x32 with the other rows as A rows and the owner rows as B columns, so
+// a lane holds, for its owner row, the 8 consecutive other rows 8g .. 8g+7 (g = lane / 16) of the step: the
+// rows of the two 16-row MFMA tiles are interleaved (tile a holds rows 8(r/4) + r%4 + 4a) to make them
+// consecutive.  Those 8 values are directly the B operand (k = other rows) of the products that contract
+// over the other rows; their A operands, the transposes of the staged tiles, come from row-major LDS with
+// ds_read_b64_tr_b16, one 32-column slab of the head dimension at a time.
+//
+// Numerics follow the tuned kernels: q^ and k^ are rounded to fp16 for the score product (also for bf16
+// inputs), scores live in the log2 domain, everything between the matrix products is fp32, P and dZ are
+// rounded (P to the input dtype, dZ to fp16) for the second products.  Nothing is accumulated with atomics:
+// dbias goes through per-group partial tiles and dlogit_scale through per-row terms, both summed in a fixed
+// order by small reduction kernels, so gradients are bit-reproducible here too.
+#include <string.h>
+
+#include "fwa2_common.hpp"
+
+namespace fwa2 {
+
+enum { G_FWD = 0, G_DQ = 1, G_DKV = 2, G_DBIAS = 3 };
+
+struct GenParams {
+    T4 q, k, v, o, d_o, dq, dk, dv;
+    const void* logit_scale;
+    int scale_kind;
+    float default_scale;
+    const void* bias;
+    int64_t bias_sh, bias_sn;
+    const void* mask;
+    int64_t mask_sw, mask_sn;
+    int mask_f32;
+    int n_windows;
+    float* lse;
+    int64_t lse_sb, lse_sh;
+    int bw, heads, n, d;
+    float* delta;         // [BW * H, row_pad] rowsum(o * dO), written by DQ, read by DKV and DBIAS
+    float* dscale_rows;   // [BW * H, row_pad] q^ . dq^ of every query row, written by DQ
+    int row_pad;
+    float* part_dbias;    // [groups, H, N, N] fp32
+    int groups;           // unit groups of the DBIAS launch (group g sums units g, g + groups, ...)
+    void* dbias;          // [H, N, N] input dtype
+    void* dscale;         // [H] input dtype
+};
+
+template <int DT, int D, int MODE>
+__global__ void __launch_bounds__(256) generic_kernel(const GenParams p) {
+    typedef typename Elem<DT>::E E;
+    typedef typename Elem<DT>::V8 V8;
+    typedef typename Elem<DT>::V4 V4;
+    typedef typename Elem<kScoreDT>::E SE;
+    typedef typename Elem<kScoreDT>::V8 SV8;
+    constexpr int S = D + 8;         // LDS row stride in elements
+    constexpr int KS = D / 32;       // 32-wide slabs of the head dimension
+    constexpr int CH = D / 8;        // 16-byte chunks per row
+    constexpr bool OWNER_IS_KEY = MODE == G_DKV;
+
+    __shared__ __attribute__((aligned(16))) SE t0[32 * S];   // other rows, normalised (k^ or q^)
+    __shared__ __attribute__((aligned(16))) E t1[32 * S];    // other rows of v (or dO)
+    __shared__ float s_lse2[32], s_delta[32];                // DKV: lse log2(e) and delta of the other rows
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int l16 = lane & 15, g = lane >> 4;
+    const int N = p.n, d = p.d;
+    const int chunks = (N + 63) / 64;
+    const int kblocks = (N + 31) / 32;
+
+    int idx = blockIdx.x, kb = 0, grp = 0, b0;
+    if (MODE == G_DBIAS) {
+        kb = idx % kblocks;
+        idx /= kblocks;
+    }
+    const int own0 = 64 * (idx % chunks);
+    idx /= chunks;
+    const int h = idx % p.heads;
+    idx /= p.heads;
+    if (MODE == G_DBIAS) { grp = idx; b0 = grp; } else { b0 = idx; }
+
+    const int own = own0 + 16 * wave + l16;     // owner row of this lane's column
+    const bool own_ok = own < N;
+
+    float scale2, scale_nat;
+    if (p.scale_kind == FWA2_SCALE_TENSOR) {
+        const float ls = (float)reinterpret_cast<const E*>(p.logit_scale)[h];
+        scale_nat = expf(fminf(ls, kLn100));
+    } else {
+        scale_nat = p.default_scale;
+    }
+    scale2 = scale_nat * kLog2e;
+
+    auto rowp = [&](const T4& t, int b, int row) -> const E* {
+        return reinterpret_cast<const E*>(t.ptr) + b * t.sb + h * t.sh + (int64_t)row * t.sn;
+    };
+
+    // ---- owner rows: B operands of the score products, one row per lane column ----
+    SV8 bs[KS];          // q^ (k^ for DKV), columns 32 s + 8 g .. + 7
+    V8 bp[KS];           // dO (v for DKV), same columns; unused by FWD
+    float own_inv = 0.f, own_lse2 = 0.f, own_delta = 0.f;
+    auto load_owner = [&](int b) __attribute__((always_inline)) {
+        const T4& ts = OWNER_IS_KEY ? p.k : p.q;
+        float x[KS][8];
+        float ss = 0.f;
+#pragma unroll
+        for (int s = 0; s < KS; s++) {
+            const int col = 32 * s + 8 * g;
+            V8 a = zero8<V8>();
+            if (own_ok && col < d) a = ld8<V8>(rowp(ts, b, own) + col);
+            unpack8(a, x[s]);
+#pragma unroll
+            for (int j = 0; j < 8; j++) ss += x[s][j] * x[s][j];
+        }
+        ss = col_add(ss);
+        own_inv = inv_norm(ss);
+#pragma unroll
+        for (int s = 0; s < KS; s++)
+#pragma unroll
+            for (int j = 0; j < 8; j++) bs[s][j] = (SE)(x[s][j] * own_inv);
+        if (MODE != G_FWD) {
+            const T4& tp = OWNER_IS_KEY ? p.v : p.d_o;
+            float dl = 0.f;
+#pragma unroll
+            for (int s = 0; s < KS; s++) {
+                const int col = 32 * s + 8 * g;
+                bp[s] = zero8<V8>();
+                if (own_ok && col < d) {
+                    bp[s] = ld8<V8>(rowp(tp, b, own) + col);
+                    if (MODE == G_DQ) {
+                        const V8 ov = ld8<V8>(rowp(p.o, b, own) + col);
+#pragma unroll
+                        for (int j = 0; j < 8; j++) dl += (float)bp[s][j] * (float)ov[j];
+                    }
+                }
+            }
+            const int64_t ro = ((int64_t)b * p.heads + h) * p.row_pad + own;
+            if (MODE == G_DQ) {
+                own_delta = col_add(dl);
+                if (g == 0 && own_ok) p.delta[ro] = own_delta;
+            }
+            if (MODE == G_DBIAS) own_delta = own_ok ? p.delta[ro] : 0.f;
+            if (MODE == G_DQ || MODE == G_DBIAS)
+                own_lse2 = own_ok ? p.lse[b * p.lse_sb + h * p.lse_sh + own] * kLog2e : 0.f;
+        }
+    };
+
+    // ---- 32 other rows starting at o0 into LDS: normalised into t0, raw into t1 ----
+    auto stage = [&](int b, int o0) __attribute__((always_inline)) {
+        const T4& ta = OWNER_IS_KEY ? p.q : p.k;
+        const T4& tb = OWNER_IS_KEY ? p.d_o : p.v;
+        for (int c = tid; c < 32 * CH; c += 256) {
+            const int r = c / CH, c8 = (c % CH) * 8;
+            const int row = o0 + r;
+            V8 a = zero8<V8>(), bb = zero8<V8>();
+            if (row < N && c8 < d) {
+                a = ld8<V8>(rowp(ta, b, row) + c8);
+                bb = ld8<V8>(rowp(tb, b, row) + c8);
+            }
+            float x[8];
+            unpack8(a, x);
+            float ss = 0.f;
+#pragma unroll
+            for (int j = 0; j < 8; j++) ss += x[j] * x[j];
+#pragma unroll
+            for (int off = CH / 2; off >= 1; off >>= 1) ss += __shfl_xor(ss, off);
+            const float inv = inv_norm(ss);
+            SV8 w;
+#pragma unroll
+            for (int j = 0; j < 8; j++) w[j] = (SE)(x[j] * inv);
+            st8<SV8>(t0 + r * S + c8, w);
+            st8<V8>(t1 + r * S + c8, bb);
+        }
+        if (MODE == G_DKV && tid < 32) {
+            const int row = o0 + tid;
+            const bool ok = row < N;
+            const int64_t ro = ((int64_t)b * p.heads + h) * p.row_pad + row;
+            s_lse2[tid] = ok ? p.lse[b * p.lse_sb + h * p.lse_sh + row] * kLog2e : 0.f;
+            s_delta[tid] = ok ? p.delta[ro] : 0.f;
+        }
+    };
+
+    // ---- one step: scores (and dP) of the staged rows against the owner rows ----
+    // z2[j], dpv[j]: other row o0 + 8 g + j against owner row `own`; ok[j]: both rows exist
+    auto tile = [&](int b, int o0, float* z2, float* dpv, bool* ok) __attribute__((always_inline)) {
+        f32x4 sa[2], da[2];
+#pragma unroll
+        for (int a = 0; a < 2; a++) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) { sa[a][i] = 0.f; da[a][i] = 0.f; }
+            const int ar = 8 * (l16 >> 2) + (l16 & 3) + 4 * a;
+#pragma unroll
+            for (int s = 0; s < KS; s++) {
+                const SV8 a0 = ld8<SV8>(t0 + ar * S + 32 * s + 8 * g);
+                sa[a] = Elem<kScoreDT>::mfma16(a0, bs[s], sa[a]);
+                if (MODE != G_FWD) {
+                    const V8 a1 = ld8<V8>(t1 + ar * S + 32 * s + 8 * g);
+                    da[a] = Elem<DT>::mfma16(a1, bp[s], da[a]);
+                }
+            }
+        }
+        const int w = b % p.n_windows;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int other = o0 + 8 * g + j;
+            const int qi = OWNER_IS_KEY ? other : own;
+            const int kj = OWNER_IS_KEY ? own : other;
+            ok[j] = own_ok && other < N;
+            float add = 0.f;
+            if (ok[j]) {
+                if (p.bias) add += (float)reinterpret_cast<const E*>(p.bias)[h * p.bias_sh + (int64_t)qi * p.bias_sn + kj];
+                if (p.mask) {
+                    const int64_t mo = w * p.mask_sw + (int64_t)qi * p.mask_sn + kj;
+                    add += p.mask_f32 ? reinterpret_cast<const float*>(p.mask)[mo]
+                                      : (float)reinterpret_cast<const E*>(p.mask)[mo];
+                }
+            }
+            z2[j] = sa[j >> 2][j & 3] * scale2 + add * kLog2e;
+            dpv[j] = da[j >> 2][j & 3];
+        }
+    };
+    // A operand = transpose of the staged tile, slab c, half dt: rows d = 32 c + 8 (m / 4) + 4 dt + m % 4,
+    // so that this lane's accumulators hold d = 32 c + 8 g + 4 dt + i of its owner row
+    auto tr0 = [&](int c, int dt) __attribute__((always_inline)) -> SV8 {
+        const SE* lo = t0 + (8 * g + (l16 >> 2)) * S + 32 * c + 8 * (l16 & 3) + 4 * dt;
+        return lds_tr8<kScoreDT>(lo, lo + 4 * S);
+    };
+    auto tr1 = [&](int c, int dt) __attribute__((always_inline)) -> V8 {
+        const E* lo = t1 + (8 * g + (l16 >> 2)) * S + 32 * c + 8 * (l16 & 3) + 4 * dt;
+        return lds_tr8<DT>(lo, lo + 4 * S);
+    };
+
+    f32x4 acc0[KS][2], acc1[KS][2];     // FWD: o; DQ: dq^; DKV: dk^ and dv
+#pragma unroll
+    for (int c = 0; c < KS; c++)
+#pragma unroll
+        for (int dt = 0; dt < 2; dt++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) { acc0[c][dt][i] = 0.f; acc1[c][dt][i] = 0.f; }
+
+    if (MODE == G_DBIAS) {
+        float db[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) db[j] = 0.f;
+        for (int b = b0; b < p.bw; b += p.groups) {
+            load_owner(b);
+            __syncthreads();
+            stage(b, 32 * kb);
+            __syncthreads();
+            float z2[8], dpv[8];
+            bool ok[8];
+            tile(b, 32 * kb, z2, dpv, ok);
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                float pr = ok[j] ? fast_exp2(z2[j] - own_lse2) : 0.f;
+                if (!(pr == pr)) pr = 0.f;     // a fully masked row: z2 = lse = -inf
+                db[j] += pr * (dpv[j] - own_delta);
+            }
+        }
+        if (own_ok) {
+            float* dst = p.part_dbias + (((int64_t)grp * p.heads + h) * N + own) * N;
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const int kj = 32 * kb + 8 * g + j;
+                if (kj < N) dst[kj] = db[j];
+            }
+        }
+        return;
+    }
+
+    const int b = b0;
+    load_owner(b);
+    float m_run = -INFINITY, l_run = 0.f;
+    for (int o0 = 0; o0 < N; o0 += 32) {
+        __syncthreads();
+        stage(b, o0);
+        __syncthreads();
+        float z2[8], dpv[8];
+        bool ok[8];
+        tile(b, o0, z2, dpv, ok);
+        if (MODE == G_FWD) {
+            float mloc = -INFINITY;
+#pragma unroll
+            for (int j = 0; j < 8; j++) mloc = fmaxf(mloc, ok[j] ? z2[j] : -INFINITY);
+            const float mnew = fmaxf(m_run, col_max(mloc));
+            const float msafe = mnew == -INFINITY ? 0.f : mnew;
+            const float alpha = fast_exp2(m_run - msafe);
+            V8 pb;
+            float ls = 0.f;
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const float pr = ok[j] ? fast_exp2(z2[j] - msafe) : 0.f;
+                ls += pr;
+                pb[j] = (E)pr;
+            }
+            l_run = l_run * alpha + ls;
+            m_run = mnew;
+#pragma unroll
+            for (int c = 0; c < KS; c++)
+#pragma unroll
+                for (int dt = 0; dt < 2; dt++) {
+#pragma unroll
+                    for (int i = 0; i < 4; i++) acc0[c][dt][i] *= alpha;
+                    acc0[c][dt] = Elem<DT>::mfma16(tr1(c, dt), pb, acc0[c][dt]);
+                }
+        } else {
+            V8 pb;
+            SV8 zb;
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const float l2 = OWNER_IS_KEY ? s_lse2[8 * g + j] : own_lse2;
+                const float dl = OWNER_IS_KEY ? s_delta[8 * g + j] : own_delta;
+                float pr = ok[j] ? fast_exp2(z2[j] - l2) : 0.f;
+                if (!(pr == pr)) pr = 0.f;     // a fully masked row: z2 = lse = -inf
+                pb[j] = (E)pr;
+                zb[j] = (SE)(pr * (dpv[j] - dl));
+            }
+#pragma unroll
+            for (int c = 0; c < KS; c++)
+#pragma unroll
+                for (int dt = 0; dt < 2; dt++) {
+                    acc0[c][dt] = Elem<kScoreDT>::mfma16(tr0(c, dt), zb, acc0[c][dt]);
+                    if (MODE == G_DKV) acc1[c][dt] = Elem<DT>::mfma16(tr1(c, dt), pb, acc1[c][dt]);
+                }
+        }
+    }
+
+    // ---- epilogue: this lane holds columns 32 c + 8 g + 4 dt + i of its owner row ----
+    if (MODE == G_FWD) {
+        const float l_tot = col_add(l_run);
+        const float inv_l = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+        if (own_ok) {
+            E* orow = reinterpret_cast<E*>(const_cast<void*>(p.o.ptr)) + b * p.o.sb + h * p.o.sh + (int64_t)own * p.o.sn;
+#pragma unroll
+            for (int c = 0; c < KS; c++)
+#pragma unroll
+                for (int dt = 0; dt < 2; dt++) {
+                    const int col = 32 * c + 8 * g + 4 * dt;
+                    if (col < d) {
+                        V4 ov;
+#pragma unroll
+                        for (int i = 0; i < 4; i++) ov[i] = (E)(acc0[c][dt][i] * inv_l);
+                        *reinterpret_cast<V4*>(orow + col) = ov;
+                    }
+                }
+            if (g == 0)
+                p.lse[b * p.lse_sb + h * p.lse_sh + own] = l_tot > 0.f ? (m_run + fast_log2(l_tot)) * kLn2 : -INFINITY;
+        }
+        return;
+    }
+
+    // dq = (dq^ - q^ (q^ . dq^)) / ||q||, dq^ = s * acc (the same for dk with k); dv = acc1
+    {
+        const T4& ts = OWNER_IS_KEY ? p.k : p.q;
+        const T4& td = OWNER_IS_KEY ? p.dk : p.dq;
+        float xh[KS][2][4];
+        float proj = 0.f;
+#pragma unroll
+        for (int c = 0; c < KS; c++)
+#pragma unroll
+            for (int dt = 0; dt < 2; dt++) {
+                const int col = 32 * c + 8 * g + 4 * dt;
+                V4 xv;
+#pragma unroll
+                for (int i = 0; i < 4; i++) xv[i] = (E)0.f;
+                if (own_ok && col < d) xv = *reinterpret_cast<const V4*>(rowp(ts, b, own) + col);
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    xh[c][dt][i] = (float)xv[i] * own_inv;
+                    acc0[c][dt][i] *= scale_nat;
+                    proj += xh[c][dt][i] * acc0[c][dt][i];
+                }
+            }
+        proj = col_add(proj);
+        if (own_ok) {
+            E* drow = reinterpret_cast<E*>(const_cast<void*>(td.ptr)) + b * td.sb + h * td.sh + (int64_t)own * td.sn;
+            E* vrow = reinterpret_cast<E*>(const_cast<void*>(p.dv.ptr)) + b * p.dv.sb + h * p.dv.sh + (int64_t)own * p.dv.sn;
+#pragma unroll
+            for (int c = 0; c < KS; c++)
+#pragma unroll
+                for (int dt = 0; dt < 2; dt++) {
+                    const int col = 32 * c + 8 * g + 4 * dt;
+                    if (col < d) {
+                        V4 ov, vv;
+#pragma unroll
+                        for (int i = 0; i < 4; i++) {
+                            ov[i] = (E)((acc0[c][dt][i] - xh[c][dt][i] * proj) * own_inv);
+                            vv[i] = (E)acc1[c][dt][i];
+                        }
+                        *reinterpret_cast<V4*>(drow + col) = ov;
+                        if (MODE == G_DKV) *reinterpret_cast<V4*>(vrow + col) = vv;
+                    }
+                }
+            if (MODE == G_DQ && g == 0) p.dscale_rows[((int64_t)b * p.heads + h) * p.row_pad + own] = proj;
+        }
+    }
+}
+
+// dbias[h, q, k] = sum over the groups' partial tiles, in order.
+template <int DT>
+__global__ void __launch_bounds__(256) generic_dbias_reduce(const GenParams p) {
+    typedef typename Elem<DT>::E E;
+    const int64_t per = (int64_t)p.heads * p.n * p.n;
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= per) return;
+    float s = 0.f;
+    for (int g = 0; g < p.groups; g++) s += p.part_dbias[g * per + i];
+    reinterpret_cast<E*>(p.dbias)[i] = (E)s;
+}
+
+// dlogit_scale[h] = [l <= ln 100] * sum over every query row of the head, in a fixed order.
+template <int DT>
+__global__ void __launch_bounds__(256) generic_dscale_reduce(const GenParams p) {
+    typedef typename Elem<DT>::E E;
+    __shared__ float part[256];
+    const int h = blockIdx.x;
+    float s = 0.f;
+    const int64_t total = (int64_t)p.bw * p.n;
+    for (int64_t i = threadIdx.x; i < total; i += 256) {
+        const int64_t b = i / p.n;
+        const int q = (int)(i - b * p.n);
+        s += p.dscale_rows[(b * p.heads + h) * p.row_pad + q];
+    }
+    part[threadIdx.x] = s;
+    __syncthreads();
+    for (int off = 128; off >= 1; off >>= 1) {
+        if ((int)threadIdx.x < off) part[threadIdx.x] += part[threadIdx.x + off];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        const float ls = (float)reinterpret_cast<const E*>(p.logit_scale)[h];
+        reinterpret_cast<E*>(p.dscale)[h] = (E)(ls <= kLn100 ? part[0] : 0.f);
+    }
+}
+
+// ---- host side -----------------------------------------------------------------
+static size_t align256g(size_t x) { return (x + 255) & ~(size_t)255; }
+
+static int generic_groups(int heads, int n, int bw) {
+    const int64_t tiles = (int64_t)heads * ((n + 63) / 64) * ((n + 31) / 32);
+    int64_t groups = 2048 / tiles;
+    if (groups < 1) groups = 1;
+    if (groups > 64) groups = 64;
+    if (groups > bw) groups = bw;
+    return (int)groups;
+}
+
+bool generic_head_dim(int d) { return d != 32; }
+
+size_t generic_workspace_bytes(int heads, int n, int bw, bool has_bias) {
+    const size_t row_pad = (size_t)((n + 63) / 64) * 64;
+    size_t total = 2 * align256g((size_t)bw * heads * row_pad * sizeof(float));
+    if (has_bias) total += align256g((size_t)generic_groups(heads, n, bw) * heads * n * n * sizeof(float));
+    return total;
+}
+
+template <int DT, int D>
+static hipError_t launch_generic_d(const GenParams& p, bool backward, hipStream_t st) {
+    const int chunks = (p.n + 63) / 64, kblocks = (p.n + 31) / 32;
+    const dim3 grid((unsigned)((int64_t)p.bw * p.heads * chunks)), block(256);
+    if (!backward) {
+        hipLaunchKernelGGL((generic_kernel<DT, D, G_FWD>), grid, block, 0, st, p);
+        return hipGetLastError();
+    }
+    hipLaunchKernelGGL((generic_kernel<DT, D, G_DQ>), grid, block, 0, st, p);
+    hipLaunchKernelGGL((generic_kernel<DT, D, G_DKV>), grid, block, 0, st, p);
+    if (p.bias) {
+        const dim3 gb((unsigned)((int64_t)p.groups * p.heads * chunks * kblocks));
+        hipLaunchKernelGGL((generic_kernel<DT, D, G_DBIAS>), gb, block, 0, st, p);
+        const int64_t per = (int64_t)p.heads * p.n * p.n;
+        hipLaunchKernelGGL(generic_dbias_reduce<DT>, dim3((unsigned)((per + 255) / 256)), block, 0, st, p);
+    }
+    if (p.scale_kind == FWA2_SCALE_TENSOR && p.dscale)
+        hipLaunchKernelGGL(generic_dscale_reduce<DT>, dim3(p.heads), block, 0, st, p);
+    return hipGetLastError();
+}
+
+template <int DT>
+static hipError_t launch_generic_dt(const GenParams& p, bool backward, hipStream_t st) {
+    if (p.d <= 32) return launch_generic_d<DT, 32>(p, backward, st);
+    if (p.d <= 64) return launch_generic_d<DT, 64>(p, backward, st);
+    return launch_generic_d<DT, 128>(p, backward, st);
+}
+
+// p: the caller's problem, already validated.  workspace (backward only): generic_workspace_bytes().
+hipError_t launch_generic(const fwa2_problem* pr, bool backward) {
+    GenParams p;
+    memset(&p, 0, sizeof(p));
+    auto t4 = [](const fwa2_tensor4& t) { return T4{t.ptr, t.stride_bw, t.stride_h, t.stride_n}; };
+    p.q = t4(pr->q); p.k = t4(pr->k); p.v = t4(pr->v); p.o = t4(pr->o);
+    p.d_o = t4(pr->d_o); p.dq = t4(pr->dq); p.dk = t4(pr->dk); p.dv = t4(pr->dv);
+    p.logit_scale = pr->logit_scale;
+    p.scale_kind = pr->scale_kind;
+    p.default_scale = 1.0f / sqrtf((float)pr->head_dim);
+    p.bias = pr->bias.ptr; p.bias_sh = pr->bias.stride_a; p.bias_sn = pr->bias.stride_n;
+    p.mask = pr->mask.ptr; p.mask_sw = pr->mask.stride_a; p.mask_sn = pr->mask.stride_n;
+    p.mask_f32 = pr->mask.ptr && pr->mask_dtype == FWA2_F32;
+    p.n_windows = pr->mask.ptr ? pr->n_windows : 1;
+    p.lse = pr->lse; p.lse_sb = pr->lse_stride_bw; p.lse_sh = pr->lse_stride_h;
+    p.bw = pr->bw; p.heads = pr->heads; p.n = pr->n; p.d = pr->head_dim;
+    p.row_pad = ((pr->n + 63) / 64) * 64;
+    if (backward) {
+        unsigned char* ws = reinterpret_cast<unsigned char*>(pr->workspace);
+        const size_t rows = align256g((size_t)p.bw * p.heads * p.row_pad * sizeof(float));
+        p.delta = reinterpret_cast<float*>(ws);
+        p.dscale_rows = reinterpret_cast<float*>(ws + rows);
+        p.part_dbias = reinterpret_cast<float*>(ws + 2 * rows);
+        p.groups = generic_groups(p.heads, p.n, p.bw);
+        p.dbias = pr->dbias;
+        p.dscale = pr->dscale;
+    }
+    hipStream_t st = (hipStream_t)pr->stream;
+    if (pr->dtype == FWA2_BF16) return launch_generic_dt<FWA2_BF16>(p, backward, st);
+    return launch_generic_dt<FWA2_F16>(p, backward, st);
+}
+
+}  // namespace fwa2

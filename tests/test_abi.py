@@ -67,8 +67,13 @@ def test_validate_accepts_and_rejects(lib):
     assert lib.fwa2_validate(p, 0) == _abi.ERR_INVALID_ARGUMENT and b"up to 128" in lib.fwa2_last_error()
 
     p = _good_problem()
-    p.head_dim = 64
-    assert lib.fwa2_validate(p, 0) == _abi.ERR_UNSUPPORTED
+    p.head_dim = 20     # rows are read in 16-byte chunks
+    assert lib.fwa2_validate(p, 0) == _abi.ERR_UNSUPPORTED and b"multiples of 8" in lib.fwa2_last_error()
+    for hd in (8, 16, 24, 32):
+        p.head_dim = hd
+        assert lib.fwa2_validate(p, 0) == _abi.OK
+    p.head_dim = 64     # the row stride of _good_problem is 32
+    assert lib.fwa2_validate(p, 0) == _abi.ERR_INVALID_ARGUMENT and b"overlaps rows" in lib.fwa2_last_error()
 
     p = _good_problem()
     p.q = _abi.Tensor4(0x10002, 4096, 2048, 32)  # rows not 16-byte aligned
@@ -102,7 +107,7 @@ def test_workspace_size_is_reported(lib):
 
 def test_status_to_exception(lib):
     p = _good_problem()
-    p.head_dim = 64
+    p.head_dim = 20
     with pytest.raises(NotImplementedError):
         _abi.check(lib.fwa2_validate(p, 0), "validate")
     p.head_dim = 200

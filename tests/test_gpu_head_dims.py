@@ -1,0 +1,50 @@
+"""GPU parity for head dimensions other than 32: the reference supports any head dimension up to 128
+(flash_win_attn_v2/kernels/attn_kernel_forward.py:267, 298).  Same oracle, same tolerances as the d = 32 tests
+(bf16: max abs 2e-2 on o, 5e-2 relative on every gradient; fp16: 5e-3 / 2e-2)."""
+import pytest
+import torch
+
+from oracle.swin_inputs import make_inputs
+from tests.test_gpu_parity import _run_and_check
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("d", [8, 16, 24, 48, 64, 96, 128])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_head_dims_with_shift_mask(d, dtype):
+    inp = make_inputs(batch=2, n_windows=4, heads=3, n=64, d=d, dtype=dtype, seed=d, resolution=16, window=8, shift=4)
+    _run_and_check(inp, dtype, tag=f"d{d}")
+
+
+@pytest.mark.parametrize("n,res,win,shift", [(49, 14, 7, 3), (144, 24, 12, 6), (256, 32, 16, 8), (16, 8, 4, 2)])
+@pytest.mark.parametrize("d", [16, 64, 128])
+def test_head_dims_across_window_sizes(n, res, win, shift, d):
+    nw = (res // win) ** 2
+    inp = make_inputs(batch=2, n_windows=nw, heads=2, n=n, d=d, dtype=torch.bfloat16, seed=n + d, resolution=res,
+                      window=win, shift=shift)
+    _run_and_check(inp, torch.bfloat16, tag=f"N{n}d{d}")
+
+
+@pytest.mark.parametrize("with_scale,with_bias,with_mask", [(0, 1, 1), (1, 0, 1), (1, 1, 0), (0, 0, 0)])
+def test_head_dim_64_optional_arguments(with_scale, with_bias, with_mask):
+    inp = make_inputs(batch=2, n_windows=4, heads=2, n=64, d=64, dtype=torch.bfloat16, seed=5, resolution=16, window=8,
+                      shift=4, with_scale=bool(with_scale), with_bias=bool(with_bias), with_mask=bool(with_mask))
+    _run_and_check(inp, torch.bfloat16, tag=f"opt{with_scale}{with_bias}{with_mask}")
+
+
+def test_head_dim_64_ragged_window_fp32_mask_and_clamped_scale():
+    """N = 37 (not a multiple of anything), fp32 mask next to bf16 inputs, many units per dbias group, and a
+    logit scale above ln 100, whose gradient must be exactly zero."""
+    inp = make_inputs(batch=70, n_windows=1, heads=2, n=37, d=64, dtype=torch.bfloat16, seed=8, with_mask=False)
+    g = torch.Generator().manual_seed(9)
+    inp["mask"] = torch.where(torch.rand(1, 37, 37, generator=g) < 0.3, -100.0, 0.0)  # fp32
+    inp["logit_scale"][1] = 5.0
+    _run_and_check(inp, torch.bfloat16, tag="ragged", dscale_l1_frac=0.1)
+
+
+def test_head_dim_must_be_a_multiple_of_8():
+    from flash_window_attention_v2_amd import flash_win_attn_v2_func
+    q = torch.randn(2, 2, 16, 20, device="cuda", dtype=torch.bfloat16)
+    with pytest.raises(NotImplementedError, match="multiples of 8"):
+        flash_win_attn_v2_func(q, q, q)
