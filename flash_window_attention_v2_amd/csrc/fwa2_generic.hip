@@ -13,7 +13,9 @@
 //   FWD    owner = queries, other = keys:     online softmax, O^T += V^T P^T
 //   DQ     owner = queries, other = keys:     delta = rowsum(o * dO), dQ^^T += K^^T dZ^T; per-row dscale terms
 //   DKV    owner = keys,    other = queries:  dK^^T += Q^^T dZ, dV^T += dO^T P
-//   DBIAS  owner = queries, other = 32 keys:  loops over the units of a group, sums dZ per (query, key)
+//   DBIAS  owner = queries, other = 32 keys:  loops over the units of a group, sums dZ per (query, key);
+//          only for windows of more than 256 tokens: up to there DQ walks a group of units itself and
+//          keeps the dZ sums of its 16 x N strip in registers
 //
 // Every score tile is v_mfma_f32_16x16x32 with the other rows as A rows and the owner rows as B columns, so
 // a lane holds, for its owner row, the 8 consecutive other rows 8g .. 8g+7 (g = lane / 16) of the step: the
@@ -46,6 +48,8 @@ struct GenParams {
     int64_t mask_sw, mask_sn;
     int mask_f32;
     int n_windows;
+    const uint8_t* mask_live;   // [n_windows] 0 = the window's mask is all zero; nullptr = unknown
+    int side_vec;               // rows of bias and mask may be read with 16-byte loads and n % 8 == 0
     float* lse;
     int64_t lse_sb, lse_sh;
     int bw, heads, n, d;
@@ -58,8 +62,11 @@ struct GenParams {
     void* dscale;         // [H] input dtype
 };
 
-template <int DT, int D, int MODE>
+// WITH_DB (DQ only, windows of up to 256 tokens): the workgroup walks the units of a group and also sums
+// dZ per (query, key) in registers, which saves the separate DBIAS pass.
+template <int DT, int D, int MODE, bool WITH_DB = false>
 __global__ void __launch_bounds__(256) generic_kernel(const GenParams p) {
+    static_assert(!WITH_DB || MODE == G_DQ, "dbias rides on the dq pass only");
     typedef typename Elem<DT>::E E;
     typedef typename Elem<DT>::V8 V8;
     typedef typename Elem<DT>::V4 V4;
@@ -73,6 +80,8 @@ __global__ void __launch_bounds__(256) generic_kernel(const GenParams p) {
     __shared__ __attribute__((aligned(16))) SE t0[32 * S];   // other rows, normalised (k^ or q^)
     __shared__ __attribute__((aligned(16))) E t1[32 * S];    // other rows of v (or dO)
     __shared__ float s_lse2[32], s_delta[32];                // DKV: lse log2(e) and delta of the other rows
+    constexpr int AS = 68;                                   // row stride of s_add
+    __shared__ float s_add[MODE == G_DKV ? 32 * AS : 1];     // DKV: (bias + mask) log2(e), [other query][owner key]
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -90,7 +99,7 @@ __global__ void __launch_bounds__(256) generic_kernel(const GenParams p) {
     idx /= chunks;
     const int h = idx % p.heads;
     idx /= p.heads;
-    if (MODE == G_DBIAS) { grp = idx; b0 = grp; } else { b0 = idx; }
+    if (MODE == G_DBIAS || WITH_DB) { grp = idx; b0 = grp; } else { b0 = idx; }
 
     const int own = own0 + 16 * wave + l16;     // owner row of this lane's column
     const bool own_ok = own < N;
@@ -184,6 +193,52 @@ __global__ void __launch_bounds__(256) generic_kernel(const GenParams p) {
             st8<SV8>(t0 + r * S + c8, w);
             st8<V8>(t1 + r * S + c8, bb);
         }
+        if (MODE == G_DKV) {
+            // (bias + mask) of the 32 staged queries against the 64 owner keys, read along the rows of the
+            // tables (the owner lanes need a column of them)
+            const int r = tid >> 3, c8 = (tid & 7) * 8;
+            const int qi = o0 + r, k0 = own0 + c8;
+            const int w = b % p.n_windows;
+            const bool mask_on = p.mask && (!p.mask_live || p.mask_live[w] != 0);
+            float add[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) add[j] = 0.f;
+            if (qi < N) {
+                const E* bptr = reinterpret_cast<const E*>(p.bias) + h * p.bias_sh + (int64_t)qi * p.bias_sn + k0;
+                const int64_t mo = w * p.mask_sw + (int64_t)qi * p.mask_sn + k0;
+                if (p.side_vec) {
+                    if (k0 < N) {
+                        if (p.bias) {
+                            const V8 bv = ld8<V8>(bptr);
+#pragma unroll
+                            for (int j = 0; j < 8; j++) add[j] += (float)bv[j];
+                        }
+                        if (mask_on && p.mask_f32) {
+                            const f32x4 m0 = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(p.mask) + mo);
+                            const f32x4 m1 = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(p.mask) + mo + 4);
+#pragma unroll
+                            for (int j = 0; j < 4; j++) { add[j] += m0[j]; add[4 + j] += m1[j]; }
+                        } else if (mask_on) {
+                            const V8 mv = ld8<V8>(reinterpret_cast<const E*>(p.mask) + mo);
+#pragma unroll
+                            for (int j = 0; j < 8; j++) add[j] += (float)mv[j];
+                        }
+                    }
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 8; j++) {
+                        if (k0 + j < N) {
+                            if (p.bias) add[j] += (float)bptr[j];
+                            if (mask_on)
+                                add[j] += p.mask_f32 ? reinterpret_cast<const float*>(p.mask)[mo + j]
+                                                     : (float)reinterpret_cast<const E*>(p.mask)[mo + j];
+                        }
+                    }
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < 8; j++) s_add[r * AS + c8 + j] = add[j] * kLog2e;
+        }
         if (MODE == G_DKV && tid < 32) {
             const int row = o0 + tid;
             const bool ok = row < N;
@@ -213,22 +268,58 @@ __global__ void __launch_bounds__(256) generic_kernel(const GenParams p) {
             }
         }
         const int w = b % p.n_windows;
+        // a window whose mask is known to be all zero needs no mask reads
+        const bool mask_on = p.mask && (!p.mask_live || p.mask_live[w] != 0);
+        float add[8];
 #pragma unroll
         for (int j = 0; j < 8; j++) {
-            const int other = o0 + 8 * g + j;
-            const int qi = OWNER_IS_KEY ? other : own;
-            const int kj = OWNER_IS_KEY ? own : other;
-            ok[j] = own_ok && other < N;
-            float add = 0.f;
-            if (ok[j]) {
-                if (p.bias) add += (float)reinterpret_cast<const E*>(p.bias)[h * p.bias_sh + (int64_t)qi * p.bias_sn + kj];
-                if (p.mask) {
-                    const int64_t mo = w * p.mask_sw + (int64_t)qi * p.mask_sn + kj;
-                    add += p.mask_f32 ? reinterpret_cast<const float*>(p.mask)[mo]
-                                      : (float)reinterpret_cast<const E*>(p.mask)[mo];
+            ok[j] = own_ok && o0 + 8 * g + j < N;
+            add[j] = 0.f;
+        }
+        if (OWNER_IS_KEY) {
+#pragma unroll
+            for (int j = 0; j < 8; j++) add[j] = s_add[(8 * g + j) * AS + 16 * wave + l16];
+        } else if (p.side_vec) {
+            // the 8 keys of this lane are consecutive entries of one bias / mask row; n % 8 == 0, so they
+            // exist together or not at all
+            if (ok[0]) {
+                const int64_t ro = (int64_t)own * p.bias_sn + o0 + 8 * g;
+                if (p.bias) {
+                    const V8 bv = ld8<V8>(reinterpret_cast<const E*>(p.bias) + h * p.bias_sh + ro);
+#pragma unroll
+                    for (int j = 0; j < 8; j++) add[j] += (float)bv[j];
+                }
+                if (mask_on) {
+                    const int64_t mo = w * p.mask_sw + (int64_t)own * p.mask_sn + o0 + 8 * g;
+                    if (p.mask_f32) {
+                        const f32x4 m0 = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(p.mask) + mo);
+                        const f32x4 m1 = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(p.mask) + mo + 4);
+#pragma unroll
+                        for (int j = 0; j < 4; j++) { add[j] += m0[j]; add[4 + j] += m1[j]; }
+                    } else {
+                        const V8 mv = ld8<V8>(reinterpret_cast<const E*>(p.mask) + mo);
+#pragma unroll
+                        for (int j = 0; j < 8; j++) add[j] += (float)mv[j];
+                    }
                 }
             }
-            z2[j] = sa[j >> 2][j & 3] * scale2 + add * kLog2e;
+        } else {
+            const int k0 = o0 + 8 * g;
+            const E* bptr = reinterpret_cast<const E*>(p.bias) + h * p.bias_sh + (int64_t)own * p.bias_sn + k0;
+            const int64_t mo = w * p.mask_sw + (int64_t)own * p.mask_sn + k0;
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                if (ok[j]) {
+                    if (p.bias) add[j] += (float)bptr[j];
+                    if (mask_on)
+                        add[j] += p.mask_f32 ? reinterpret_cast<const float*>(p.mask)[mo + j]
+                                             : (float)reinterpret_cast<const E*>(p.mask)[mo + j];
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            z2[j] = sa[j >> 2][j & 3] * scale2 + (OWNER_IS_KEY ? add[j] : add[j] * kLog2e);
             dpv[j] = da[j >> 2][j & 3];
         }
     };
@@ -281,89 +372,8 @@ __global__ void __launch_bounds__(256) generic_kernel(const GenParams p) {
         return;
     }
 
-    const int b = b0;
-    load_owner(b);
-    float m_run = -INFINITY, l_run = 0.f;
-    for (int o0 = 0; o0 < N; o0 += 32) {
-        __syncthreads();
-        stage(b, o0);
-        __syncthreads();
-        float z2[8], dpv[8];
-        bool ok[8];
-        tile(b, o0, z2, dpv, ok);
-        if (MODE == G_FWD) {
-            float mloc = -INFINITY;
-#pragma unroll
-            for (int j = 0; j < 8; j++) mloc = fmaxf(mloc, ok[j] ? z2[j] : -INFINITY);
-            const float mnew = fmaxf(m_run, col_max(mloc));
-            const float msafe = mnew == -INFINITY ? 0.f : mnew;
-            const float alpha = fast_exp2(m_run - msafe);
-            V8 pb;
-            float ls = 0.f;
-#pragma unroll
-            for (int j = 0; j < 8; j++) {
-                const float pr = ok[j] ? fast_exp2(z2[j] - msafe) : 0.f;
-                ls += pr;
-                pb[j] = (E)pr;
-            }
-            l_run = l_run * alpha + ls;
-            m_run = mnew;
-#pragma unroll
-            for (int c = 0; c < KS; c++)
-#pragma unroll
-                for (int dt = 0; dt < 2; dt++) {
-#pragma unroll
-                    for (int i = 0; i < 4; i++) acc0[c][dt][i] *= alpha;
-                    acc0[c][dt] = Elem<DT>::mfma16(tr1(c, dt), pb, acc0[c][dt]);
-                }
-        } else {
-            V8 pb;
-            SV8 zb;
-#pragma unroll
-            for (int j = 0; j < 8; j++) {
-                const float l2 = OWNER_IS_KEY ? s_lse2[8 * g + j] : own_lse2;
-                const float dl = OWNER_IS_KEY ? s_delta[8 * g + j] : own_delta;
-                float pr = ok[j] ? fast_exp2(z2[j] - l2) : 0.f;
-                if (!(pr == pr)) pr = 0.f;     // a fully masked row: z2 = lse = -inf
-                pb[j] = (E)pr;
-                zb[j] = (SE)(pr * (dpv[j] - dl));
-            }
-#pragma unroll
-            for (int c = 0; c < KS; c++)
-#pragma unroll
-                for (int dt = 0; dt < 2; dt++) {
-                    acc0[c][dt] = Elem<kScoreDT>::mfma16(tr0(c, dt), zb, acc0[c][dt]);
-                    if (MODE == G_DKV) acc1[c][dt] = Elem<DT>::mfma16(tr1(c, dt), pb, acc1[c][dt]);
-                }
-        }
-    }
-
-    // ---- epilogue: this lane holds columns 32 c + 8 g + 4 dt + i of its owner row ----
-    if (MODE == G_FWD) {
-        const float l_tot = col_add(l_run);
-        const float inv_l = l_tot > 0.f ? 1.0f / l_tot : 0.f;
-        if (own_ok) {
-            E* orow = reinterpret_cast<E*>(const_cast<void*>(p.o.ptr)) + b * p.o.sb + h * p.o.sh + (int64_t)own * p.o.sn;
-#pragma unroll
-            for (int c = 0; c < KS; c++)
-#pragma unroll
-                for (int dt = 0; dt < 2; dt++) {
-                    const int col = 32 * c + 8 * g + 4 * dt;
-                    if (col < d) {
-                        V4 ov;
-#pragma unroll
-                        for (int i = 0; i < 4; i++) ov[i] = (E)(acc0[c][dt][i] * inv_l);
-                        *reinterpret_cast<V4*>(orow + col) = ov;
-                    }
-                }
-            if (g == 0)
-                p.lse[b * p.lse_sb + h * p.lse_sh + own] = l_tot > 0.f ? (m_run + fast_log2(l_tot)) * kLn2 : -INFINITY;
-        }
-        return;
-    }
-
     // dq = (dq^ - q^ (q^ . dq^)) / ||q||, dq^ = s * acc (the same for dk with k); dv = acc1
-    {
+    auto finish_grad = [&](int b) __attribute__((always_inline)) {
         const T4& ts = OWNER_IS_KEY ? p.k : p.q;
         const T4& td = OWNER_IS_KEY ? p.dk : p.dq;
         float xh[KS][2][4];
@@ -406,33 +416,162 @@ __global__ void __launch_bounds__(256) generic_kernel(const GenParams p) {
                 }
             if (MODE == G_DQ && g == 0) p.dscale_rows[((int64_t)b * p.heads + h) * p.row_pad + own] = proj;
         }
+    };
+
+    float m_run = -INFINITY, l_run = 0.f;
+    // one step of 32 other rows; dbr: this lane's 8 dbias sums of the step (WITH_DB) or nullptr
+    auto step = [&](int b, int o0, float* dbr) __attribute__((always_inline)) {
+        __syncthreads();
+        stage(b, o0);
+        __syncthreads();
+        float z2[8], dpv[8];
+        bool ok[8];
+        tile(b, o0, z2, dpv, ok);
+        if (MODE == G_FWD) {
+            float mloc = -INFINITY;
+#pragma unroll
+            for (int j = 0; j < 8; j++) mloc = fmaxf(mloc, ok[j] ? z2[j] : -INFINITY);
+            const float mnew = fmaxf(m_run, col_max(mloc));
+            const float msafe = mnew == -INFINITY ? 0.f : mnew;
+            const float alpha = fast_exp2(m_run - msafe);
+            V8 pb;
+            float ls = 0.f;
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const float pr = ok[j] ? fast_exp2(z2[j] - msafe) : 0.f;
+                ls += pr;
+                pb[j] = (E)pr;
+            }
+            l_run = l_run * alpha + ls;
+            m_run = mnew;
+#pragma unroll
+            for (int c = 0; c < KS; c++)
+#pragma unroll
+                for (int dt = 0; dt < 2; dt++) {
+#pragma unroll
+                    for (int i = 0; i < 4; i++) acc0[c][dt][i] *= alpha;
+                    acc0[c][dt] = Elem<DT>::mfma16(tr1(c, dt), pb, acc0[c][dt]);
+                }
+        } else {
+            V8 pb;
+            SV8 zb;
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const float l2 = OWNER_IS_KEY ? s_lse2[8 * g + j] : own_lse2;
+                const float dl = OWNER_IS_KEY ? s_delta[8 * g + j] : own_delta;
+                float pr = ok[j] ? fast_exp2(z2[j] - l2) : 0.f;
+                if (!(pr == pr)) pr = 0.f;     // a fully masked row: z2 = lse = -inf
+                pb[j] = (E)pr;
+                const float dz = pr * (dpv[j] - dl);
+                zb[j] = (SE)dz;
+                if (WITH_DB) dbr[j] += dz;
+            }
+#pragma unroll
+            for (int c = 0; c < KS; c++)
+#pragma unroll
+                for (int dt = 0; dt < 2; dt++) {
+                    acc0[c][dt] = Elem<kScoreDT>::mfma16(tr0(c, dt), zb, acc0[c][dt]);
+                    if (MODE == G_DKV) acc1[c][dt] = Elem<DT>::mfma16(tr1(c, dt), pb, acc1[c][dt]);
+                }
+        }
+    };
+
+    if (WITH_DB) {
+        float db[8][8];
+#pragma unroll
+        for (int t = 0; t < 8; t++)
+#pragma unroll
+            for (int j = 0; j < 8; j++) db[t][j] = 0.f;
+        for (int b = b0; b < p.bw; b += p.groups) {
+            load_owner(b);
+#pragma unroll
+            for (int c = 0; c < KS; c++)
+#pragma unroll
+                for (int dt = 0; dt < 2; dt++)
+#pragma unroll
+                    for (int i = 0; i < 4; i++) acc0[c][dt][i] = 0.f;
+#pragma unroll
+            for (int t = 0; t < 8; t++)
+                if (32 * t < N) step(b, 32 * t, db[t]);
+            finish_grad(b);
+        }
+        if (own_ok) {
+            float* dst = p.part_dbias + (((int64_t)grp * p.heads + h) * N + own) * N;
+#pragma unroll
+            for (int t = 0; t < 8; t++)
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    const int kj = 32 * t + 8 * g + j;
+                    if (kj < N) dst[kj] = db[t][j];
+                }
+        }
+        return;
     }
+
+    const int b = b0;
+    load_owner(b);
+    for (int o0 = 0; o0 < N; o0 += 32) step(b, o0, nullptr);
+
+    // ---- epilogue: this lane holds columns 32 c + 8 g + 4 dt + i of its owner row ----
+    if (MODE == G_FWD) {
+        const float l_tot = col_add(l_run);
+        const float inv_l = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+        if (own_ok) {
+            E* orow = reinterpret_cast<E*>(const_cast<void*>(p.o.ptr)) + b * p.o.sb + h * p.o.sh + (int64_t)own * p.o.sn;
+#pragma unroll
+            for (int c = 0; c < KS; c++)
+#pragma unroll
+                for (int dt = 0; dt < 2; dt++) {
+                    const int col = 32 * c + 8 * g + 4 * dt;
+                    if (col < d) {
+                        V4 ov;
+#pragma unroll
+                        for (int i = 0; i < 4; i++) ov[i] = (E)(acc0[c][dt][i] * inv_l);
+                        *reinterpret_cast<V4*>(orow + col) = ov;
+                    }
+                }
+            if (g == 0)
+                p.lse[b * p.lse_sb + h * p.lse_sh + own] = l_tot > 0.f ? (m_run + fast_log2(l_tot)) * kLn2 : -INFINITY;
+        }
+        return;
+    }
+
+    if (MODE != G_FWD) finish_grad(b);
 }
 
-// dbias[h, q, k] = sum over the groups' partial tiles, in order.
+// dbias[h, q, k] = sum over the groups' partial tiles in a fixed order: 32 elements per workgroup, the
+// groups dealt to 8 slices that are combined at the end.
 template <int DT>
 __global__ void __launch_bounds__(256) generic_dbias_reduce(const GenParams p) {
     typedef typename Elem<DT>::E E;
+    __shared__ float part[8][32];
     const int64_t per = (int64_t)p.heads * p.n * p.n;
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= per) return;
+    const int e = threadIdx.x & 31, sl = threadIdx.x >> 5;
+    const int64_t i = (int64_t)blockIdx.x * 32 + e;
     float s = 0.f;
-    for (int g = 0; g < p.groups; g++) s += p.part_dbias[g * per + i];
-    reinterpret_cast<E*>(p.dbias)[i] = (E)s;
+    if (i < per)
+        for (int g = sl; g < p.groups; g += 8) s += p.part_dbias[g * per + i];
+    part[sl][e] = s;
+    __syncthreads();
+    if (sl == 0 && i < per) {
+        float t = 0.f;
+#pragma unroll
+        for (int k = 0; k < 8; k++) t += part[k][e];
+        reinterpret_cast<E*>(p.dbias)[i] = (E)t;
+    }
 }
 
-// dlogit_scale[h] = [l <= ln 100] * sum over every query row of the head, in a fixed order.
-template <int DT>
-__global__ void __launch_bounds__(256) generic_dscale_reduce(const GenParams p) {
-    typedef typename Elem<DT>::E E;
+// dlogit_scale[h] = [l <= ln 100] * sum over every query row of the head, in a fixed order: kDsSlices
+// workgroups per head sum the units b = slice, slice + kDsSlices, ... into one partial each (kept in the
+// delta buffer, which nobody reads any more), a last small kernel adds the partials.
+constexpr int kDsSlices = 128;
+__global__ void __launch_bounds__(256) generic_dscale_partial(const GenParams p) {
     __shared__ float part[256];
-    const int h = blockIdx.x;
+    const int h = blockIdx.x / kDsSlices, sl = blockIdx.x % kDsSlices;
     float s = 0.f;
-    const int64_t total = (int64_t)p.bw * p.n;
-    for (int64_t i = threadIdx.x; i < total; i += 256) {
-        const int64_t b = i / p.n;
-        const int q = (int)(i - b * p.n);
-        s += p.dscale_rows[(b * p.heads + h) * p.row_pad + q];
+    for (int b = sl; b < p.bw; b += kDsSlices) {
+        const float* row = p.dscale_rows + ((int64_t)b * p.heads + h) * p.row_pad;
+        for (int q = threadIdx.x; q < p.n; q += 256) s += row[q];
     }
     part[threadIdx.x] = s;
     __syncthreads();
@@ -440,29 +579,53 @@ __global__ void __launch_bounds__(256) generic_dscale_reduce(const GenParams p) 
         if ((int)threadIdx.x < off) part[threadIdx.x] += part[threadIdx.x + off];
         __syncthreads();
     }
-    if (threadIdx.x == 0) {
-        const float ls = (float)reinterpret_cast<const E*>(p.logit_scale)[h];
-        reinterpret_cast<E*>(p.dscale)[h] = (E)(ls <= kLn100 ? part[0] : 0.f);
-    }
+    if (threadIdx.x == 0) p.delta[blockIdx.x] = part[0];
+}
+template <int DT>
+__global__ void __launch_bounds__(64) generic_dscale_final(const GenParams p) {
+    typedef typename Elem<DT>::E E;
+    const int h = blockIdx.x;
+    if (threadIdx.x != 0) return;
+    float s = 0.f;
+    for (int k = 0; k < kDsSlices; k++) s += p.delta[h * kDsSlices + k];
+    const float ls = (float)reinterpret_cast<const E*>(p.logit_scale)[h];
+    reinterpret_cast<E*>(p.dscale)[h] = (E)(ls <= kLn100 ? s : 0.f);
 }
 
 // ---- host side -----------------------------------------------------------------
 static size_t align256g(size_t x) { return (x + 255) & ~(size_t)255; }
 
+constexpr int kDbInDqMaxN = 256;   // windows up to this size sum dbias inside the dq pass
+
+// Unit groups of the pass that sums dbias: enough workgroups to fill the chip, bounded partial tiles.
 static int generic_groups(int heads, int n, int bw) {
-    const int64_t tiles = (int64_t)heads * ((n + 63) / 64) * ((n + 31) / 32);
-    int64_t groups = 2048 / tiles;
+    const int64_t chunks = (n + 63) / 64, kblocks = (n + 31) / 32;
+    int64_t groups;
+    if (n <= kDbInDqMaxN) {
+        groups = 1024 / (heads * chunks);
+        const int64_t cap = ((int64_t)64 << 20) / ((int64_t)heads * n * n * 4);
+        if (groups > cap) groups = cap;
+    } else {
+        groups = 2048 / (heads * chunks * kblocks);
+        if (groups > 64) groups = 64;
+    }
     if (groups < 1) groups = 1;
-    if (groups > 64) groups = 64;
     if (groups > bw) groups = bw;
     return (int)groups;
 }
 
 bool generic_head_dim(int d) { return d != 32; }
 
+// One [BW * H, row_pad] fp32 buffer (delta, dscale rows); never smaller than the dscale partial sums.
+static size_t generic_rows_bytes(int heads, int bw, size_t row_pad) {
+    size_t rows = (size_t)bw * heads * row_pad;
+    if (rows < (size_t)heads * kDsSlices) rows = (size_t)heads * kDsSlices;
+    return align256g(rows * sizeof(float));
+}
+
 size_t generic_workspace_bytes(int heads, int n, int bw, bool has_bias) {
     const size_t row_pad = (size_t)((n + 63) / 64) * 64;
-    size_t total = 2 * align256g((size_t)bw * heads * row_pad * sizeof(float));
+    size_t total = 2 * generic_rows_bytes(heads, bw, row_pad);
     if (has_bias) total += align256g((size_t)generic_groups(heads, n, bw) * heads * n * n * sizeof(float));
     return total;
 }
@@ -475,16 +638,27 @@ static hipError_t launch_generic_d(const GenParams& p, bool backward, hipStream_
         hipLaunchKernelGGL((generic_kernel<DT, D, G_FWD>), grid, block, 0, st, p);
         return hipGetLastError();
     }
-    hipLaunchKernelGGL((generic_kernel<DT, D, G_DQ>), grid, block, 0, st, p);
+    const bool db_in_dq = p.bias && p.n <= kDbInDqMaxN;
+    if (db_in_dq) {
+        const dim3 gq((unsigned)((int64_t)p.groups * p.heads * chunks));
+        hipLaunchKernelGGL((generic_kernel<DT, D, G_DQ, true>), gq, block, 0, st, p);
+    } else {
+        hipLaunchKernelGGL((generic_kernel<DT, D, G_DQ>), grid, block, 0, st, p);
+    }
     hipLaunchKernelGGL((generic_kernel<DT, D, G_DKV>), grid, block, 0, st, p);
     if (p.bias) {
-        const dim3 gb((unsigned)((int64_t)p.groups * p.heads * chunks * kblocks));
-        hipLaunchKernelGGL((generic_kernel<DT, D, G_DBIAS>), gb, block, 0, st, p);
+        if (!db_in_dq) {
+            const dim3 gb((unsigned)((int64_t)p.groups * p.heads * chunks * kblocks));
+            hipLaunchKernelGGL((generic_kernel<DT, D, G_DBIAS>), gb, block, 0, st, p);
+        }
         const int64_t per = (int64_t)p.heads * p.n * p.n;
-        hipLaunchKernelGGL(generic_dbias_reduce<DT>, dim3((unsigned)((per + 255) / 256)), block, 0, st, p);
+        hipLaunchKernelGGL(generic_dbias_reduce<DT>, dim3((unsigned)((per + 31) / 32)), block, 0, st, p);
     }
-    if (p.scale_kind == FWA2_SCALE_TENSOR && p.dscale)
-        hipLaunchKernelGGL(generic_dscale_reduce<DT>, dim3(p.heads), block, 0, st, p);
+    if (p.scale_kind == FWA2_SCALE_TENSOR && p.dscale) {
+        // after DKV and DBIAS (same stream), so the delta buffer is free for the partial sums
+        hipLaunchKernelGGL(generic_dscale_partial, dim3(p.heads * kDsSlices), block, 0, st, p);
+        hipLaunchKernelGGL(generic_dscale_final<DT>, dim3(p.heads), dim3(64), 0, st, p);
+    }
     return hipGetLastError();
 }
 
@@ -509,12 +683,17 @@ hipError_t launch_generic(const fwa2_problem* pr, bool backward) {
     p.mask = pr->mask.ptr; p.mask_sw = pr->mask.stride_a; p.mask_sn = pr->mask.stride_n;
     p.mask_f32 = pr->mask.ptr && pr->mask_dtype == FWA2_F32;
     p.n_windows = pr->mask.ptr ? pr->n_windows : 1;
+    p.mask_live = pr->mask.ptr ? pr->mask_live : nullptr;
+    auto rows16 = [&](const fwa2_tensor3& t, int esize) {
+        return t.ptr == nullptr || (((uintptr_t)t.ptr & 15) == 0 && (t.stride_a * esize) % 16 == 0 && (t.stride_n * esize) % 16 == 0);
+    };
+    p.side_vec = pr->n % 8 == 0 && rows16(pr->bias, 2) && rows16(pr->mask, pr->mask_dtype == FWA2_F32 ? 4 : 2);
     p.lse = pr->lse; p.lse_sb = pr->lse_stride_bw; p.lse_sh = pr->lse_stride_h;
     p.bw = pr->bw; p.heads = pr->heads; p.n = pr->n; p.d = pr->head_dim;
     p.row_pad = ((pr->n + 63) / 64) * 64;
     if (backward) {
         unsigned char* ws = reinterpret_cast<unsigned char*>(pr->workspace);
-        const size_t rows = align256g((size_t)p.bw * p.heads * p.row_pad * sizeof(float));
+        const size_t rows = generic_rows_bytes(p.heads, p.bw, (size_t)p.row_pad);
         p.delta = reinterpret_cast<float*>(ws);
         p.dscale_rows = reinterpret_cast<float*>(ws + rows);
         p.part_dbias = reinterpret_cast<float*>(ws + 2 * rows);
