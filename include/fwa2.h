@@ -41,7 +41,7 @@ extern "C" {
 typedef enum fwa2_status {
     FWA2_OK = 0,
     FWA2_ERR_INVALID_ARGUMENT = 1, /* contract violation (the reference's AssertionError) */
-    FWA2_ERR_UNSUPPORTED = 2,      /* legal for the reference, not built here (e.g. head dim != 32) */
+    FWA2_ERR_UNSUPPORTED = 2,      /* legal for the reference, not built here (e.g. head dim % 8 != 0) */
     FWA2_ERR_HIP = 3,              /* a HIP runtime call failed */
     FWA2_ERR_NO_DEVICE = 4         /* no gfx950 device available for the launch */
 } fwa2_status;
@@ -86,7 +86,7 @@ typedef struct fwa2_problem {
     int32_t bw;              /* batch * windows-per-image */
     int32_t heads;
     int32_t n;               /* tokens per window (queries == keys) */
-    int32_t head_dim;
+    int32_t head_dim;        /* multiple of 8, at most 128; 32 runs on the tuned kernels */
     int32_t n_windows;       /* leading extent of mask; window of row b is b % n_windows; 1 if no mask */
 
     fwa2_tensor4 q, k, v;    /* inputs */
