@@ -7,7 +7,6 @@ Every buffer -- outputs, log-sum-exp, gradients and the backward workspace --
 is a torch tensor allocated here, so torch's allocator statistics stay honest
 and the C side allocates nothing.
 """
-import math
 
 import torch
 
@@ -145,7 +144,10 @@ class FlashWindowAttentionV2(torch.autograd.Function):
             logit_scale = logit_scale if logit_scale.stride(-1) == 1 else logit_scale.contiguous()
         else:
             scale_type = "scalar"
-            logit_scale = torch.tensor(1.0 / math.sqrt(q.shape[-1]), device=q.device)
+            # placeholder for the saved-tensor slot (the reference keeps 1/sqrt(d) there, fn.py:15-17); the
+            # kernels derive the default scale from head_dim, and filling a device scalar from the host
+            # would synchronise and break stream capture
+            logit_scale = torch.empty((), device=q.device)
 
         _check_inputs(q, k, v, logit_scale, bias, mask, scale_type)
         q, k, v = (_kernel_ready(x) for x in (q, k, v))
@@ -222,7 +224,10 @@ class FlashWindowAttentionV2QKVPacked(torch.autograd.Function):
             logit_scale = logit_scale.contiguous()
         else:
             scale_type = "scalar"
-            logit_scale = torch.tensor(1.0 / math.sqrt(q.shape[-1]), device=q.device)
+            # placeholder for the saved-tensor slot (the reference keeps 1/sqrt(d) there, fn.py:15-17); the
+            # kernels derive the default scale from head_dim, and filling a device scalar from the host
+            # would synchronise and break stream capture
+            logit_scale = torch.empty((), device=q.device)
         _check_inputs(q, k, v, logit_scale, bias, mask, scale_type)
         if bias is not None and bias.stride(-1) != 1:
             bias = bias.contiguous()
@@ -301,7 +306,10 @@ class FlashWindowAttentionV2Grid(torch.autograd.Function):
             logit_scale = logit_scale.contiguous()
         else:
             scale_type = "scalar"
-            logit_scale = torch.tensor(1.0 / math.sqrt(q.shape[-1]), device=q.device)
+            # placeholder for the saved-tensor slot (the reference keeps 1/sqrt(d) there, fn.py:15-17); the
+            # kernels derive the default scale from head_dim, and filling a device scalar from the host
+            # would synchronise and break stream capture
+            logit_scale = torch.empty((), device=q.device)
         b, heads, length, d = q.shape
         n, nw = wh * ww, (gh // wh) * (gw // ww)
         assert d <= 128, "FlashAttention only support head dimensions up to 128"
