@@ -175,7 +175,7 @@ __device__ __forceinline__ void unit_blocks(BwdLds<DT, NQB>& L, WaveRegs<DT, NQB
 // one (uniform per unit, so no block ever branches on the mask).  MODE 2: one launch walks both
 // kinds (windows of up to 128 tokens, where both copies fit the register file without scratch);
 // MODE 0 / 1: a launch for the units with an all-zero mask and one for the others.
-// BIG: windows of more than 256 tokens.  The N x N score matrix is cut into 256 x 256 super-tiles;
+// BIG: windows of more than 256 tokens.  The N x N score matrix is cut into 256 x 256 (or 192 x 192) super-tiles;
 // a workgroup then belongs to one (head, query chunk, key chunk), reads only those rows, keeps that
 // tile of dbias in registers and writes its share of dk / dv (already taken back through the
 // normalisation, which is linear) as fp32 partials that dkv_reduce_kernel sums over the query chunks.
@@ -640,7 +640,7 @@ hipError_t launch_backward_dq_resident(const BwdParams& p, int dtype, bool has_b
 
 struct BwdPlan {
     int waves, groups, npk, r, nqb_t, kt, dq_waves, dq_chunks, ds_parts, dq_max_groups;
-    int n_chunks;   // > 1: windows of more than 256 tokens, cut into 256 x 256 super-tiles
+    int n_chunks;   // > 1: windows of more than 256 tokens, cut into 256 x 256 or 192 x 192 super-tiles
     size_t off_dbias, off_dscale, off_bias_t, off_mask_t, off_delta, off_dk, off_dv, total;
     size_t smem;
 };
@@ -651,11 +651,16 @@ static BwdPlan make_plan(int heads, int n, int bw, bool has_bias, bool has_mask,
     pl.n_chunks = (n + 255) / 256;
     int wg_per_cu;
     if (pl.n_chunks > 1) {
-        // every workgroup is a full 256 x 256 super-tile kernel; npk / r are the padded totals
-        pl.nqb_t = 8;
+        // every workgroup is a full super-tile kernel of 256 x 256, or of 192 x 192 where that pads the
+        // window less (576 = 3 x 192 tokens: 9 exact tiles instead of 9 tiles covering 768 x 768);
+        // npk / r are the padded totals
+        const int c192 = (n + 191) / 192;
+        const int tile = 192 * c192 < 256 * pl.n_chunks ? 192 : 256;
+        if (tile == 192) pl.n_chunks = c192;
+        pl.nqb_t = tile / 32;
         pl.kt = 2;
-        pl.waves = 8;
-        pl.npk = pl.r = 256 * pl.n_chunks;
+        pl.waves = tile / 32;
+        pl.npk = pl.r = tile * pl.n_chunks;
         wg_per_cu = 1;
     } else {
         pl.nqb_t = nqb <= 2 ? 2 : (nqb <= 4 ? 4 : 8);
@@ -765,6 +770,7 @@ static hipError_t launch_nqb(const BwdParams& p, const BwdPlan& pl, hipStream_t 
         if (pl.kt == 1) return launch_main<DT, HAS_BIAS, MASK_DT, 8, 1, false, true>(p, pl, st, groups_out);
         return launch_main<DT, HAS_BIAS, MASK_DT, 8, 2, false, true>(p, pl, st, groups_out);
     }
+    if (pl.n_chunks > 1 && pl.nqb_t == 6) return launch_main<DT, HAS_BIAS, MASK_DT, 6, 2, true>(p, pl, st, groups_out);
     if (pl.n_chunks > 1) return launch_main<DT, HAS_BIAS, MASK_DT, 8, 2, true>(p, pl, st, groups_out);
     if (pl.nqb_t == 2) return launch_main<DT, HAS_BIAS, MASK_DT, 2, 1, false>(p, pl, st, groups_out);
     if (pl.nqb_t == 4) return launch_main<DT, HAS_BIAS, MASK_DT, 4, 1, false>(p, pl, st, groups_out);

@@ -344,10 +344,12 @@ def test_recompute_under_checkpoint():
     assert _rel(dev["q"].grad, ref["dq"]) <= 5e-2 and _rel(dev["bias"].grad, ref["dbias"]) <= 5e-2
 
 
-@pytest.mark.parametrize("n,dtype", [(576, torch.bfloat16), (1024, torch.bfloat16), (320, torch.float16)])
+@pytest.mark.parametrize("n,dtype", [(576, torch.bfloat16), (1024, torch.bfloat16), (320, torch.float16),
+                                     (784, torch.bfloat16), (530, torch.float16)])
 def test_large_windows(n, dtype):
-    """N = 576 and 1024 (windows 24 and 32 of the sweep) and a ragged 320: several LDS key chunks per
-    workgroup in the forward, 256 x 256 super-tiles with summed dk / dv partials in the backward."""
+    """N = 576 and 1024 (windows 24 and 32 of the sweep), 784 = 28 x 28 and the ragged 320 and 530: several
+    LDS key chunks per workgroup in the forward; in the backward super-tiles of 256 x 256 (320, 1024) or
+    192 x 192 (576 exactly, 530 and 784 with a partly empty last tile) with summed dk / dv partials."""
     inp = make_inputs(batch=1, n_windows=2, heads=2, n=n, dtype=dtype, seed=n, with_mask=False)
     _run_and_check(inp, dtype, tag=f"N{n}")
 
