@@ -15,8 +15,8 @@ hipError_t launch_mask_scan(const void* mask, int mask_dt, int64_t sw, int64_t s
                             uint8_t* live, hipStream_t st);
 hipError_t launch_backward(const BwdParams& p, int dtype, bool has_bias, int mask_dt, hipStream_t st);
 size_t backward_workspace_bytes(int heads, int n, int bw, bool has_bias, bool has_mask, int n_windows, int cus);
-bool generic_head_dim(int d);
-size_t generic_workspace_bytes(int heads, int n, int bw, bool has_bias);
+bool generic_problem(int d, int n, int nk);
+size_t generic_workspace_bytes(int heads, int n, int nk, int bw, bool has_bias);
 hipError_t launch_generic(const fwa2_problem* p, bool backward);
 int backward_supported(int n);
 hipError_t launch_cpb_bias_forward(const void* table, int dtype, int heads, int wh, int ww, void* bias, hipStream_t st);
@@ -86,15 +86,17 @@ int validate(const fwa2_problem* p, int backward) {
     } else if (p->scale_kind != FWA2_SCALE_DEFAULT) {
         return fail(FWA2_ERR_INVALID_ARGUMENT, "scale_kind %d unknown", p->scale_kind);
     }
-    if (p->bias.ptr && p->bias.stride_n < p->n)
-        return fail(FWA2_ERR_INVALID_ARGUMENT, "bias: row stride %lld < n", (long long)p->bias.stride_n);
+    if (p->n_keys < 0 || p->reserved0 != 0) return fail(FWA2_ERR_INVALID_ARGUMENT, "n_keys must not be negative, reserved0 must be 0");
+    const int nk = p->n_keys > 0 ? p->n_keys : p->n;
+    if (p->bias.ptr && p->bias.stride_n < nk)
+        return fail(FWA2_ERR_INVALID_ARGUMENT, "bias: row stride %lld < number of keys", (long long)p->bias.stride_n);
     if (p->mask.ptr) {
         if (p->mask_dtype != p->dtype && p->mask_dtype != FWA2_F32)
             return fail(FWA2_ERR_INVALID_ARGUMENT, "mask dtype must be the input dtype or fp32");
         if (p->n_windows <= 0 || p->bw % p->n_windows)
             return fail(FWA2_ERR_INVALID_ARGUMENT, "bw %d is not a multiple of n_windows %d", p->bw, p->n_windows);
-        if (p->mask.stride_n < p->n)
-            return fail(FWA2_ERR_INVALID_ARGUMENT, "mask: row stride %lld < n", (long long)p->mask.stride_n);
+        if (p->mask.stride_n < nk)
+            return fail(FWA2_ERR_INVALID_ARGUMENT, "mask: row stride %lld < number of keys", (long long)p->mask.stride_n);
     }
     if (p->grid_h != 0 || p->grid_w != 0 || p->win_h != 0 || p->win_w != 0 || p->shift_h != 0 || p->shift_w != 0) {
         if (p->grid_h <= 0 || p->grid_w <= 0 || p->win_h <= 0 || p->win_w <= 0 || p->grid_h % p->win_h || p->grid_w % p->win_w)
@@ -108,8 +110,8 @@ int validate(const fwa2_problem* p, int backward) {
         if (p->bw % nw) return fail(FWA2_ERR_INVALID_ARGUMENT, "window map: bw %d is not a multiple of %d windows per image", p->bw, nw);
         if (p->mask.ptr && p->n_windows != nw)
             return fail(FWA2_ERR_INVALID_ARGUMENT, "window map: mask has %d windows, the grid %d", p->n_windows, nw);
-        if (fwa2::generic_head_dim(p->head_dim))
-            return fail(FWA2_ERR_UNSUPPORTED, "window map: head_dim %d is not supported with a window map (32 only)", p->head_dim);
+        if (fwa2::generic_problem(p->head_dim, p->n, nk))
+            return fail(FWA2_ERR_UNSUPPORTED, "window map: needs head_dim 32 and as many keys as queries");
         if (p->win_w > 64 || p->n > fwa2::kMapMaxN)
             return fail(FWA2_ERR_UNSUPPORTED, "window map: windows of more than %d tokens (or wider than 64) are not supported",
                         fwa2::kMapMaxN);
@@ -167,8 +169,8 @@ int fwa2_validate(const fwa2_problem* p, int backward) {
 
 size_t fwa2_backward_workspace_bytes(const fwa2_problem* p) {
     if (p == nullptr) return 0;
-    if (fwa2::generic_head_dim(p->head_dim))
-        return fwa2::generic_workspace_bytes(p->heads, p->n, p->bw, p->bias.ptr != nullptr);
+    if (fwa2::generic_problem(p->head_dim, p->n, p->n_keys > 0 ? p->n_keys : p->n))
+        return fwa2::generic_workspace_bytes(p->heads, p->n, p->n_keys > 0 ? p->n_keys : p->n, p->bw, p->bias.ptr != nullptr);
     return fwa2::backward_workspace_bytes(p->heads, p->n, p->bw, p->bias.ptr != nullptr, p->mask.ptr != nullptr,
                                           p->n_windows, cu_count());
 }
@@ -221,7 +223,7 @@ int fwa2_forward(const fwa2_problem* p) {
     g_err[0] = 0;
     int rc = validate(p, 0);
     if (rc) return rc;
-    if (fwa2::generic_head_dim(p->head_dim)) {
+    if (fwa2::generic_problem(p->head_dim, p->n, p->n_keys > 0 ? p->n_keys : p->n)) {
         hipError_t eg = fwa2::launch_generic(p, false);
         if (eg != hipSuccess) return fail(FWA2_ERR_HIP, "forward launch: %s", hipGetErrorString(eg));
         return FWA2_OK;
@@ -252,7 +254,7 @@ int fwa2_backward(const fwa2_problem* p) {
     g_err[0] = 0;
     int rc = validate(p, 1);
     if (rc) return rc;
-    if (fwa2::generic_head_dim(p->head_dim)) {
+    if (fwa2::generic_problem(p->head_dim, p->n, p->n_keys > 0 ? p->n_keys : p->n)) {
         hipError_t eg = fwa2::launch_generic(p, true);
         if (eg != hipSuccess) return fail(FWA2_ERR_HIP, "backward launch: %s", hipGetErrorString(eg));
         return FWA2_OK;

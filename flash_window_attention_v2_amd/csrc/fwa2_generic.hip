@@ -52,7 +52,7 @@ struct GenParams {
     int side_vec;               // rows of bias and mask may be read with 16-byte loads and n % 8 == 0
     float* lse;
     int64_t lse_sb, lse_sh;
-    int bw, heads, n, d;
+    int bw, heads, n, nk, d;   // n queries, nk keys per unit
     float* delta;         // [BW * H, row_pad] rowsum(o * dO), written by DQ, read by DKV and DBIAS
     float* dscale_rows;   // [BW * H, row_pad] q^ . dq^ of every query row, written by DQ
     int row_pad;
@@ -86,9 +86,12 @@ __global__ void __launch_bounds__(256) generic_kernel(const GenParams p) {
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int l16 = lane & 15, g = lane >> 4;
-    const int N = p.n, d = p.d;
-    const int chunks = (N + 63) / 64;
-    const int kblocks = (N + 31) / 32;
+    const int d = p.d;
+    const int NO = OWNER_IS_KEY ? p.nk : p.n;    // owner rows of a unit
+    const int NX = OWNER_IS_KEY ? p.n : p.nk;    // other rows of a unit
+    const int NQ = p.n, NKEY = p.nk;
+    const int chunks = (NO + 63) / 64;
+    const int kblocks = (NX + 31) / 32;
 
     int idx = blockIdx.x, kb = 0, grp = 0, b0;
     if (MODE == G_DBIAS) {
@@ -102,7 +105,7 @@ __global__ void __launch_bounds__(256) generic_kernel(const GenParams p) {
     if (MODE == G_DBIAS || WITH_DB) { grp = idx; b0 = grp; } else { b0 = idx; }
 
     const int own = own0 + 16 * wave + l16;     // owner row of this lane's column
-    const bool own_ok = own < N;
+    const bool own_ok = own < NO;
 
     float scale2, scale_nat;
     if (p.scale_kind == FWA2_SCALE_TENSOR) {
@@ -175,7 +178,7 @@ __global__ void __launch_bounds__(256) generic_kernel(const GenParams p) {
             const int r = c / CH, c8 = (c % CH) * 8;
             const int row = o0 + r;
             V8 a = zero8<V8>(), bb = zero8<V8>();
-            if (row < N && c8 < d) {
+            if (row < NX && c8 < d) {
                 a = ld8<V8>(rowp(ta, b, row) + c8);
                 bb = ld8<V8>(rowp(tb, b, row) + c8);
             }
@@ -203,11 +206,11 @@ __global__ void __launch_bounds__(256) generic_kernel(const GenParams p) {
             float add[8];
 #pragma unroll
             for (int j = 0; j < 8; j++) add[j] = 0.f;
-            if (qi < N) {
+            if (qi < NQ) {
                 const E* bptr = reinterpret_cast<const E*>(p.bias) + h * p.bias_sh + (int64_t)qi * p.bias_sn + k0;
                 const int64_t mo = w * p.mask_sw + (int64_t)qi * p.mask_sn + k0;
                 if (p.side_vec) {
-                    if (k0 < N) {
+                    if (k0 < NKEY) {
                         if (p.bias) {
                             const V8 bv = ld8<V8>(bptr);
 #pragma unroll
@@ -227,7 +230,7 @@ __global__ void __launch_bounds__(256) generic_kernel(const GenParams p) {
                 } else {
 #pragma unroll
                     for (int j = 0; j < 8; j++) {
-                        if (k0 + j < N) {
+                        if (k0 + j < NKEY) {
                             if (p.bias) add[j] += (float)bptr[j];
                             if (mask_on)
                                 add[j] += p.mask_f32 ? reinterpret_cast<const float*>(p.mask)[mo + j]
@@ -241,7 +244,7 @@ __global__ void __launch_bounds__(256) generic_kernel(const GenParams p) {
         }
         if (MODE == G_DKV && tid < 32) {
             const int row = o0 + tid;
-            const bool ok = row < N;
+            const bool ok = row < NX;
             const int64_t ro = ((int64_t)b * p.heads + h) * p.row_pad + row;
             s_lse2[tid] = ok ? p.lse[b * p.lse_sb + h * p.lse_sh + row] * kLog2e : 0.f;
             s_delta[tid] = ok ? p.delta[ro] : 0.f;
@@ -273,7 +276,7 @@ __global__ void __launch_bounds__(256) generic_kernel(const GenParams p) {
         float add[8];
 #pragma unroll
         for (int j = 0; j < 8; j++) {
-            ok[j] = own_ok && o0 + 8 * g + j < N;
+            ok[j] = own_ok && o0 + 8 * g + j < NX;
             add[j] = 0.f;
         }
         if (OWNER_IS_KEY) {
@@ -362,11 +365,11 @@ __global__ void __launch_bounds__(256) generic_kernel(const GenParams p) {
             }
         }
         if (own_ok) {
-            float* dst = p.part_dbias + (((int64_t)grp * p.heads + h) * N + own) * N;
+            float* dst = p.part_dbias + (((int64_t)grp * p.heads + h) * NQ + own) * NKEY;
 #pragma unroll
             for (int j = 0; j < 8; j++) {
                 const int kj = 32 * kb + 8 * g + j;
-                if (kj < N) dst[kj] = db[j];
+                if (kj < NKEY) dst[kj] = db[j];
             }
         }
         return;
@@ -492,17 +495,17 @@ __global__ void __launch_bounds__(256) generic_kernel(const GenParams p) {
                     for (int i = 0; i < 4; i++) acc0[c][dt][i] = 0.f;
 #pragma unroll
             for (int t = 0; t < 8; t++)
-                if (32 * t < N) step(b, 32 * t, db[t]);
+                if (32 * t < NX) step(b, 32 * t, db[t]);
             finish_grad(b);
         }
         if (own_ok) {
-            float* dst = p.part_dbias + (((int64_t)grp * p.heads + h) * N + own) * N;
+            float* dst = p.part_dbias + (((int64_t)grp * p.heads + h) * NQ + own) * NKEY;
 #pragma unroll
             for (int t = 0; t < 8; t++)
 #pragma unroll
                 for (int j = 0; j < 8; j++) {
                     const int kj = 32 * t + 8 * g + j;
-                    if (kj < N) dst[kj] = db[t][j];
+                    if (kj < NKEY) dst[kj] = db[t][j];
                 }
         }
         return;
@@ -510,7 +513,7 @@ __global__ void __launch_bounds__(256) generic_kernel(const GenParams p) {
 
     const int b = b0;
     load_owner(b);
-    for (int o0 = 0; o0 < N; o0 += 32) step(b, o0, nullptr);
+    for (int o0 = 0; o0 < NX; o0 += 32) step(b, o0, nullptr);
 
     // ---- epilogue: this lane holds columns 32 c + 8 g + 4 dt + i of its owner row ----
     if (MODE == G_FWD) {
@@ -545,7 +548,7 @@ template <int DT>
 __global__ void __launch_bounds__(256) generic_dbias_reduce(const GenParams p) {
     typedef typename Elem<DT>::E E;
     __shared__ float part[8][32];
-    const int64_t per = (int64_t)p.heads * p.n * p.n;
+    const int64_t per = (int64_t)p.heads * p.n * p.nk;
     const int e = threadIdx.x & 31, sl = threadIdx.x >> 5;
     const int64_t i = (int64_t)blockIdx.x * 32 + e;
     float s = 0.f;
@@ -598,12 +601,12 @@ static size_t align256g(size_t x) { return (x + 255) & ~(size_t)255; }
 constexpr int kDbInDqMaxN = 256;   // windows up to this size sum dbias inside the dq pass
 
 // Unit groups of the pass that sums dbias: enough workgroups to fill the chip, bounded partial tiles.
-static int generic_groups(int heads, int n, int bw) {
-    const int64_t chunks = (n + 63) / 64, kblocks = (n + 31) / 32;
+static int generic_groups(int heads, int n, int nk, int bw) {
+    const int64_t chunks = (n + 63) / 64, kblocks = (nk + 31) / 32;
     int64_t groups;
-    if (n <= kDbInDqMaxN) {
+    if (nk <= kDbInDqMaxN) {
         groups = 1024 / (heads * chunks);
-        const int64_t cap = ((int64_t)64 << 20) / ((int64_t)heads * n * n * 4);
+        const int64_t cap = ((int64_t)64 << 20) / ((int64_t)heads * n * nk * 4);
         if (groups > cap) groups = cap;
     } else {
         groups = 2048 / (heads * chunks * kblocks);
@@ -614,7 +617,8 @@ static int generic_groups(int heads, int n, int bw) {
     return (int)groups;
 }
 
-bool generic_head_dim(int d) { return d != 32; }
+// The tuned kernels cover head_dim 32 with as many keys as queries; everything else runs here.
+bool generic_problem(int d, int n, int nk) { return d != 32 || nk != n; }
 
 // One [BW * H, row_pad] fp32 buffer (delta, dscale rows); never smaller than the dscale partial sums.
 static size_t generic_rows_bytes(int heads, int bw, size_t row_pad) {
@@ -623,35 +627,35 @@ static size_t generic_rows_bytes(int heads, int bw, size_t row_pad) {
     return align256g(rows * sizeof(float));
 }
 
-size_t generic_workspace_bytes(int heads, int n, int bw, bool has_bias) {
+size_t generic_workspace_bytes(int heads, int n, int nk, int bw, bool has_bias) {
     const size_t row_pad = (size_t)((n + 63) / 64) * 64;
     size_t total = 2 * generic_rows_bytes(heads, bw, row_pad);
-    if (has_bias) total += align256g((size_t)generic_groups(heads, n, bw) * heads * n * n * sizeof(float));
+    if (has_bias) total += align256g((size_t)generic_groups(heads, n, nk, bw) * heads * n * nk * sizeof(float));
     return total;
 }
 
 template <int DT, int D>
 static hipError_t launch_generic_d(const GenParams& p, bool backward, hipStream_t st) {
-    const int chunks = (p.n + 63) / 64, kblocks = (p.n + 31) / 32;
-    const dim3 grid((unsigned)((int64_t)p.bw * p.heads * chunks)), block(256);
+    const int chunks = (p.n + 63) / 64, kchunks = (p.nk + 63) / 64, kblocks = (p.nk + 31) / 32;
+    const dim3 grid((unsigned)((int64_t)p.bw * p.heads * chunks)), gridk((unsigned)((int64_t)p.bw * p.heads * kchunks)), block(256);
     if (!backward) {
         hipLaunchKernelGGL((generic_kernel<DT, D, G_FWD>), grid, block, 0, st, p);
         return hipGetLastError();
     }
-    const bool db_in_dq = p.bias && p.n <= kDbInDqMaxN;
+    const bool db_in_dq = p.bias && p.nk <= kDbInDqMaxN;
     if (db_in_dq) {
         const dim3 gq((unsigned)((int64_t)p.groups * p.heads * chunks));
         hipLaunchKernelGGL((generic_kernel<DT, D, G_DQ, true>), gq, block, 0, st, p);
     } else {
         hipLaunchKernelGGL((generic_kernel<DT, D, G_DQ>), grid, block, 0, st, p);
     }
-    hipLaunchKernelGGL((generic_kernel<DT, D, G_DKV>), grid, block, 0, st, p);
+    hipLaunchKernelGGL((generic_kernel<DT, D, G_DKV>), gridk, block, 0, st, p);
     if (p.bias) {
         if (!db_in_dq) {
             const dim3 gb((unsigned)((int64_t)p.groups * p.heads * chunks * kblocks));
             hipLaunchKernelGGL((generic_kernel<DT, D, G_DBIAS>), gb, block, 0, st, p);
         }
-        const int64_t per = (int64_t)p.heads * p.n * p.n;
+        const int64_t per = (int64_t)p.heads * p.n * p.nk;
         hipLaunchKernelGGL(generic_dbias_reduce<DT>, dim3((unsigned)((per + 31) / 32)), block, 0, st, p);
     }
     if (p.scale_kind == FWA2_SCALE_TENSOR && p.dscale) {
@@ -687,9 +691,10 @@ hipError_t launch_generic(const fwa2_problem* pr, bool backward) {
     auto rows16 = [&](const fwa2_tensor3& t, int esize) {
         return t.ptr == nullptr || (((uintptr_t)t.ptr & 15) == 0 && (t.stride_a * esize) % 16 == 0 && (t.stride_n * esize) % 16 == 0);
     };
-    p.side_vec = pr->n % 8 == 0 && rows16(pr->bias, 2) && rows16(pr->mask, pr->mask_dtype == FWA2_F32 ? 4 : 2);
+    p.side_vec = (pr->n_keys > 0 ? pr->n_keys : pr->n) % 8 == 0 && rows16(pr->bias, 2) && rows16(pr->mask, pr->mask_dtype == FWA2_F32 ? 4 : 2);
     p.lse = pr->lse; p.lse_sb = pr->lse_stride_bw; p.lse_sh = pr->lse_stride_h;
     p.bw = pr->bw; p.heads = pr->heads; p.n = pr->n; p.d = pr->head_dim;
+    p.nk = pr->n_keys > 0 ? pr->n_keys : pr->n;
     p.row_pad = ((pr->n + 63) / 64) * 64;
     if (backward) {
         unsigned char* ws = reinterpret_cast<unsigned char*>(pr->workspace);
@@ -697,7 +702,7 @@ hipError_t launch_generic(const fwa2_problem* pr, bool backward) {
         p.delta = reinterpret_cast<float*>(ws);
         p.dscale_rows = reinterpret_cast<float*>(ws + rows);
         p.part_dbias = reinterpret_cast<float*>(ws + 2 * rows);
-        p.groups = generic_groups(p.heads, p.n, p.bw);
+        p.groups = generic_groups(p.heads, p.n, p.nk, p.bw);
         p.dbias = pr->dbias;
         p.dscale = pr->dscale;
     }

@@ -93,6 +93,8 @@ def _describe(q, k, v, o, lse, logit_scale, bias, mask, mask_live, scale_type, w
     p.dtype = _DTYPES[q.dtype]
     p.scale_kind = _abi.SCALE_TENSOR if scale_type == "tensor" else _abi.SCALE_DEFAULT
     p.bw, p.heads, p.n, p.head_dim = bw, heads, n, d
+    if window_map is None and k.shape[2] != n:
+        p.n_keys = k.shape[2]
     p.n_windows = mask.shape[0] if mask is not None else 1
     _set_t4(p.q, q); _set_t4(p.k, k); _set_t4(p.v, v); _set_t4(p.o, o)
     if scale_type == "tensor":
@@ -114,8 +116,8 @@ def _describe(q, k, v, o, lse, logit_scale, bias, mask, mask_live, scale_type, w
 def _check_inputs(q, k, v, logit_scale, bias, mask, scale_type):
     """The reference launcher's assertions (attn_kernel_forward.py:263-292)."""
     bw, heads, n, d = q.shape
-    assert k.shape == (bw, heads, k.shape[2], d) and v.shape == k.shape, "q, k, v shapes do not match"
-    assert k.shape[2] == n, "this build requires as many keys as queries (every caller of the reference does)"
+    n_k = k.shape[2]      # may differ from n (attn_kernel_forward.py:263-264); no caller of the reference does
+    assert k.shape == (bw, heads, n_k, d) and v.shape == k.shape, "q, k, v shapes do not match"
     assert d <= 128, "FlashAttention only support head dimensions up to 128"
     assert q.dtype == k.dtype == v.dtype, "All tensors must have the same type"
     assert q.dtype in (torch.float16, torch.bfloat16), "Only support fp16 and bf16"
@@ -127,11 +129,12 @@ def _check_inputs(q, k, v, logit_scale, bias, mask, scale_type):
     if bias is not None:
         assert bias.dtype == q.dtype
         assert bias.is_cuda
-        assert bias.shape == (heads, n, n)
+        assert bias.shape == (heads, n, n_k)
     if mask is not None:
         assert mask.dtype in (q.dtype, torch.float32)
         assert mask.is_cuda
-        assert mask.dim() == 3 and mask.shape[1:] == (n, n) and bw % mask.shape[0] == 0, "mask must be [nW, N, N] with BW % nW == 0"
+        assert mask.dim() == 3 and mask.shape[1:] == (n, n_k) and bw % mask.shape[0] == 0, \
+            "mask must be [nW, N, N_k] with BW % nW == 0"
 
 
 class FlashWindowAttentionV2(torch.autograd.Function):
@@ -164,7 +167,8 @@ class FlashWindowAttentionV2(torch.autograd.Function):
         o = torch.empty_like(q)
         if not _rows_16b_aligned(o):
             o = torch.empty(q.shape, device=q.device, dtype=q.dtype)
-        mask_live = mask_window_flags(mask) if mask is not None else None
+        # the flag scan covers square masks; with other key counts the kernels go without the flags
+        mask_live = mask_window_flags(mask) if mask is not None and mask.shape[1] == mask.shape[2] else None
         p = _describe(q, k, v, o, lse, logit_scale, bias, mask, mask_live, scale_type)
         with _on_device(q.device) as stream:
             p.stream = stream

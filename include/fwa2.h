@@ -128,6 +128,15 @@ typedef struct fwa2_problem {
     int32_t grid_h, grid_w;
     int32_t win_h, win_w;
     int32_t shift_h, shift_w;
+
+    /*
+     * Keys (rows of k and v) per unit when they differ from the n queries, which the reference's kernels allow
+     * (attn_kernel_forward.py:263-264) although none of its callers does; 0 = n.  bias is then [H, n, n_keys],
+     * mask [nW, n, n_keys], lse and the q-side tensors keep n rows, dk / dv have n_keys rows.  Runs on the plain
+     * kernels that also serve head dimensions other than 32; not combined with a window map.
+     */
+    int32_t n_keys;
+    int32_t reserved0;       /* must be 0 */
 } fwa2_problem;
 
 /* Library / ABI identification.  Returns FWA2_ABI_VERSION. */

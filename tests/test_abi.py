@@ -76,6 +76,20 @@ def test_validate_accepts_and_rejects(lib):
     assert lib.fwa2_validate(p, 0) == _abi.ERR_INVALID_ARGUMENT and b"overlaps rows" in lib.fwa2_last_error()
 
     p = _good_problem()
+    p.n_keys = 96       # more keys than queries: legal, bias / mask rows must then hold 96 entries
+    assert lib.fwa2_validate(p, 0) == _abi.OK
+    p.bias = _abi.Tensor3(0x10000, 64 * 64, 64)
+    assert lib.fwa2_validate(p, 0) == _abi.ERR_INVALID_ARGUMENT and b"number of keys" in lib.fwa2_last_error()
+    p.bias = _abi.Tensor3(0x10000, 64 * 96, 96)
+    assert lib.fwa2_validate(p, 0) == _abi.OK
+    p.grid_h, p.grid_w, p.win_h, p.win_w = 16, 16, 8, 8     # a window map needs keys == queries
+    p.bw = 8
+    assert lib.fwa2_validate(p, 0) == _abi.ERR_UNSUPPORTED and b"window map" in lib.fwa2_last_error()
+    p = _good_problem()
+    p.reserved0 = 1
+    assert lib.fwa2_validate(p, 0) == _abi.ERR_INVALID_ARGUMENT
+
+    p = _good_problem()
     p.q = _abi.Tensor4(0x10002, 4096, 2048, 32)  # rows not 16-byte aligned
     assert lib.fwa2_validate(p, 0) == _abi.ERR_UNSUPPORTED
 

@@ -48,3 +48,40 @@ def test_head_dim_must_be_a_multiple_of_8():
     q = torch.randn(2, 2, 16, 20, device="cuda", dtype=torch.bfloat16)
     with pytest.raises(NotImplementedError, match="multiples of 8"):
         flash_win_attn_v2_func(q, q, q)
+
+
+@pytest.mark.parametrize("nq,nk,d", [(64, 96, 32), (100, 49, 32), (49, 128, 64), (300, 64, 32), (37, 290, 16)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_more_or_fewer_keys_than_queries(nq, nk, d, dtype):
+    """The reference's kernels take k / v with a row count of their own (attn_kernel_forward.py:263-264):
+    bias is [H, Nq, Nk], mask [nW, Nq, Nk], dk / dv follow k / v.  300 queries and 290 keys also cross the
+    bound up to which dbias is summed inside the dq pass."""
+    from oracle.classic_torch import classic_fwd_bwd
+    from tests.test_gpu_parity import TOL, _rel
+    from flash_window_attention_v2_amd import flash_win_attn_v2_func
+    bw, heads, nw = 6, 2, 3
+    g = torch.Generator().manual_seed(nq + nk)
+    rnd = lambda *s: torch.randn(*s, generator=g)
+    q, do = rnd(bw, heads, nq, d).to(dtype), rnd(bw, heads, nq, d).to(dtype)
+    k, v = rnd(bw, heads, nk, d).to(dtype), rnd(bw, heads, nk, d).to(dtype)
+    bias = (16 * torch.sigmoid(rnd(heads, nq, nk))).to(dtype)
+    scale = torch.full((heads, 1, 1), 2.3).to(dtype)
+    mask = torch.where(torch.rand(nw, nq, nk, generator=g) < 0.3, -100.0, 0.0)
+    mask[0] = 0
+    mask[:, :, 0] = 0                                   # every row keeps a key
+    mask = mask.to(dtype)
+    ref = classic_fwd_bwd(q, k, v, scale, bias, mask, do)
+
+    dq_, dk_, dv_, ds_, db_ = (t.cuda().requires_grad_() for t in (q, k, v, scale, bias))
+    o = flash_win_attn_v2_func(dq_, dk_, dv_, ds_, db_, mask.cuda())
+    assert o.shape == (bw, heads, nq, d)
+    o.backward(do.cuda())
+    tol_o, tol_g = TOL[dtype]
+    assert float((o.detach().float().cpu() - ref["o"]).abs().max()) <= tol_o
+    assert dk_.grad.shape == k.shape and dv_.grad.shape == v.shape and db_.grad.shape == bias.shape
+    for got, name in ((dq_, "dq"), (dk_, "dk"), (dv_, "dv"), (db_, "dbias")):
+        assert _rel(got.grad, ref[name]) <= tol_g, name
+    diff = (ds_.grad.float().cpu().flatten() - ref["dscale"].float().cpu().flatten()).abs()
+    bound = torch.maximum(ref["dscale"].float().cpu().flatten().abs().max().expand_as(diff),
+                          0.1 * ref["dscale_l1"].float().cpu().flatten())
+    assert bool((diff <= tol_g * bound).all())
