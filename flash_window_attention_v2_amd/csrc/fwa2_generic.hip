@@ -170,31 +170,28 @@ __global__ void __launch_bounds__(256) generic_kernel(const GenParams p) {
         }
     };
 
-    // ---- 32 other rows starting at o0 into LDS: normalised into t0, raw into t1 ----
-    auto stage = [&](int b, int o0) __attribute__((always_inline)) {
+    // ---- 32 other rows starting at o0: fetch() brings this thread's share into registers (issued a step
+    // ahead, so the loads fly during the matrix work), commit() normalises and stores it to LDS ----
+    constexpr int NCH = (32 * CH + 255) / 256;     // 16-byte chunks of each tile per thread
+    struct Staged {
+        V8 a[NCH], bb[NCH];
+        float add[8];          // DKV: (bias + mask) of one query against 8 owner keys
+        float lse2, delta;     // DKV: of other row tid (threads 0 .. 31)
+    };
+    auto fetch = [&](int b, int o0, Staged& st) __attribute__((always_inline)) {
         const T4& ta = OWNER_IS_KEY ? p.q : p.k;
         const T4& tb = OWNER_IS_KEY ? p.d_o : p.v;
-        for (int c = tid; c < 32 * CH; c += 256) {
+#pragma unroll
+        for (int u = 0; u < NCH; u++) {
+            const int c = tid + 256 * u;
             const int r = c / CH, c8 = (c % CH) * 8;
             const int row = o0 + r;
-            V8 a = zero8<V8>(), bb = zero8<V8>();
-            if (row < NX && c8 < d) {
-                a = ld8<V8>(rowp(ta, b, row) + c8);
-                bb = ld8<V8>(rowp(tb, b, row) + c8);
+            st.a[u] = zero8<V8>();
+            st.bb[u] = zero8<V8>();
+            if (c < 32 * CH && row < NX && c8 < d) {
+                st.a[u] = ld8<V8>(rowp(ta, b, row) + c8);
+                st.bb[u] = ld8<V8>(rowp(tb, b, row) + c8);
             }
-            float x[8];
-            unpack8(a, x);
-            float ss = 0.f;
-#pragma unroll
-            for (int j = 0; j < 8; j++) ss += x[j] * x[j];
-#pragma unroll
-            for (int off = CH / 2; off >= 1; off >>= 1) ss += __shfl_xor(ss, off);
-            const float inv = inv_norm(ss);
-            SV8 w;
-#pragma unroll
-            for (int j = 0; j < 8; j++) w[j] = (SE)(x[j] * inv);
-            st8<SV8>(t0 + r * S + c8, w);
-            st8<V8>(t1 + r * S + c8, bb);
         }
         if (MODE == G_DKV) {
             // (bias + mask) of the 32 staged queries against the 64 owner keys, read along the rows of the
@@ -203,7 +200,7 @@ __global__ void __launch_bounds__(256) generic_kernel(const GenParams p) {
             const int qi = o0 + r, k0 = own0 + c8;
             const int w = b % p.n_windows;
             const bool mask_on = p.mask && (!p.mask_live || p.mask_live[w] != 0);
-            float add[8];
+            float* add = st.add;
 #pragma unroll
             for (int j = 0; j < 8; j++) add[j] = 0.f;
             if (qi < NQ) {
@@ -239,15 +236,44 @@ __global__ void __launch_bounds__(256) generic_kernel(const GenParams p) {
                     }
                 }
             }
-#pragma unroll
-            for (int j = 0; j < 8; j++) s_add[r * AS + c8 + j] = add[j] * kLog2e;
+            st.lse2 = 0.f;
+            st.delta = 0.f;
+            if (tid < 32 && o0 + tid < NX) {
+                const int row = o0 + tid;
+                st.lse2 = p.lse[b * p.lse_sb + h * p.lse_sh + row] * kLog2e;
+                st.delta = p.delta[((int64_t)b * p.heads + h) * p.row_pad + row];
+            }
         }
-        if (MODE == G_DKV && tid < 32) {
-            const int row = o0 + tid;
-            const bool ok = row < NX;
-            const int64_t ro = ((int64_t)b * p.heads + h) * p.row_pad + row;
-            s_lse2[tid] = ok ? p.lse[b * p.lse_sb + h * p.lse_sh + row] * kLog2e : 0.f;
-            s_delta[tid] = ok ? p.delta[ro] : 0.f;
+    };
+    auto commit = [&](const Staged& st) __attribute__((always_inline)) {
+#pragma unroll
+        for (int u = 0; u < NCH; u++) {
+            const int c = tid + 256 * u;
+            if (c < 32 * CH) {       // whole aligned groups of CH lanes take part, so the shuffles stay inside
+                const int r = c / CH, c8 = (c % CH) * 8;
+                float x[8];
+                unpack8(st.a[u], x);
+                float ss = 0.f;
+#pragma unroll
+                for (int j = 0; j < 8; j++) ss += x[j] * x[j];
+#pragma unroll
+                for (int off = CH / 2; off >= 1; off >>= 1) ss += __shfl_xor(ss, off);
+                const float inv = inv_norm(ss);
+                SV8 w;
+#pragma unroll
+                for (int j = 0; j < 8; j++) w[j] = (SE)(x[j] * inv);
+                st8<SV8>(t0 + r * S + c8, w);
+                st8<V8>(t1 + r * S + c8, st.bb[u]);
+            }
+        }
+        if (MODE == G_DKV) {
+            const int r = tid >> 3, c8 = (tid & 7) * 8;
+#pragma unroll
+            for (int j = 0; j < 8; j++) s_add[r * AS + c8 + j] = st.add[j] * kLog2e;
+            if (tid < 32) {
+                s_lse2[tid] = st.lse2;
+                s_delta[tid] = st.delta;
+            }
         }
     };
 
@@ -349,11 +375,14 @@ __global__ void __launch_bounds__(256) generic_kernel(const GenParams p) {
         float db[8];
 #pragma unroll
         for (int j = 0; j < 8; j++) db[j] = 0.f;
+        Staged st;
+        if (b0 < p.bw) fetch(b0, 32 * kb, st);
         for (int b = b0; b < p.bw; b += p.groups) {
             load_owner(b);
             __syncthreads();
-            stage(b, 32 * kb);
+            commit(st);
             __syncthreads();
+            if (b + p.groups < p.bw) fetch(b + p.groups, 32 * kb, st);
             float z2[8], dpv[8];
             bool ok[8];
             tile(b, 32 * kb, z2, dpv, ok);
@@ -423,10 +452,13 @@ __global__ void __launch_bounds__(256) generic_kernel(const GenParams p) {
 
     float m_run = -INFINITY, l_run = 0.f;
     // one step of 32 other rows; dbr: this lane's 8 dbias sums of the step (WITH_DB) or nullptr
+    Staged st;
     auto step = [&](int b, int o0, float* dbr) __attribute__((always_inline)) {
+        if (o0 == 0) fetch(b, 0, st);      // first step of a unit; later ones were fetched a step ahead
         __syncthreads();
-        stage(b, o0);
+        commit(st);
         __syncthreads();
+        if (o0 + 32 < NX) fetch(b, o0 + 32, st);
         float z2[8], dpv[8];
         bool ok[8];
         tile(b, o0, z2, dpv, ok);
