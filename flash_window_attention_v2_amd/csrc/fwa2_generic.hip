@@ -4,7 +4,7 @@
 // (flash_win_attn_v2/kernels/attn_kernel_forward.py:267, 298); every configuration it benchmarks uses 32,
 // which the tuned kernels of this library cover.  The kernels here restore the rest of that contract with
 // one plain skeleton instead of five tuned ones: no register-resident bias, no persistent workgroups, no
-// asynchronous prefetch.
+// LDS DMA (the rows of the next step are fetched into registers while this step computes).
 //
 // One skeleton, four modes.  A workgroup of four wavefronts works on one (batch*window, head) unit and 64
 // "owner" rows, 16 per wavefront, one per lane column (lane % 16); it walks over the "other" rows in steps
