@@ -3,7 +3,7 @@
 backward, on one MI355X.
 
 A "step" is one forward + backward of the operator on the benchmark's
-synthetic batch (BASELINE config 3: B=64 images x 64 windows of N=256 tokens,
+synthetic batch (benchmark configuration 3: B=64 images x 64 windows of N=256 tokens,
 3 heads, head dim 32, bf16, shifted-window mask, bias = 16*sigmoid(N(0,1)),
 logit_scale = ln 10), inputs already resident in HBM.  One JSON line goes to
 stdout; progress goes to stderr.

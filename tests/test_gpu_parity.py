@@ -75,7 +75,7 @@ def _run_and_check(inp, dtype, backward=True, tag="", dscale_l1_frac=0.02):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_config1_shape(dtype):
-    """BASELINE config 1 (B2, 16 windows of 8x8, H4, d32, shift 4) on the GPU in low precision."""
+    """Benchmark configuration 1 (B2, 16 windows of 8x8, H4, d32, shift 4) on the GPU in low precision."""
     _run_and_check(make_inputs(**CONFIGS["C1"], dtype=dtype, seed=1), dtype, tag="C1")
 
 
@@ -383,7 +383,7 @@ def _classic_on_gpu_fp32(dev, chunk):
 
 @pytest.mark.parametrize("cfg", ["C2", "C3"])
 def test_full_benchmark_shapes(cfg):
-    """BASELINE configs 2 and 3 at full size (BW = 4096, H = 3, N = 64 / 256, bf16, shift mask)."""
+    """Benchmark configurations 2 and 3 at full size (BW = 4096, H = 3, N = 64 / 256, bf16, shift mask)."""
     dtype = torch.bfloat16
     inp = make_inputs(**CONFIGS[cfg], dtype=dtype, seed=0)
     dev = _to_dev(inp)
