@@ -99,6 +99,9 @@ class WindowAttention(nn.Module):
     #: let the kernels do the cyclic shift and the window partition / reverse of the enclosing block by
     #: address arithmetic (flash path only; used by SwinTransformerBlock when `grid_ready` says so)
     fused_grid = True
+    #: keep the position bias between calls that record no gradient (see relative_position_bias)
+    cache_bias = True
+    _bias_cache = None
 
     def __init__(self, dim, window_size, num_heads, is_flash=True, qkv_bias=True, attn_drop=0., proj_drop=0.,
                  pretrained_window_size=[0, 0]):
@@ -157,7 +160,23 @@ class WindowAttention(nn.Module):
         return seen[2]
 
     def relative_position_bias(self):
-        """[H, N, N] bias = 16 sigmoid(cpb_mlp(table)[index]) (swin_transformer_v2.py:283-287)."""
+        """[H, N, N] bias = 16 sigmoid(cpb_mlp(table)[index]) (swin_transformer_v2.py:283-287).
+
+        The bias depends on parameters and buffers only.  When no gradient is recorded (inference) it is kept
+        until one of them changes (their version counters, dtype or device), which saves the two small GEMMs
+        and the gather of every call; with gradients on it is rebuilt every call, as the reference does."""
+        if torch.is_grad_enabled() or not self.cache_bias:
+            self._bias_cache = None
+            return self._build_relative_position_bias()
+        srcs = (*self.cpb_mlp.parameters(), self.relative_coords_table, self.relative_position_index)
+        key = tuple((t._version, t.data_ptr(), t.dtype) for t in srcs) + (torch.is_autocast_enabled(),)
+        cached = self._bias_cache
+        if cached is None or cached[0] != key:
+            cached = (key, self._build_relative_position_bias())
+            self._bias_cache = cached
+        return cached[1]
+
+    def _build_relative_position_bias(self):
         n = self.window_size[0] * self.window_size[1]
         per_offset = self.cpb_mlp(self.relative_coords_table).view(-1, self.num_heads)
         if (self.is_flash and self.fused_bias and per_offset.is_cuda

@@ -350,3 +350,31 @@ def test_model_checkpointing_gpu():
         # backward) may reorder their sums, hence a tolerance rather than bit equality
         scale = float(a.grad.float().abs().max()) + 1e-6
         assert float((a.grad.float() - b.grad.float()).abs().max()) <= 2e-2 * scale, k
+
+
+def test_position_bias_cache_follows_the_parameters():
+    """Without gradients the bias is kept between calls; an optimiser step, load_state_dict or a dtype change
+    (all bump version counters or move storage) must invalidate it; with gradients on nothing is kept."""
+    torch.manual_seed(0)
+    att = swin.WindowAttention(32, (4, 4), 2, is_flash=False)
+    with torch.no_grad():
+        b1 = att.relative_position_bias()
+        assert att.relative_position_bias() is b1                       # served from the cache
+        att.cpb_mlp[2].weight.mul_(1.5)                                 # in-place update, as an optimiser does
+        b2 = att.relative_position_bias()
+        assert b2 is not b1 and not torch.equal(b1, b2)
+        fresh = att._build_relative_position_bias()
+        assert torch.equal(b2, fresh)
+        att.double()
+        assert att.relative_position_bias().dtype == torch.float64     # new storage, new dtype
+        att.float()
+        state = {k: v.clone() for k, v in att.state_dict().items()}
+        state["cpb_mlp.0.bias"] += 1.0
+        b3 = att.relative_position_bias()
+        att.load_state_dict(state)
+        assert not torch.equal(att.relative_position_bias(), b3)
+    b4 = att.relative_position_bias()
+    assert b4.requires_grad and att._bias_cache is None                 # training: rebuilt, nothing kept
+    att.cache_bias = False
+    with torch.no_grad():
+        assert att.relative_position_bias() is not att.relative_position_bias()
