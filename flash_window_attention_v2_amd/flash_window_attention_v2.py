@@ -63,11 +63,19 @@ def _kernel_ready(t):
     return t if _rows_16b_aligned(t) else t.contiguous()
 
 
+def tensor_version(t):
+    """The in-place modification counter of `t`, or None for a tensor created under torch.inference_mode,
+    which keeps none (asking for it raises)."""
+    return None if t.is_inference() else t._version
+
+
 def mask_window_flags(mask):
     """uint8[nW]: 1 where a window's mask has a non-zero entry (device tensor).
-    Cached on the mask tensor object and refreshed if the tensor is modified in place."""
+    Cached on the mask tensor object and refreshed if the tensor is modified in place (a mask created under
+    torch.inference_mode tracks no modifications: edit such a mask by making a new tensor)."""
     cached = getattr(mask, "_fwa2_live", None)
-    if cached is not None and cached[0] == mask._version and cached[1].device == mask.device:
+    version = tensor_version(mask)
+    if cached is not None and cached[0] == version and cached[1].device == mask.device:
         return cached[1]
     lib = _abi.load()
     live = torch.empty(mask.shape[0], dtype=torch.uint8, device=mask.device)
@@ -76,7 +84,7 @@ def mask_window_flags(mask):
                                 mask.stride(1), live.data_ptr(), stream)
     _abi.check(st, "fwa2_mask_scan")
     try:
-        mask._fwa2_live = (mask._version, live)
+        mask._fwa2_live = (version, live)
     except Exception:
         pass
     return live

@@ -19,7 +19,7 @@ from torch.utils.checkpoint import checkpoint
 
 from .win_attention_func import (flash_win_attn_v2_func, flash_win_attn_v2_grid_func, flash_win_attn_v2_qkvpacked_func,
                                  win_attention_torch)
-from .flash_window_attention_v2 import CpbBias, MAPPED_MAX_N
+from .flash_window_attention_v2 import CpbBias, MAPPED_MAX_N, tensor_version
 
 
 def _pair(x):
@@ -150,12 +150,13 @@ class WindowAttention(nn.Module):
         form the fused bias kernels compute on the fly; checked once per buffer version."""
         buf = self.relative_position_index
         seen = getattr(self, "_index_checked", None)
-        if seen is None or seen[0] != buf._version or seen[1] != buf.data_ptr():
+        version = tensor_version(buf)
+        if seen is None or seen[0] != version or seen[1] != buf.data_ptr():
             wh, ww = self.window_size
             rows = torch.arange(wh, device=buf.device).repeat_interleave(ww)
             cols = torch.arange(ww, device=buf.device).repeat(wh)
             want = (rows[:, None] - rows[None, :] + wh - 1) * (2 * ww - 1) + (cols[:, None] - cols[None, :] + ww - 1)
-            seen = (buf._version, buf.data_ptr(), bool(torch.equal(buf, want)))
+            seen = (version, buf.data_ptr(), bool(torch.equal(buf, want)))
             self._index_checked = seen
         return seen[2]
 
@@ -165,10 +166,11 @@ class WindowAttention(nn.Module):
         The bias depends on parameters and buffers only.  When no gradient is recorded (inference) it is kept
         until one of them changes (their version counters, dtype or device), which saves the two small GEMMs
         and the gather of every call; with gradients on it is rebuilt every call, as the reference does."""
-        if torch.is_grad_enabled() or not self.cache_bias:
+        srcs = (*self.cpb_mlp.parameters(), self.relative_coords_table, self.relative_position_index)
+        # parameters created under torch.inference_mode track no modifications: nothing is kept for them
+        if torch.is_grad_enabled() or not self.cache_bias or any(t.is_inference() for t in srcs):
             self._bias_cache = None
             return self._build_relative_position_bias()
-        srcs = (*self.cpb_mlp.parameters(), self.relative_coords_table, self.relative_position_index)
         key = tuple((t._version, t.data_ptr(), t.dtype) for t in srcs) + (torch.is_autocast_enabled(),)
         cached = self._bias_cache
         if cached is None or cached[0] != key:

@@ -378,3 +378,42 @@ def test_position_bias_cache_follows_the_parameters():
     att.cache_bias = False
     with torch.no_grad():
         assert att.relative_position_bias() is not att.relative_position_bias()
+
+
+def test_model_built_and_run_under_inference_mode_cpu():
+    """The reference's forward benchmark builds and runs the model inside torch.inference_mode
+    (benchmark/bench_model.py:14-19); tensors made there track no version counter, which the caches
+    around the operator must not ask for."""
+    @torch.inference_mode()
+    def run():
+        torch.manual_seed(0)
+        m = swin.SwinTransformerV2(img_size=64, patch_size=4, embed_dim=32, depths=[2, 2], num_heads=[2, 4],
+                                   window_size=4, num_classes=10, drop_path_rate=0.0, is_flash=False)
+        x = torch.randn(2, 3, 64, 64)
+        return m(x), m(x), m.layers[0].blocks[0].attn
+    y1, y2, attn = run()
+    assert y1.shape == (2, 10) and torch.equal(y1, y2)
+    assert attn._bias_cache is None         # inference-mode parameters: the bias is rebuilt every call
+
+
+@pytest.mark.gpu
+def test_model_built_and_run_under_inference_mode_gpu():
+    """The same on the GPU in fp16 through the fused kernels, against the classic path on the same weights."""
+    @torch.inference_mode()
+    def run():
+        torch.manual_seed(0)
+        kw = dict(img_size=64, patch_size=4, embed_dim=96, depths=[2, 2], num_heads=[3, 6], window_size=8, num_classes=10,
+                  drop_path_rate=0.0)
+        flash = swin.SwinTransformerV2(is_flash=True, **kw).to(dtype=torch.float16, device="cuda")
+        classic = swin.SwinTransformerV2(is_flash=False, **kw).to(device="cuda")
+        classic.load_state_dict({k: v.float() for k, v in flash.state_dict().items()})
+        for mod in flash.modules():
+            if isinstance(mod, torch.nn.LayerNorm):      # the post-norms start at zero weight in this model
+                mod.weight.fill_(1.0)
+        classic.load_state_dict({k: v.float() for k, v in flash.state_dict().items()})
+        x = torch.randn(4, 3, 64, 64, device="cuda", dtype=torch.float16)
+        flash(x)        # the convolution library may settle on another kernel after its first call
+        return flash(x), flash(x), classic(x.float())
+    y1, y2, ref = run()
+    assert torch.equal(y1, y2)
+    assert float((y1.float() - ref).abs().max() / ref.abs().max()) < 2e-2
