@@ -145,12 +145,14 @@ def test_ragged_window_sizes(n):
     _run_and_check(inp, dtype, backward=n > 1, tag=f"ragged N={n}", dscale_l1_frac=0.1)
 
 
-def test_random_inf_mask_and_random_scale():
+@pytest.mark.parametrize("n,d", [(64, 32), (144, 32), (256, 32), (576, 32), (64, 64), (144, 128)])
+def test_random_inf_mask_and_random_scale(n, d):
     """The reference's own check protocol: randn bias and logit_scale, ~half the mask entries -inf
-    (benchmark/check.py:23-33), here with every row keeping at least one open key."""
+    (benchmark/check.py:23-33), here with every row keeping at least one open key, at the window sizes of
+    its benchmark sweep (benchmark/config.py:9) and at two other head dimensions."""
     dtype = torch.float16
-    g = torch.Generator().manual_seed(3)
-    bw, nw, h, n, d = 8, 4, 3, 64, 32
+    g = torch.Generator().manual_seed(3 + n + d)
+    bw, nw, h = 8, 4, 3
     rnd = lambda *s: torch.randn(*s, generator=g)
     mask = torch.zeros(nw, n, n).masked_fill(rnd(nw, n, n) < 0, -float("inf"))
     mask[:, torch.arange(n), torch.arange(n)] = 0.0
