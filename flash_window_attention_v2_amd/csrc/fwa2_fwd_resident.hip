@@ -18,8 +18,9 @@
 // range, m is folded into the resident registers and the softmax needs no
 // running maximum at all: P~ = 2^acc, l = sum P~, o = (P~ V) / l,
 // lse = (m + log2 l) ln 2.  Otherwise (fp16 P would underflow, scales near the
-// clamp of 100, masks with positive entries or fully masked rows) the same
-// loop runs with the usual running maximum.
+// clamp of 100, masks with positive entries or fully masked rows) a first
+// pass of score products alone finds the exact row maximum, and the same loop
+// then runs against it.
 //
 // Per unit: K and V rows of the NEXT unit are fetched straight into an LDS
 // landing area (global_load_lds, no registers held) before the tiles of the
@@ -290,8 +291,7 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
         for (int dt = 0; dt < 2; dt++)
 #pragma unroll
             for (int i = 0; i < 4; i++) oacc[dt][i] = 0.f;
-        float l_run = 0.f;     // online path: this lane's share of the running row sum
-        float m_run = 0.f;     // online path: running maximum relative to m_fixed
+        float m_run = 0.f;     // exact-maximum path: row maximum relative to m_fixed
 
         // scores of keys 32 kp .. 32 kp + 31: MFMA tile A holds keys 8r/4 + r%4 in its rows r, tile B
         // the keys 4 further on, so that this lane's 8 values are keys 8g .. 8g+7 of the group
@@ -340,39 +340,39 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
                 }
             }
         } else {
-            m_run = -INFINITY;
+            // fp16 (P would underflow against a mere bound) or a very large scale: the exact row maximum
+            // first, from a pass of score products alone; the matrix pipe has the room, and the second pass
+            // then needs no running maximum, no rescaling of o and no VALU row sum
+            float bm = -INFINITY;
 #pragma unroll
             for (int kp = 0; kp < NT / 2; kp++) {
                 if (32 * kp < N) {
                     f32x4 s0, s1;
                     scores(kp, s0, s1);
-                    float bm = fmaxf(fmaxf(s0[0], s0[1]), fmaxf(s0[2], s0[3]));
+                    bm = fmaxf(bm, fmaxf(fmaxf(s0[0], s0[1]), fmaxf(s0[2], s0[3])));
                     bm = fmaxf(bm, fmaxf(fmaxf(s1[0], s1[1]), fmaxf(s1[2], s1[3])));
-                    bm = col_max(bm);
-                    const float m_new = fmaxf(m_run, bm);
-                    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-                    const float alpha = fast_exp2(m_run - m_use);
-                    m_run = m_new;
-                    float ps = 0.f;
+                }
+            }
+            m_run = col_max(bm);
+            const float m_use = (m_run == -INFINITY) ? 0.f : m_run;
+#pragma unroll
+            for (int kp = 0; kp < NT / 2; kp++) {
+                if (32 * kp < N) {
+                    f32x4 s0, s1;
+                    scores(kp, s0, s1);
 #pragma unroll
                     for (int i = 0; i < 4; i++) {
                         s0[i] = fast_exp2(s0[i] - m_use);
                         s1[i] = fast_exp2(s1[i] - m_use);
-                        ps += s0[i] + s1[i];
                     }
-                    l_run = l_run * alpha + ps;
-#pragma unroll
-                    for (int dt = 0; dt < 2; dt++)
-#pragma unroll
-                        for (int i = 0; i < 4; i++) oacc[dt][i] *= alpha;
-                    pv(kp, s0, s1, false);
+                    pv(kp, s0, s1, true);
                 }
             }
         }
 
         if (more) stage(cur ^ 1);     // before the stores below, so the wait covers only the fetch
         // ---- normalise, write o (input dtype) and lse (natural log, fp32) ----
-        const float l_tot = fast ? lacc[0] : col_add(l_run);
+        const float l_tot = lacc[0];
         const float inv_l = l_tot > 0.f ? 1.0f / l_tot : 0.f;
         int ln2 = lane;
         asm volatile("" : "+v"(ln2));
