@@ -68,6 +68,21 @@ class Mlp(nn.Module):
         return self.drop(self.fc2(self.drop(self.act(self.fc1(x)))))
 
 
+def trunc_normal_(tensor, mean=0., std=1., a=-2., b=2.):
+    """Truncated-normal initialiser under the reference's name (swin_transformer_v2.py:88-113)."""
+    return nn.init.trunc_normal_(tensor, mean=mean, std=std, a=a, b=b)
+
+
+def drop_path(input, drop_prob=0.0, training=False):
+    """Stochastic depth as a function (swin_transformer_v2.py:116-139): whole samples of a residual branch
+    are dropped with probability `drop_prob` while training, the survivors scaled by 1 / (1 - drop_prob)."""
+    if drop_prob == 0. or not training:
+        return input
+    keep = 1.0 - drop_prob
+    gate = input.new_empty((input.shape[0],) + (1,) * (input.dim() - 1)).bernoulli_(keep)
+    return input * gate / keep
+
+
 class DropPath(nn.Module):
     """Stochastic depth: drops whole samples of a residual branch while training."""
 
@@ -76,11 +91,7 @@ class DropPath(nn.Module):
         self.drop_prob = drop_prob
 
     def forward(self, x):
-        if self.drop_prob == 0. or not self.training:
-            return x
-        keep = 1.0 - self.drop_prob
-        gate = x.new_empty((x.shape[0],) + (1,) * (x.dim() - 1)).bernoulli_(keep)
-        return x * gate / keep
+        return drop_path(x, self.drop_prob, self.training)
 
     def extra_repr(self):
         return f"p={self.drop_prob}"
@@ -208,6 +219,12 @@ class WindowAttention(nn.Module):
             out = out.transpose(1, 2).reshape(b_, n, c)
         return self.proj_drop(self.proj(out))
 
+    def flops(self, N):
+        """Multiply-accumulates of one window of N tokens, by the reference's count
+        (swin_transformer_v2.py:304-315): qkv projection, q k^T, attn v, output projection."""
+        head_dim = self.dim // self.num_heads
+        return (N * self.dim * 3 * self.dim + 2 * self.num_heads * N * N * head_dim + N * self.dim * self.dim)
+
     def grid_ready(self, x):
         """True when `forward_grid` can take `x`: the fused path on the GPU in half precision, and a window the
         library addresses through a window map."""
@@ -289,6 +306,13 @@ class SwinTransformerBlock(nn.Module):
         x = shortcut + self.drop_path(self.norm1(x.reshape(b, h * w, c)))
         return x + self.drop_path(self.norm2(self.mlp(x)))
 
+    def flops(self):
+        """The reference's count (swin_transformer_v2.py:453-465): two norms, the windows' attention, the MLP."""
+        h, w = self.input_resolution
+        n_windows = h * w / self.window_size / self.window_size
+        return (2 * self.dim * h * w + n_windows * self.attn.flops(self.window_size * self.window_size)
+                + 2 * h * w * self.dim * self.dim * self.mlp_ratio)
+
     def extra_repr(self):
         return (f"dim={self.dim}, input_resolution={self.input_resolution}, num_heads={self.num_heads}, "
                 f"window_size={self.window_size}, shift_size={self.shift_size}, mlp_ratio={self.mlp_ratio}")
@@ -313,6 +337,11 @@ class PatchMerging(nn.Module):
         # channel order (row parity, column parity) = (0,0), (1,0), (0,1), (1,1)
         x = x.permute(0, 1, 3, 4, 2, 5).reshape(b, (h // 2) * (w // 2), 4 * c)
         return self.norm(self.reduction(x))
+
+    def flops(self):
+        """The reference's count (swin_transformer_v2.py:510-514): the 4C -> 2C reduction and the norm."""
+        h, w = self.input_resolution
+        return (h // 2) * (w // 2) * 4 * self.dim * 2 * self.dim + h * w * self.dim // 2
 
 
 class BasicLayer(nn.Module):
@@ -342,6 +371,10 @@ class BasicLayer(nn.Module):
             x = checkpoint(blk, x, use_reentrant=False) if self.use_checkpoint else blk(x)
         return self.downsample(x) if self.downsample is not None else x
 
+    def flops(self):
+        total = sum(blk.flops() for blk in self.blocks)
+        return total + (self.downsample.flops() if self.downsample is not None else 0)
+
     def _init_respostnorm(self):
         """Residual post-norm starts as the identity: both LayerNorms of every block at zero."""
         for blk in self.blocks:
@@ -369,6 +402,12 @@ class PatchEmbed(nn.Module):
             f"Input image size ({x.shape[2]}*{x.shape[3]}) doesn't match model ({self.img_size[0]}*{self.img_size[1]})."
         x = self.proj(x).flatten(2).transpose(1, 2)
         return self.norm(x) if self.norm is not None else x
+
+    def flops(self):
+        """The reference's count (swin_transformer_v2.py:660-665): the patch projection and its norm."""
+        ho, wo = self.patches_resolution
+        total = ho * wo * self.embed_dim * self.in_chans * (self.patch_size[0] * self.patch_size[1])
+        return total + (ho * wo * self.embed_dim if self.norm is not None else 0)
 
 
 class SwinTransformerV2(nn.Module):
@@ -447,3 +486,9 @@ class SwinTransformerV2(nn.Module):
 
     def forward(self, x):
         return self.head(self.forward_features(x))
+
+    def flops(self):
+        """The reference's count (swin_transformer_v2.py:816-823): embedding, stages, final norm, head."""
+        total = self.patch_embed.flops() + sum(layer.flops() for layer in self.layers)
+        total += self.num_features * self.patches_resolution[0] * self.patches_resolution[1] // (2 ** self.num_layers)
+        return total + self.num_features * self.num_classes

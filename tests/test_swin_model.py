@@ -417,3 +417,27 @@ def test_model_built_and_run_under_inference_mode_gpu():
     y1, y2, ref = run()
     assert torch.equal(y1, y2)
     assert float((y1.float() - ref).abs().max() / ref.abs().max()) < 2e-2
+
+
+def test_flops_accounting_known_answers():
+    """`flops()` by the reference's convention (swin_transformer_v2.py:304-315, 453-465, 510-514, 660-665,
+    816-823) against the figures published for SwinV2-T at 256 x 256: 5.9 G with window 8, 6.6 G with
+    window 16; and against the closed form of one attention module."""
+    m8 = swin.SwinTransformerV2(is_flash=False, window_size=8)
+    m16 = swin.SwinTransformerV2(is_flash=False, window_size=16)
+    assert round(m8.flops() / 1e9, 1) == 5.9
+    assert round(m16.flops() / 1e9, 1) == 6.6
+    att = swin.WindowAttention(96, (8, 8), 3, is_flash=False)
+    assert att.flops(64) == 64 * 96 * 288 + 2 * 3 * 64 * 64 * 32 + 64 * 96 * 96
+
+
+def test_module_level_helpers_of_the_reference():
+    x = torch.ones(64, 3)
+    assert swin.drop_path(x, 0.5, training=False) is x and swin.drop_path(x, 0.0, training=True) is x
+    torch.manual_seed(0)
+    y = swin.drop_path(x, 0.5, training=True)
+    rows = y[:, 0]
+    assert set(rows.tolist()) <= {0.0, 2.0} and 0 < int((rows == 0).sum()) < 64     # dropped or scaled by 1 / keep
+    assert torch.equal(y[:, 0], y[:, 1])                                                # whole samples
+    w = swin.trunc_normal_(torch.empty(1000), std=0.02)
+    assert float(w.abs().max()) <= 2.0 and 0.015 < float(w.std()) < 0.025
