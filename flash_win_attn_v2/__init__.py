@@ -9,9 +9,9 @@ from flash_window_attention_v2_amd import (FlashWindowAttentionV2, FlashWindowAt
                                            flash_win_attn_v2_func, flash_win_attn_v2_grid_func,
                                            flash_win_attn_v2_qkvpacked_func, win_attention_torch,
                                            win_attention_torch_compile)
-from flash_window_attention_v2_amd import flash_window_attention_v2, swin_transformer_v2, win_attention_func
+from flash_window_attention_v2_amd import flash_window_attention_v2, kernels, swin_transformer_v2, win_attention_func
 
-for _name in ("flash_window_attention_v2", "swin_transformer_v2", "win_attention_func"):
+for _name in ("flash_window_attention_v2", "kernels", "swin_transformer_v2", "win_attention_func"):
     sys.modules[__name__ + "." + _name] = getattr(_impl, _name)
 
 __all__ = _impl.__all__
