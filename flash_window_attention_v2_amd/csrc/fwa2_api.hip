@@ -110,8 +110,8 @@ int validate(const fwa2_problem* p, int backward) {
         if (p->bw % nw) return fail(FWA2_ERR_INVALID_ARGUMENT, "window map: bw %d is not a multiple of %d windows per image", p->bw, nw);
         if (p->mask.ptr && p->n_windows != nw)
             return fail(FWA2_ERR_INVALID_ARGUMENT, "window map: mask has %d windows, the grid %d", p->n_windows, nw);
-        if (fwa2::generic_problem(p->head_dim, p->n, nk))
-            return fail(FWA2_ERR_UNSUPPORTED, "window map: needs head_dim 32 and as many keys as queries");
+        if (nk != p->n)
+            return fail(FWA2_ERR_UNSUPPORTED, "window map: needs as many keys as queries");
         if (p->win_w > 64 || p->n > fwa2::kMapMaxN)
             return fail(FWA2_ERR_UNSUPPORTED, "window map: windows of more than %d tokens (or wider than 64) are not supported",
                         fwa2::kMapMaxN);

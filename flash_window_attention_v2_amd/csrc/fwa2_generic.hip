@@ -39,6 +39,7 @@ enum { G_FWD = 0, G_DQ = 1, G_DKV = 2, G_DBIAS = 3 };
 
 struct GenParams {
     T4 q, k, v, o, d_o, dq, dk, dv;
+    WinMap map;           // nw == 0: off
     const void* logit_scale;
     int scale_kind;
     float default_scale;
@@ -116,8 +117,11 @@ __global__ void __launch_bounds__(256) generic_kernel(const GenParams p) {
     }
     scale2 = scale_nat * kLog2e;
 
+    // row `row` of unit b; with a window map the unit's rows lie scattered over the token grid
+    const bool mapped = p.map.nw > 0;
     auto rowp = [&](const T4& t, int b, int row) -> const E* {
-        return reinterpret_cast<const E*>(t.ptr) + b * t.sb + h * t.sh + (int64_t)row * t.sn;
+        const int64_t off = mapped ? row_off<true>(t, p.map, b, h, row) : row_off<false>(t, p.map, b, h, row);
+        return reinterpret_cast<const E*>(t.ptr) + off;
     };
 
     // ---- owner rows: B operands of the score products, one row per lane column ----
@@ -428,8 +432,8 @@ __global__ void __launch_bounds__(256) generic_kernel(const GenParams p) {
             }
         proj = col_add(proj);
         if (own_ok) {
-            E* drow = reinterpret_cast<E*>(const_cast<void*>(td.ptr)) + b * td.sb + h * td.sh + (int64_t)own * td.sn;
-            E* vrow = reinterpret_cast<E*>(const_cast<void*>(p.dv.ptr)) + b * p.dv.sb + h * p.dv.sh + (int64_t)own * p.dv.sn;
+            E* drow = const_cast<E*>(rowp(td, b, own));
+            E* vrow = const_cast<E*>(rowp(p.dv, b, own));
 #pragma unroll
             for (int c = 0; c < KS; c++)
 #pragma unroll
@@ -552,7 +556,7 @@ __global__ void __launch_bounds__(256) generic_kernel(const GenParams p) {
         const float l_tot = col_add(l_run);
         const float inv_l = l_tot > 0.f ? 1.0f / l_tot : 0.f;
         if (own_ok) {
-            E* orow = reinterpret_cast<E*>(const_cast<void*>(p.o.ptr)) + b * p.o.sb + h * p.o.sh + (int64_t)own * p.o.sn;
+            E* orow = const_cast<E*>(rowp(p.o, b, own));
 #pragma unroll
             for (int c = 0; c < KS; c++)
 #pragma unroll
@@ -712,6 +716,14 @@ hipError_t launch_generic(const fwa2_problem* pr, bool backward) {
     auto t4 = [](const fwa2_tensor4& t) { return T4{t.ptr, t.stride_bw, t.stride_h, t.stride_n}; };
     p.q = t4(pr->q); p.k = t4(pr->k); p.v = t4(pr->v); p.o = t4(pr->o);
     p.d_o = t4(pr->d_o); p.dq = t4(pr->dq); p.dk = t4(pr->dk); p.dv = t4(pr->dv);
+    if (pr->grid_h > 0) {
+        p.map.nwx = pr->grid_w / pr->win_w;
+        p.map.nw = (pr->grid_h / pr->win_h) * p.map.nwx;
+        p.map.gh = pr->grid_h; p.map.gw = pr->grid_w;
+        p.map.wh = pr->win_h; p.map.ww = pr->win_w;
+        p.map.sh = pr->shift_h; p.map.sw = pr->shift_w;
+        p.map.inv_ww = 65536 / pr->win_w + 1;
+    }
     p.logit_scale = pr->logit_scale;
     p.scale_kind = pr->scale_kind;
     p.default_scale = 1.0f / sqrtf((float)pr->head_dim);

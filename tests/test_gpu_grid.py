@@ -88,6 +88,24 @@ def test_grid_matches_partitioned_call(case, dtype):
     assert torch.equal(scale_a.grad, scale_b.grad)
 
 
+@pytest.mark.parametrize("d", [16, 64, 128])
+@pytest.mark.parametrize("case", [CASES[0], CASES[2], CASES[7]], ids=["w8x8", "w4x8", "w16x16"])
+def test_grid_with_other_head_dimensions(case, d):
+    """The window map on the plain kernels that serve head dimensions other than 32."""
+    from flash_window_attention_v2_amd import flash_win_attn_v2_grid_func, flash_win_attn_v2_qkvpacked_func
+    batch, grid, window, shift, heads, with_mask = case
+    qkv, scale, bias, mask, dout = _inputs(batch, grid, window, heads, d, torch.bfloat16, 17, with_mask)
+    a = qkv.clone().requires_grad_(True)
+    scale_a, bias_a = scale.clone().requires_grad_(True), bias.clone().requires_grad_(True)
+    flash_win_attn_v2_grid_func(a, grid, window, shift, scale_a, bias_a, mask).backward(dout)
+    b = qkv.clone().requires_grad_(True)
+    scale_b, bias_b = scale.clone().requires_grad_(True), bias.clone().requires_grad_(True)
+    o_w = flash_win_attn_v2_qkvpacked_func(_partition(b, grid, window, shift), scale_b, bias_b, mask)
+    _reverse(o_w, grid, window, shift).backward(dout)
+    assert torch.equal(a.grad, b.grad)
+    assert torch.equal(bias_a.grad, bias_b.grad) and torch.equal(scale_a.grad, scale_b.grad)
+
+
 def test_grid_rejects_windows_longer_than_256_tokens():
     """Windows of more than 256 tokens run on the streaming kernels, which take no map: the library must
     say so instead of computing on wrong addresses."""
