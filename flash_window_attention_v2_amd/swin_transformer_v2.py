@@ -232,7 +232,7 @@ class WindowAttention(nn.Module):
             return False
         if x.dtype not in (torch.float16, torch.bfloat16) and not torch.is_autocast_enabled():
             return False
-        return self.window_size[0] * self.window_size[1] <= MAPPED_MAX_N
+        return self.window_size[0] * self.window_size[1] <= MAPPED_MAX_N and self.window_size[1] <= 64
 
     def forward_grid(self, x, grid, shift, mask=None):
         """The attention of every (shifted) window of the token grid x [B, gh * gw, C], result in the same
