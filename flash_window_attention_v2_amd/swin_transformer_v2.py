@@ -206,18 +206,33 @@ class WindowAttention(nn.Module):
             bias = torch.cat((self.q_bias, torch.zeros_like(self.v_bias, requires_grad=False), self.v_bias))
         qkv = F.linear(x, self.qkv.weight, bias).reshape(b_, n, 3, self.num_heads, -1)
         rel_bias = self.relative_position_bias()
+        scale = self.logit_scale
+        if self.is_flash:
+            scale, rel_bias = self._operator_dtype(qkv, scale, rel_bias)
         if self.is_flash and self.packed_qkv:
             # the kernels read q, k, v out of the GEMM output and write [B_, N, H, d]: no copies either
             # side, and one packed gradient instead of three that autograd would have to re-pack
-            out = flash_win_attn_v2_qkvpacked_func(qkv, self.logit_scale, rel_bias, mask).reshape(b_, n, c)
+            out = flash_win_attn_v2_qkvpacked_func(qkv, scale, rel_bias, mask).reshape(b_, n, c)
         else:
             q, k, v = qkv.permute(2, 0, 3, 1, 4).unbind(0)      # strided views, unit inner stride
             if self.is_flash:
-                out = flash_win_attn_v2_func(q, k, v, self.logit_scale, rel_bias, mask)
+                out = flash_win_attn_v2_func(q, k, v, scale, rel_bias, mask)
             else:
-                out = win_attention_torch(q, k, v, self.logit_scale, rel_bias, mask)
+                out = win_attention_torch(q, k, v, scale, rel_bias, mask)
             out = out.transpose(1, 2).reshape(b_, n, c)
         return self.proj_drop(self.proj(out))
+
+    @staticmethod
+    def _operator_dtype(qkv, scale, rel_bias):
+        """Under autocast the projection comes out in half precision while the parameters stay fp32; the
+        fused operator wants its scale and bias in the dtype of q (attn_kernel_forward.py:274, 282), so they
+        are cast on the way in (autograd casts the gradients back).  A module cast as a whole, as the
+        reference's benchmarks do, passes through untouched."""
+        if scale.dtype != qkv.dtype:
+            scale = scale.to(qkv.dtype)
+        if rel_bias.dtype != qkv.dtype:
+            rel_bias = rel_bias.to(qkv.dtype)
+        return scale, rel_bias
 
     def flops(self, N):
         """Multiply-accumulates of one window of N tokens, by the reference's count
@@ -245,7 +260,8 @@ class WindowAttention(nn.Module):
             bias = torch.cat((self.q_bias, torch.zeros_like(self.v_bias, requires_grad=False), self.v_bias))
         qkv = F.linear(x, self.qkv.weight, bias).reshape(b, length, 3, self.num_heads, -1)
         rel_bias = self.relative_position_bias()
-        out = flash_win_attn_v2_grid_func(qkv, grid, self.window_size, shift, self.logit_scale, rel_bias, mask)
+        scale, rel_bias = self._operator_dtype(qkv, self.logit_scale, rel_bias)
+        out = flash_win_attn_v2_grid_func(qkv, grid, self.window_size, shift, scale, rel_bias, mask)
         return self.proj_drop(self.proj(out.reshape(b, length, c)))
 
     def extra_repr(self):

@@ -469,3 +469,34 @@ def test_model_with_head_dimension_64_gpu():
     rel = lambda a, b: float((a.float() - b).abs().max() / b.abs().max())
     assert rel(yf, yc) < 3e-2
     assert rel(xf.grad, xc.grad) < 6e-2
+
+
+@pytest.mark.gpu
+def test_fp32_model_under_autocast_gpu():
+    """An fp32 model under torch.autocast(bfloat16): q, k, v arrive in bf16 while logit_scale stays an fp32
+    parameter, which the reference's kernels reject (attn_kernel_forward.py:274); here the module casts on the
+    way in.  Loss and gradients against the classic operator on the same weights without autocast."""
+    torch.manual_seed(0)
+    kw = dict(img_size=64, patch_size=4, embed_dim=96, depths=[2, 2], num_heads=[3, 6], window_size=8, num_classes=10,
+              drop_path_rate=0.0)
+    flash = swin.SwinTransformerV2(is_flash=True, **kw).cuda()
+    with torch.no_grad():
+        for mod in flash.modules():
+            if isinstance(mod, torch.nn.LayerNorm):
+                mod.weight.fill_(1.0)
+    classic = swin.SwinTransformerV2(is_flash=False, **kw).cuda()
+    classic.load_state_dict(flash.state_dict())
+    x = torch.randn(4, 3, 64, 64, device="cuda")
+    g = torch.randn(4, 10, device="cuda")
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        yf = flash(x)
+    yf.float().backward(g)
+    yc = classic(x)
+    yc.backward(g)
+    rel = lambda a, b: float((a.float() - b).abs().max() / b.abs().max())
+    assert rel(yf, yc) < 3e-2
+    for name in ("layers.0.blocks.1.attn.logit_scale", "layers.0.blocks.1.attn.cpb_mlp.2.weight",
+                 "layers.0.blocks.0.attn.qkv.weight", "patch_embed.proj.weight"):
+        pf, pc = dict(flash.named_parameters())[name].grad, dict(classic.named_parameters())[name].grad
+        # dlogit_scale is a signed sum that nearly cancels (and every GEMM around it ran in bf16 here)
+        assert pf is not None and pf.dtype == torch.float32 and rel(pf, pc) < (0.25 if "logit_scale" in name else 8e-2), name
