@@ -30,6 +30,12 @@
 // and are fetched one block ahead of their use.
 #include "fwa2_common.hpp"
 
+// FWA2_HALF splits this translation unit for the build: 0 (default) the whole file; 1 everything except the
+// fp16 instantiations, which it reaches through launch_backward_f16(); 2 the fp16 instantiations alone.
+#ifndef FWA2_HALF
+#define FWA2_HALF 0
+#endif
+
 namespace fwa2 {
 
 constexpr int kRow = 40;    // LDS row stride of 16-bit tiles, in elements (80 bytes)
@@ -626,7 +632,9 @@ __global__ void __launch_bounds__(256) dkv_reduce_kernel(const BwdParams p) {
 // ---- host side -----------------------------------------------------------------
 static size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
+#if FWA2_HALF != 2
 int backward_supported(int n) { return n >= 1; }
+#endif
 
 void dq_geometry(int n, int* waves, int* chunks);
 hipError_t launch_backward_dq(const BwdParams& p, int dtype, bool has_bias, int mask_dt, hipStream_t st);
@@ -704,10 +712,12 @@ static BwdPlan make_plan(int heads, int n, int bw, bool has_bias, bool has_mask,
     return pl;
 }
 
+#if FWA2_HALF != 2
 size_t backward_workspace_bytes(int heads, int n, int bw, bool has_bias, bool has_mask, int n_windows, int cus) {
     if (!backward_supported(n)) return 0;
     return make_plan(heads, n, bw, has_bias, has_mask, n_windows, cus).total;
 }
+#endif
 
 // Persistent workgroups must all be resident at once: ask the runtime how many fit on a CU.
 template <class K>
@@ -869,9 +879,22 @@ static hipError_t launch_bwd_dt(BwdParams p, bool has_bias, int mask_dt, hipStre
     return e;
 }
 
-hipError_t launch_backward(const BwdParams& p, int dtype, bool has_bias, int mask_dt, hipStream_t st) {
-    if (dtype == FWA2_BF16) return launch_bwd_dt<FWA2_BF16>(p, has_bias, mask_dt, st);
+#if FWA2_HALF == 2
+hipError_t launch_backward_f16(const BwdParams& p, bool has_bias, int mask_dt, hipStream_t st) {
     return launch_bwd_dt<FWA2_F16>(p, has_bias, mask_dt, st);
 }
+#else
+#if FWA2_HALF == 1
+hipError_t launch_backward_f16(const BwdParams& p, bool has_bias, int mask_dt, hipStream_t st);
+#endif
+hipError_t launch_backward(const BwdParams& p, int dtype, bool has_bias, int mask_dt, hipStream_t st) {
+    if (dtype == FWA2_BF16) return launch_bwd_dt<FWA2_BF16>(p, has_bias, mask_dt, st);
+#if FWA2_HALF == 1
+    return launch_backward_f16(p, has_bias, mask_dt, st);
+#else
+    return launch_bwd_dt<FWA2_F16>(p, has_bias, mask_dt, st);
+#endif
+}
+#endif
 
 }  // namespace fwa2

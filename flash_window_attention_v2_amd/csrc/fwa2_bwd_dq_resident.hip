@@ -22,6 +22,12 @@
 // delta = rowsum(o * dO) is read from the buffer the key-side kernel wrote.
 #include "fwa2_common.hpp"
 
+// FWA2_HALF splits this translation unit for the build: 0 (default) the whole file; 1 everything except the
+// fp16 instantiations, which it reaches through launch_backward_dq_resident_f16(); 2 the fp16 instantiations alone.
+#ifndef FWA2_HALF
+#define FWA2_HALF 0
+#endif
+
 namespace fwa2 {
 
 constexpr int kDqSub = 2;    // 16-row query tiles per wavefront (see below)
@@ -410,7 +416,9 @@ __global__ void __launch_bounds__(64 * NT / SUB) bwd_dq_resident_kernel(const Bw
 }
 
 // ---- host side -----------------------------------------------------------------
+#if FWA2_HALF != 2
 int backward_dq_resident_supported(int n) { return n >= 1 && n <= 256; }
+#endif
 
 template <class K>
 static int resident_fit(K kern, int threads) {
@@ -497,10 +505,25 @@ static hipError_t launch_dt(const BwdParams& p, bool has_bias, int mask_dt, hipS
 }
 
 // max_groups: workgroups per head and launch that the workspace has dscale slots for.
+#if FWA2_HALF == 2
+hipError_t launch_backward_dq_resident_f16(const BwdParams& p, bool has_bias, int mask_dt, hipStream_t st, int max_groups,
+                                           int* ds_parts_out) {
+    return launch_dt<FWA2_F16>(p, has_bias, mask_dt, st, max_groups, ds_parts_out);
+}
+#else
+#if FWA2_HALF == 1
+hipError_t launch_backward_dq_resident_f16(const BwdParams& p, bool has_bias, int mask_dt, hipStream_t st, int max_groups,
+                                           int* ds_parts_out);
+#endif
 hipError_t launch_backward_dq_resident(const BwdParams& p, int dtype, bool has_bias, int mask_dt, hipStream_t st,
                                        int max_groups, int* ds_parts_out) {
     if (dtype == FWA2_BF16) return launch_dt<FWA2_BF16>(p, has_bias, mask_dt, st, max_groups, ds_parts_out);
+#if FWA2_HALF == 1
+    return launch_backward_dq_resident_f16(p, has_bias, mask_dt, st, max_groups, ds_parts_out);
+#else
     return launch_dt<FWA2_F16>(p, has_bias, mask_dt, st, max_groups, ds_parts_out);
+#endif
 }
+#endif
 
 }  // namespace fwa2

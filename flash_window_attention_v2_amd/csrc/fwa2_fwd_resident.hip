@@ -30,6 +30,12 @@
 // instantiation, so the common unmasked code carries no mask registers.
 #include "fwa2_common.hpp"
 
+// FWA2_HALF splits this translation unit for the build: 0 (default) the whole file; 1 everything except the
+// fp16 instantiations, which it reaches through launch_forward_resident_f16(); 2 the fp16 instantiations alone.
+#ifndef FWA2_HALF
+#define FWA2_HALF 0
+#endif
+
 namespace fwa2 {
 
 // NT = compile-time bound on the 16-key tiles of a unit (N <= 16 NT); the workgroup has
@@ -396,7 +402,9 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
 }
 
 // ---- host side -----------------------------------------------------------------
+#if FWA2_HALF != 2
 int forward_resident_supported(int n) { return n >= 1 && n <= 256; }
+#endif
 
 template <class K>
 static int resident_fit(K kern, int threads) {
@@ -464,9 +472,22 @@ static hipError_t launch_dt(const FwdParams& p, bool has_bias, int mask_dt, hipS
     return launch_mask<DT, false, DT>(p, st);
 }
 
-hipError_t launch_forward_resident(const FwdParams& p, int dtype, bool has_bias, int mask_dt, hipStream_t st) {
-    if (dtype == FWA2_BF16) return launch_dt<FWA2_BF16>(p, has_bias, mask_dt, st);
+#if FWA2_HALF == 2
+hipError_t launch_forward_resident_f16(const FwdParams& p, bool has_bias, int mask_dt, hipStream_t st) {
     return launch_dt<FWA2_F16>(p, has_bias, mask_dt, st);
 }
+#else
+#if FWA2_HALF == 1
+hipError_t launch_forward_resident_f16(const FwdParams& p, bool has_bias, int mask_dt, hipStream_t st);
+#endif
+hipError_t launch_forward_resident(const FwdParams& p, int dtype, bool has_bias, int mask_dt, hipStream_t st) {
+    if (dtype == FWA2_BF16) return launch_dt<FWA2_BF16>(p, has_bias, mask_dt, st);
+#if FWA2_HALF == 1
+    return launch_forward_resident_f16(p, has_bias, mask_dt, st);
+#else
+    return launch_dt<FWA2_F16>(p, has_bias, mask_dt, st);
+#endif
+}
+#endif
 
 }  // namespace fwa2
