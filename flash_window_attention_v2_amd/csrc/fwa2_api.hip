@@ -46,6 +46,9 @@ int check_t4(const char* name, const fwa2_tensor4& t, int head_dim) {
         return fail(FWA2_ERR_UNSUPPORTED,
                     "%s: rows must start on 16-byte boundaries (pointer 16-byte aligned, strides multiples of 8 elements)",
                     name);
+    if (t.stride_n >= (1 << 24))
+        return fail(FWA2_ERR_UNSUPPORTED, "%s: row stride %lld is beyond the 2^24 elements the kernels address rows with", name,
+                    (long long)t.stride_n);
     if (t.stride_n < head_dim) return fail(FWA2_ERR_INVALID_ARGUMENT, "%s: row stride %lld overlaps rows", name, (long long)t.stride_n);
     return FWA2_OK;
 }
@@ -85,6 +88,15 @@ int validate(const fwa2_problem* p, int backward) {
         if (p->logit_scale == nullptr) return fail(FWA2_ERR_INVALID_ARGUMENT, "logit_scale: null with FWA2_SCALE_TENSOR");
     } else if (p->scale_kind != FWA2_SCALE_DEFAULT) {
         return fail(FWA2_ERR_INVALID_ARGUMENT, "scale_kind %d unknown", p->scale_kind);
+    }
+    {
+        // rows inside a unit (an image with a window map) are addressed with 32-bit byte offsets
+        const int64_t rows = p->grid_h > 0 ? (int64_t)p->grid_h * p->grid_w : (p->n_keys > p->n ? p->n_keys : p->n);
+        const fwa2_tensor4* ts[] = {&p->q, &p->k, &p->v, &p->o, &p->d_o, &p->dq, &p->dk, &p->dv};
+        for (int i = 0; i < (backward ? 8 : 4); i++)
+            if (rows >= (1 << 24) || rows * ts[i]->stride_n >= (1LL << 30))
+                return fail(FWA2_ERR_UNSUPPORTED, "a unit spans more than 2^31 bytes (rows %lld, row stride %lld)", (long long)rows,
+                            (long long)ts[i]->stride_n);
     }
     if (p->n_keys < 0 || p->reserved0 != 0) return fail(FWA2_ERR_INVALID_ARGUMENT, "n_keys must not be negative, reserved0 must be 0");
     const int nk = p->n_keys > 0 ? p->n_keys : p->n;

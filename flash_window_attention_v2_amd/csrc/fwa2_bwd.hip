@@ -334,19 +334,20 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
             const int r = row0 + (lane >> 2);
             if constexpr (MAPPED) {
                 if (r < N) {
-                    async_row_chunk(reinterpret_cast<const E*>(p.q.ptr) + row_off<true>(p.q, p.map, b, h, r) + dc, L.rawQ + row0 * 32);
-                    async_row_chunk(reinterpret_cast<const E*>(p.d_o.ptr) + row_off<true>(p.d_o, p.map, b, h, r) + dc, L.rawDO + row0 * 32);
-                    async_row_chunk(reinterpret_cast<const E*>(p.o.ptr) + row_off<true>(p.o, p.map, b, h, r) + dc, L.rawO + row0 * 32);
-                    async_row_chunk(reinterpret_cast<const E*>(p.k.ptr) + row_off<true>(p.k, p.map, b, h, r) + dc, L.rawK + row0 * 32);
+                    const int pos = unit_row<true>(p.map, b, r);
+                    async_row_chunk(row_at(unit_ptr<true, E>(p.q, p.map, b, h), pos, p.q.sn, dc), L.rawQ + row0 * 32);
+                    async_row_chunk(row_at(unit_ptr<true, E>(p.d_o, p.map, b, h), pos, p.d_o.sn, dc), L.rawDO + row0 * 32);
+                    async_row_chunk(row_at(unit_ptr<true, E>(p.o, p.map, b, h), pos, p.o.sn, dc), L.rawO + row0 * 32);
+                    async_row_chunk(row_at(unit_ptr<true, E>(p.k, p.map, b, h), pos, p.k.sn, dc), L.rawK + row0 * 32);
                 }
                 continue;
             }
             if (r < N) {
-                async_row_chunk(qptr + (int64_t)r * p.q.sn + dc, L.rawQ + row0 * 32);
-                async_row_chunk(doptr + (int64_t)r * p.d_o.sn + dc, L.rawDO + row0 * 32);
-                async_row_chunk(optr + (int64_t)r * p.o.sn + dc, L.rawO + row0 * 32);
+                async_row_chunk(row_at(qptr, r, p.q.sn, dc), L.rawQ + row0 * 32);
+                async_row_chunk(row_at(doptr, r, p.d_o.sn, dc), L.rawDO + row0 * 32);
+                async_row_chunk(row_at(optr, r, p.o.sn, dc), L.rawO + row0 * 32);
             }
-            if (r < NK) async_row_chunk(kptr + (int64_t)r * p.k.sn + dc, L.rawK + row0 * 32);
+            if (r < NK) async_row_chunk(row_at(kptr, r, p.k.sn, dc), L.rawK + row0 * 32);
         }
         // v: every wavefront fetches exactly the key rows it owns, so nobody else reads them
 #pragma unroll
@@ -354,10 +355,10 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
             const int row0 = (wave * KT + kt) * 16;
             const int r = row0 + (lane >> 2);
             if constexpr (MAPPED) {
-                if (r < NK) async_row_chunk(reinterpret_cast<const E*>(p.v.ptr) + row_off<true>(p.v, p.map, b, h, r) + dc, L.rawV + row0 * 32);
+                if (r < NK) async_row_chunk(row_ptr<true, E>(p.v, p.map, b, h, r, dc), L.rawV + row0 * 32);
                 continue;
             }
-            if (r < NK) async_row_chunk(vptr + (int64_t)r * p.v.sn + dc, L.rawV + row0 * 32);
+            if (r < NK) async_row_chunk(row_at(vptr, r, p.v.sn, dc), L.rawV + row0 * 32);
         }
         for (int r0 = wave * 64; r0 < N; r0 += 64 * p.waves) {
             if (r0 + lane < N)
@@ -496,8 +497,8 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
                         *reinterpret_cast<f32x4*>(p.part_dv + row * 32 + 8 * g + 4 * dt) = v4;
                     }
                 } else {
-                    E* dkp = reinterpret_cast<E*>(const_cast<void*>(p.dk.ptr)) + row_off<MAPPED>(p.dk, p.map, b, h, key);
-                    E* dvp = reinterpret_cast<E*>(const_cast<void*>(p.dv.ptr)) + row_off<MAPPED>(p.dv, p.map, b, h, key);
+                    E* dkp = const_cast<E*>(row_ptr<MAPPED, E>(p.dk, p.map, b, h, key));
+                    E* dvp = const_cast<E*>(row_ptr<MAPPED, E>(p.dv, p.map, b, h, key));
                     V8 o8, v8;
 #pragma unroll
                     for (int j = 0; j < 8; j++) {

@@ -231,10 +231,10 @@ __global__ void __launch_bounds__(64 * NT / SUB) bwd_dq_resident_kernel(const Bw
             const int row0 = wave * WR + 16 * u;
             const int frow = row0 + (ln >> 2);
             if (frow < N) {
-                dma16(reinterpret_cast<const E*>(p.k.ptr) + row_off<MAPPED>(p.k, p.map, b, h, frow) + fc8, lds_rawK + row0 * 32);
-                dma16(reinterpret_cast<const E*>(p.v.ptr) + row_off<MAPPED>(p.v, p.map, b, h, frow) + fc8, lds_rawV + row0 * 32);
-                dma16(reinterpret_cast<const E*>(p.q.ptr) + row_off<MAPPED>(p.q, p.map, b, h, frow) + fc8, lds_rawQ + row0 * 32);
-                dma16(reinterpret_cast<const E*>(p.d_o.ptr) + row_off<MAPPED>(p.d_o, p.map, b, h, frow) + fc8,
+                dma16(row_ptr<MAPPED, E>(p.k, p.map, b, h, frow, fc8), lds_rawK + row0 * 32);
+                dma16(row_ptr<MAPPED, E>(p.v, p.map, b, h, frow, fc8), lds_rawV + row0 * 32);
+                dma16(row_ptr<MAPPED, E>(p.q, p.map, b, h, frow, fc8), lds_rawQ + row0 * 32);
+                dma16(row_ptr<MAPPED, E>(p.d_o, p.map, b, h, frow, fc8),
                       lds_rawDO + row0 * 32);
             }
             const int q = row0 + (ln & 15);
@@ -388,7 +388,7 @@ __global__ void __launch_bounds__(64 * NT / SUB) bwd_dq_resident_kernel(const Bw
             const float f = s_true * inv[u];
             const int q = wave * WR + 16 * u + (ln2 & 15);
             if (q < N) {
-                E* dqrow = reinterpret_cast<E*>(const_cast<void*>(p.dq.ptr)) + row_off<MAPPED>(p.dq, p.map, b, h, q);
+                E* dqrow = const_cast<E*>(row_ptr<MAPPED, E>(p.dq, p.map, b, h, q));
                 V8 o8;
 #pragma unroll
                 for (int j = 0; j < 8; j++) o8[j] = (E)(f * (dqacc[u][j >> 2][j & 3] - qh[j] * proj));

@@ -186,7 +186,7 @@ __global__ void __launch_bounds__(64 * NT, 3) bwd_fused_kernel(const BwdParams p
     // query in the operand layout (lane (query, g) takes columns 8g .. 8g+7); rows >= n read as zeros ----
     struct Rows { V8 k, v, q, dO, o; float lse; };
     auto ldrow = [&](const T4& t, int b, int row, int col) -> V8 {
-        return ld8<V8>(reinterpret_cast<const E*>(t.ptr) + row_off<MAPPED>(t, p.map, b, h, row) + col);
+        return ld8<V8>(row_ptr<MAPPED, E>(t, p.map, b, h, row, col));
     };
     auto fetch = [&](int b, Rows& r) __attribute__((always_inline)) {
         int ln = lane;                     // re-derived per call: no address lives across the unit loop
@@ -353,7 +353,7 @@ __global__ void __launch_bounds__(64 * NT, 3) bwd_fused_kernel(const BwdParams p
             const float f = s_true * inv;
             const int q = wave * 16 + (ln2 & 15);
             if (q < N) {
-                E* dqrow = reinterpret_cast<E*>(const_cast<void*>(p.dq.ptr)) + row_off<MAPPED>(p.dq, p.map, b, h, q);
+                E* dqrow = const_cast<E*>(row_ptr<MAPPED, E>(p.dq, p.map, b, h, q));
                 V8 o8;
 #pragma unroll
                 for (int j = 0; j < 8; j++) o8[j] = (E)(f * (dqacc[j >> 2][j & 3] - qh[j] * proj));
@@ -410,8 +410,8 @@ __global__ void __launch_bounds__(64 * NT, 3) bwd_fused_kernel(const BwdParams p
             const float kinv = fabsf(ki);
             const float proj = ki > 0.f ? dot : 0.f;
             if (key < N) {
-                E* dkp = reinterpret_cast<E*>(const_cast<void*>(p.dk.ptr)) + row_off<MAPPED>(p.dk, p.map, b, h, key);
-                E* dvp = reinterpret_cast<E*>(const_cast<void*>(p.dv.ptr)) + row_off<MAPPED>(p.dv, p.map, b, h, key);
+                E* dkp = const_cast<E*>(row_ptr<MAPPED, E>(p.dk, p.map, b, h, key));
+                E* dvp = const_cast<E*>(row_ptr<MAPPED, E>(p.dv, p.map, b, h, key));
                 V8 o8, v8;
 #pragma unroll
                 for (int j = 0; j < 8; j++) {

@@ -240,6 +240,41 @@ __device__ __forceinline__ int64_t row_off(const T4& t, const WinMap& m, int b, 
     return img * t.sb + h * t.sh + (int64_t)(y * m.gw + x) * t.sn;
 }
 
+// Row `row` of a tensor whose unit starts at `unit` (a wavefront-uniform pointer): one full-rate 24-bit
+// multiply and a 32-bit byte offset on the uniform base, instead of the 64-bit multiply-add chain (three
+// quarter-rate instructions and two 64-bit adds per address) that `unit + row * sn` costs with 64-bit strides.
+// The host checks that rows and row strides stay below 2^24 and their product below 2^31.
+template <class E>
+__device__ __forceinline__ const E* row_at(const E* unit, int row, int64_t sn, int col = 0) {
+    uint32_t prod;      // strides are wavefront-uniform (kernel arguments): src0 may be a scalar register
+    asm("v_mul_u32_u24 %0, %1, %2" : "=v"(prod) : "s"((uint32_t)sn), "v"((uint32_t)row));
+    const uint32_t boff = (prod + (uint32_t)col) * (uint32_t)sizeof(E);
+    return reinterpret_cast<const E*>(reinterpret_cast<const char*>(unit) + boff);
+}
+// Uniform start of unit b, head h (of its image with a window map) and the row's position inside it.
+template <bool MAPPED, class E>
+__device__ __forceinline__ const E* unit_ptr(const T4& t, const WinMap& m, int b, int h) {
+    const int64_t u = MAPPED ? (int64_t)(b / m.nw) * t.sb : (int64_t)b * t.sb;
+    return reinterpret_cast<const E*>(t.ptr) + u + h * t.sh;
+}
+template <bool MAPPED>
+__device__ __forceinline__ int unit_row(const WinMap& m, int b, int row) {
+    if (!MAPPED) return row;
+    const int w = b % m.nw;
+    const int wy = w / m.nwx, wx = w - wy * m.nwx;
+    const int r = (row * m.inv_ww) >> 16, c = row - r * m.ww;
+    int y = wy * m.wh + r + m.sh;
+    int x = wx * m.ww + c + m.sw;
+    y -= y >= m.gh ? m.gh : 0;
+    x -= x >= m.gw ? m.gw : 0;
+    return y * m.gw + x;
+}
+// The two together: address of row `row` of unit b, head h.
+template <bool MAPPED, class E>
+__device__ __forceinline__ const E* row_ptr(const T4& t, const WinMap& m, int b, int h, int row, int col = 0) {
+    return row_at(unit_ptr<MAPPED, E>(t, m, b, h), unit_row<MAPPED>(m, b, row), t.sn, col);
+}
+
 struct FwdParams {
     T4 q, k, v, o;
     WinMap map;

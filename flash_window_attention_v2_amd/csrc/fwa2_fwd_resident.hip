@@ -225,8 +225,8 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
         const int frow = wave * 16 + (ln >> 2);
         const int fc8 = (ln & 3) * 8;
         if (frow < N) {
-            const E* kp = reinterpret_cast<const E*>(p.k.ptr) + row_off<MAPPED>(p.k, p.map, b, h, frow) + fc8;
-            const E* vp = reinterpret_cast<const E*>(p.v.ptr) + row_off<MAPPED>(p.v, p.map, b, h, frow) + fc8;
+            const E* kp = row_ptr<MAPPED, E>(p.k, p.map, b, h, frow, fc8);
+            const E* vp = row_ptr<MAPPED, E>(p.v, p.map, b, h, frow, fc8);
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)kp,
                                              (__attribute__((address_space(3))) void*)(lds_rawK + wave * 16 * 32), 16, 0, kStreamPolicy);
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)vp,
@@ -234,7 +234,7 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
         }
         qq = zero8<V8>();
         const int fq = wave * 16 + (ln & 15);
-        if (fq < N) qq = ld8<V8>(reinterpret_cast<const E*>(p.q.ptr) + row_off<MAPPED>(p.q, p.map, b, h, fq) + 8 * (ln >> 4));
+        if (fq < N) qq = ld8<V8>(row_ptr<MAPPED, E>(p.q, p.map, b, h, fq, 8 * (ln >> 4)));
     };
     // landing area -> tiles: K normalised and rounded to fp16, V as is (rows >= n stay zero)
     auto stage = [&](int buf) __attribute__((always_inline)) {
@@ -384,7 +384,7 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
         asm volatile("" : "+v"(ln2));
         const int oq = wave * 16 + (ln2 & 15);
         if (qv) {
-            E* orow = reinterpret_cast<E*>(const_cast<void*>(p.o.ptr)) + row_off<MAPPED>(p.o, p.map, b, h, oq);
+            E* orow = const_cast<E*>(row_ptr<MAPPED, E>(p.o, p.map, b, h, oq));
             V8 ov;
 #pragma unroll
             for (int j = 0; j < 8; j++) ov[j] = (E)(oacc[j >> 2][j & 3] * inv_l);

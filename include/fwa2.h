@@ -21,7 +21,11 @@
  *   - strides are in ELEMENTS of the tensor's own type; the innermost (head
  *     dim) stride of q, k, v, o, do, dq, dk, dv is 1 and is not passed.  The
  *     other three strides are free, as in the reference
- *     (flash_window_attention_v2.py:20, attn_kernel_forward.py:313-328).
+ *     (flash_window_attention_v2.py:20, attn_kernel_forward.py:313-328),
+ *     within these bounds: row strides multiples of 8 elements and below
+ *     2^24, and one unit (a window's rows, or a whole image's token grid with
+ *     a window map) spanning less than 2^31 bytes, since rows inside a unit
+ *     are addressed with 32-bit offsets; unit and head strides are 64-bit.
  *   - all functions are re-entrant; the error string is thread-local.
  *   - return value 0 = FWA2_OK, otherwise an fwa2_status; fwa2_last_error()
  *     then describes the failure.

@@ -94,6 +94,15 @@ def test_validate_accepts_and_rejects(lib):
     assert lib.fwa2_validate(p, 0) == _abi.ERR_UNSUPPORTED
 
     p = _good_problem()
+    big = 1 << 24       # rows are addressed with a 24-bit multiply and a 32-bit byte offset inside a unit
+    p.q = _abi.Tensor4(0x10000, 2 * 64 * big, 64 * big, big)
+    assert lib.fwa2_validate(p, 0) == _abi.ERR_UNSUPPORTED and b"2^24" in lib.fwa2_last_error()
+    p = _good_problem(n=1 << 16)
+    wide = 1 << 14      # 2^16 rows of 2^14 elements: 2^31 bytes in one unit
+    p.q = _abi.Tensor4(0x10000, 2 * (1 << 16) * wide, (1 << 16) * wide, wide)
+    assert lib.fwa2_validate(p, 0) == _abi.ERR_UNSUPPORTED and b"2^31 bytes" in lib.fwa2_last_error()
+
+    p = _good_problem()
     p.scale_kind = _abi.SCALE_TENSOR  # without a pointer
     assert lib.fwa2_validate(p, 0) == _abi.ERR_INVALID_ARGUMENT
 
