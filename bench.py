@@ -104,14 +104,14 @@ def cpu_baseline(cfg, torch):
 
     cores = len(os.sched_getaffinity(0))
     torch.set_num_threads(cores)
-    sample_batch = 1
+    sample_batch = 8     # about 0.4 GB per N x N fp32 tensor; 10-20 s of host work in all
     small = dict(cfg, batch=sample_batch)
     inp = make_inputs(**small, dtype=torch.bfloat16, seed=0)
     args = (inp["q"], inp["k"], inp["v"], inp["logit_scale"], inp["bias"], inp["mask"], inp["do"])
     classic_fwd_bwd(*args)                       # warm-up
     times = []
-    t_end = time.perf_counter() + 20.0
-    while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 10):
+    t_end = time.perf_counter() + 15.0
+    while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 20):
         t0 = time.perf_counter()
         classic_fwd_bwd(*args)
         times.append(time.perf_counter() - t0)
