@@ -13,6 +13,7 @@ stdout; progress goes to stderr.
 import argparse
 import ctypes
 import json
+import math
 import os
 import sys
 import time
@@ -125,6 +126,75 @@ def cpu_baseline(cfg, torch):
     }
 
 
+def window_sweep(torch, steps, warmup):
+    """The reference's window-size sweep (benchmark/config.py: B16 x 16 windows, H6, d32, windows of 8, 12, 16, 24
+    and 32 tokens a side, bias = 16 sigmoid(randn), tensor logit scale ln 10, no mask) in bf16 and fp16, forward
+    and forward + backward.  Every case is timed twice: as eager calls, and as one captured HIP graph replayed
+    `steps` times, which takes the host out of the figure (at 1 536 units the eager calls are bound by it up to
+    256 tokens).  TFLOP/s count the matrix products only (4 N^2 d forward, 14 N^2 d forward + backward)."""
+    from flash_window_attention_v2_amd import flash_win_attn_v2_func
+
+    def timed(fn):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / steps
+
+    def captured(fn):
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                fn()
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            fn()
+        return graph.replay
+
+    bw, heads, d = 16 * 16, 6, 32
+    rows = []
+    for dtype in (torch.bfloat16, torch.float16):
+        for n in (64, 144, 256, 576, 1024):
+            g = torch.Generator(device="cpu").manual_seed(0)
+            q, k, v, do = (torch.randn(bw, heads, n, d, generator=g).to(dtype).cuda() for _ in range(4))
+            bias = (16 * torch.sigmoid(torch.randn(heads, n, n, generator=g))).to(dtype).cuda()
+            ls = torch.full((heads, 1, 1), math.log(10.0), dtype=dtype, device="cuda")
+            leaves = (q, k, v, bias, ls)
+            for t in leaves:
+                t.requires_grad_(True)
+
+            def fwd():
+                with torch.no_grad():
+                    return flash_win_attn_v2_func(q, k, v, ls, bias, None)
+
+            def fwd_bwd():
+                for t in leaves:
+                    t.grad = None
+                flash_win_attn_v2_func(q, k, v, ls, bias, None).backward(do)
+
+            fl = flops_matmul(bw, heads, n, d, bwd=False)
+            fl_all = flops_matmul(bw, heads, n, d)
+            row = {"dtype": str(dtype).split(".")[-1], "n": n}
+            for tag, fn, f in (("fwd", fwd, fl), ("fwd_bwd", fwd_bwd, fl_all)):
+                ms_e = timed(fn)
+                ms_g = timed(captured(fn))
+                row[tag + "_ms"] = round(ms_e, 4)
+                row[tag + "_tflops"] = round(f / ms_e * 1e-9, 1)
+                row[tag + "_graph_ms"] = round(ms_g, 4)
+                row[tag + "_graph_tflops"] = round(f / ms_g * 1e-9, 1)
+            log(f"[bench] sweep {row}")
+            rows.append(row)
+    return {"sweep": "B16 x 16 windows, H6, d32, bias, tensor scale, no mask; TFLOP/s of the matrix products",
+            "steps": steps, "warmup": warmup, "rows": rows}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -132,6 +202,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip forward-only, N=64 and memory figures")
+    ap.add_argument("--sweep", action="store_true",
+                    help="instead of the benchmark line, print the window-size sweep (TFLOP/s versus N) as one JSON line")
     ap.add_argument("--copy-bytes", type=int, default=0,
                     help="also run one plain device copy of this many bytes (reference point for HBM counters)")
     args = ap.parse_args()
@@ -147,6 +219,9 @@ def main():
         sys.exit("bench.py: no GPU visible")
     lib = _abi.load()
     torch.cuda.set_device(0)
+    if args.sweep:
+        print(json.dumps(window_sweep(torch, args.steps, args.warmup)), flush=True)
+        return
 
     def setup(cfg):
         inp = make_inputs(**cfg, dtype=torch.bfloat16, seed=0)
