@@ -28,6 +28,8 @@
 // bias and mask are read key-major (transposed once per call by a small
 // pre-pass into the workspace) so that a lane's scores are one vector load,
 // and are fetched one block ahead of their use.
+#include <atomic>
+
 #include "fwa2_common.hpp"
 
 // FWA2_HALF splits this translation unit for the build: 0 (default) the whole file; 1 everything except the
@@ -720,7 +722,8 @@ size_t backward_workspace_bytes(int heads, int n, int bw, bool has_bias, bool ha
 }
 #endif
 
-// Persistent workgroups must all be resident at once: ask the runtime how many fit on a CU.
+// Persistent workgroups should all be resident at once (one that waits for a slot starts its share late; nothing
+// depends on it for correctness): ask the runtime how many fit on a CU.
 template <class K>
 static int resident_per_cu(K kern, int threads) {
     int n = 0;
@@ -733,17 +736,21 @@ static hipError_t launch_main(BwdParams p, const BwdPlan& pl, hipStream_t st, in
     // Up to 64 tokens one launch walks masked and unmasked units alike; above that the two copies of
     // the block sequence cost occupancy (128 tokens) or spill (256), and each kind gets a launch.
     constexpr bool kOneLaunch = MASK_DT >= 0 && NQB <= 2 && !BIG;
-    // never more workgroups per head (and super-tile) than the plan sized the workspace for
-    static const int fit = [&] {
+    // asked once per block size (the wavefront count follows the window length); a benign race at worst repeats the query
+    static std::atomic<int> fit_by_waves[17];
+    int fit = pl.waves <= 16 ? fit_by_waves[pl.waves].load(std::memory_order_relaxed) : 0;
+    if (fit == 0) {
         if constexpr (kOneLaunch) {
-            return resident_per_cu(bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, 2, BIG, MAPPED>, 64 * pl.waves);
+            fit = resident_per_cu(bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, 2, BIG, MAPPED>, 64 * pl.waves);
         } else {
             const int a = resident_per_cu(bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, 0, BIG, MAPPED>, 64 * pl.waves);
             const int b = MASK_DT >= 0 ? resident_per_cu(bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, 1, BIG, MAPPED>, 64 * pl.waves) : a;
-            return a < b ? a : b;
+            fit = a < b ? a : b;
         }
-    }();
+        if (pl.waves <= 16) fit_by_waves[pl.waves].store(fit, std::memory_order_relaxed);
+    }
     const int tiles = pl.n_chunks * pl.n_chunks;
+    // never more workgroups per head (and super-tile) than the plan sized the workspace for
     int groups = (p.cus * fit) / (p.heads * tiles);
     if (groups < 1) groups = 1;
     if (groups > pl.groups) groups = pl.groups;
