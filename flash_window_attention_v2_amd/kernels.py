@@ -161,6 +161,8 @@ def _flash_attn_forward(q, k, v, logit_scale, bias=None, mask=None, scale_type="
     lib = _abi.load()
     lse = torch.empty((bw, heads, (n + 63) // 64 * 64), device=q.device, dtype=torch.float32)
     o = torch.empty_like(q)
+    if bw == 0:         # nothing to launch: the classic path returns an empty output here too
+        return o, lse, logit_scale
     if not _rows_16b_aligned(o):
         o = torch.empty(q.shape, device=q.device, dtype=q.dtype)
     p = _describe(q, k, v, o, lse, logit_scale, bias, mask, _flags_for(mask), scale_type)
@@ -174,6 +176,11 @@ def _flash_attn_backward(do, q, k, v, logit_scale, o, lse, dq, dk, dv, dscale, d
                          scale_type="scalar"):
     """Fills dq, dk, dv (and dscale, db when given) in place, as the reference's launcher does
     (attn_kernel_backward.py:567-711); dscale already carries the clamp mask (l <= ln 100)."""
+    if q.shape[0] == 0:     # an empty batch: the sums over units are empty
+        for t in (db, dscale):
+            if t is not None:
+                t.zero_()
+        return
     do, q, k, v, o = (_kernel_ready(x) for x in (do, q, k, v, o))
     if bias is not None and bias.stride(-1) != 1:
         bias = bias.contiguous()

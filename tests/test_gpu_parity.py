@@ -457,3 +457,25 @@ def test_launchers_under_the_reference_names():
     o2, _, _ = _flash_attn_forward(q, k, v, torch.empty((), device="cuda"), bias=bias, mask=mask, scale_type="scalar")
     ref2 = classic_fwd_bwd(inp["q"], inp["k"], inp["v"], None, inp["bias"], inp["mask"], inp["do"])
     assert float((o2.float().cpu() - ref2["o"]).abs().max()) <= 2e-2
+
+
+def test_empty_batch():
+    """No units: an empty output, empty q / k / v gradients and zero bias / scale gradients, as the classic path gives."""
+    from flash_window_attention_v2_amd import flash_win_attn_v2_func, win_attention_torch
+    heads, n, d = 2, 64, 32
+    q, k, v = (torch.zeros(0, heads, n, d, device="cuda", dtype=torch.bfloat16, requires_grad=True) for _ in range(3))
+    bias = torch.randn(heads, n, n, device="cuda", dtype=torch.bfloat16, requires_grad=True)
+    scale = torch.full((heads, 1, 1), 2.0, device="cuda", dtype=torch.bfloat16, requires_grad=True)
+    got = {}
+    for name, fn in (("flash", flash_win_attn_v2_func), ("classic", win_attention_torch)):
+        for t in (q, k, v, bias, scale):
+            t.grad = None
+        o = fn(q, k, v, scale, bias, None)
+        assert o.shape == q.shape and o.dtype == q.dtype
+        o.backward(torch.zeros_like(o))
+        got[name] = [None if t.grad is None else t.grad.clone() for t in (q, k, v, bias, scale)]
+    for a, b, t in zip(got["flash"], got["classic"], (q, k, v, bias, scale)):
+        assert a is not None and a.shape == t.shape
+        assert float(a.abs().sum()) == 0.0
+        if b is not None:
+            assert torch.equal(a.float(), b.float())
