@@ -692,7 +692,7 @@ static BwdPlan make_plan(int heads, int n, int bw, bool has_bias, bool has_mask,
         pl.npk = pl.r = tile * pl.n_chunks;
         wg_per_cu = 1;
     } else {
-        pl.nqb_t = nqb <= 2 ? 2 : (nqb <= 4 ? 4 : 8);
+        pl.nqb_t = nqb <= 2 ? 2 : (nqb <= 4 ? 4 : (nqb == 5 ? 5 : 8));   // 5: 129 .. 160 tokens, tiles of 160 rows
         pl.r = 32 * pl.nqb_t;
         // up to 160 queries a wavefront owns one 16-key tile (<= 128 registers; several workgroups
         // per CU up to 128 queries, and at 129 .. 160 nine or ten wavefronts instead of five, which
@@ -803,14 +803,14 @@ static hipError_t launch_nqb(const BwdParams& p, const BwdPlan& pl, hipStream_t 
         // windows of up to 64 tokens with a map go to the fused kernel, longer than 256 are refused earlier
         if (pl.n_chunks > 1 || pl.nqb_t == 2) return hipErrorInvalidValue;
         if (pl.nqb_t == 4) return launch_main<DT, HAS_BIAS, MASK_DT, 4, 1, false, true>(p, pl, st, groups_out);
-        if (pl.kt == 1) return launch_main<DT, HAS_BIAS, MASK_DT, 8, 1, false, true>(p, pl, st, groups_out);
+        if (pl.kt == 1) return launch_main<DT, HAS_BIAS, MASK_DT, 5, 1, false, true>(p, pl, st, groups_out);
         return launch_main<DT, HAS_BIAS, MASK_DT, 8, 2, false, true>(p, pl, st, groups_out);
     }
     if (pl.n_chunks > 1 && pl.nqb_t == 6) return launch_main<DT, HAS_BIAS, MASK_DT, 6, 2, true>(p, pl, st, groups_out);
     if (pl.n_chunks > 1) return launch_main<DT, HAS_BIAS, MASK_DT, 8, 2, true>(p, pl, st, groups_out);
     if (pl.nqb_t == 2) return launch_main<DT, HAS_BIAS, MASK_DT, 2, 1, false>(p, pl, st, groups_out);
     if (pl.nqb_t == 4) return launch_main<DT, HAS_BIAS, MASK_DT, 4, 1, false>(p, pl, st, groups_out);
-    if (pl.kt == 1) return launch_main<DT, HAS_BIAS, MASK_DT, 8, 1, false>(p, pl, st, groups_out);
+    if (pl.kt == 1) return launch_main<DT, HAS_BIAS, MASK_DT, 5, 1, false>(p, pl, st, groups_out);
     return launch_main<DT, HAS_BIAS, MASK_DT, 8, 2, false>(p, pl, st, groups_out);
 }
 
