@@ -472,23 +472,24 @@ static hipError_t launch_mask(const BwdParams& p, hipStream_t st, int mg, int* o
         if (nt == 4) return hipErrorInvalidValue;
         if (p.side_vec) {
             if (nt == 8) return launch_nt<DT, HAS_BIAS, MASK_DT, 8, true, kDqSub, true>(p, st, mg, out);
-            if (p.n <= 160) return launch_nt<DT, HAS_BIAS, MASK_DT, 16, true, 1, true>(p, st, mg, out);
+            if (p.n <= 160) return launch_nt<DT, HAS_BIAS, MASK_DT, 10, true, 1, true>(p, st, mg, out);
             return launch_nt<DT, HAS_BIAS, MASK_DT, 16, true, kDqSub, true>(p, st, mg, out);
         }
         if (nt == 8) return launch_nt<DT, HAS_BIAS, MASK_DT, 8, false, kDqSub, true>(p, st, mg, out);
-        if (p.n <= 160) return launch_nt<DT, HAS_BIAS, MASK_DT, 16, false, 1, true>(p, st, mg, out);
+        if (p.n <= 160) return launch_nt<DT, HAS_BIAS, MASK_DT, 10, false, 1, true>(p, st, mg, out);
         return launch_nt<DT, HAS_BIAS, MASK_DT, 16, false, kDqSub, true>(p, st, mg, out);
     }
     if (p.side_vec) {
         if (nt == 4) return launch_nt<DT, HAS_BIAS, MASK_DT, 4, true>(p, st, mg, out);
         if (nt == 8) return launch_nt<DT, HAS_BIAS, MASK_DT, 8, true>(p, st, mg, out);
-        // 129 .. 160 tokens: 16 rows per wavefront give nine or ten wavefronts instead of five
-        if (p.n <= 160) return launch_nt<DT, HAS_BIAS, MASK_DT, 16, true, 1>(p, st, mg, out);
+        // 129 .. 160 tokens: tiles of 160 keys (40 registers of resident bias per 16 rows instead of 64), and 16 rows
+        // per wavefront, which gives nine or ten wavefronts instead of five
+        if (p.n <= 160) return launch_nt<DT, HAS_BIAS, MASK_DT, 10, true, 1>(p, st, mg, out);
         return launch_nt<DT, HAS_BIAS, MASK_DT, 16, true>(p, st, mg, out);
     }
     if (nt == 4) return launch_nt<DT, HAS_BIAS, MASK_DT, 4, false>(p, st, mg, out);
     if (nt == 8) return launch_nt<DT, HAS_BIAS, MASK_DT, 8, false>(p, st, mg, out);
-    if (p.n <= 160) return launch_nt<DT, HAS_BIAS, MASK_DT, 16, false, 1>(p, st, mg, out);
+    if (p.n <= 160) return launch_nt<DT, HAS_BIAS, MASK_DT, 10, false, 1>(p, st, mg, out);
     return launch_nt<DT, HAS_BIAS, MASK_DT, 16, false>(p, st, mg, out);
 }
 
