@@ -113,9 +113,10 @@ __device__ __forceinline__ void unit_blocks(BwdLds<DT, NQB>& L, WaveRegs<DT, NQB
 
     // The operands of a block's first query tile (q_hat and dO rows, -lse and -delta) are read from LDS while the
     // previous block finishes, so that a block does not open with a wait for them.
-    // (not with a live mask, whose values in flight take the registers this needs, nor with one key tile per
-    // wavefront, where the budget is 128 registers: both would spill)
-    constexpr bool PF = !MASKED && KT == 2;
+    // (with a live mask only the two rows: the mask values in flight take the registers of the accumulator inits;
+    // not with one key tile per wavefront, where the budget is 128 registers and any of it would spill)
+    constexpr bool PF = KT == 2;              // the two rows
+    constexpr bool PFI = !MASKED && KT == 2;  // and the accumulator inits
     V8 aq0, ado0;
     f32x4 nl0, nd0;
     auto fetch_first = [&](int qbn) __attribute__((always_inline)) {
@@ -123,8 +124,10 @@ __device__ __forceinline__ void unit_blocks(BwdLds<DT, NQB>& L, WaveRegs<DT, NQB
         const int rowq = 32 * qbn + 8 * (l16 >> 2) + (l16 & 3);
         aq0 = ld8<V8>(L.Qs + rowq * kRow + 8 * g);
         ado0 = ld8<V8>(L.dOs + rowq * kRow + 8 * g);
-        nl0 = *reinterpret_cast<const f32x4*>(L.nlse2 + 32 * qbn + 8 * g);
-        nd0 = *reinterpret_cast<const f32x4*>(L.ndelta + 32 * qbn + 8 * g);
+        if (PFI) {
+            nl0 = *reinterpret_cast<const f32x4*>(L.nlse2 + 32 * qbn + 8 * g);
+            nd0 = *reinterpret_cast<const f32x4*>(L.ndelta + 32 * qbn + 8 * g);
+        }
     };
     fetch_first(0);
 
@@ -153,8 +156,8 @@ __device__ __forceinline__ void unit_blocks(BwdLds<DT, NQB>& L, WaveRegs<DT, NQB
                     const V8 aq = (PF && t == 0) ? aq0 : ld8<V8>(L.Qs + rowq * kRow + 8 * g);
                     const V8 ado = (PF && t == 0) ? ado0 : ld8<V8>(L.dOs + rowq * kRow + 8 * g);
                     // accumulator inits: -lse*log2e and -delta of this lane's 4 queries
-                    const f32x4 nl = (PF && t == 0) ? nl0 : *reinterpret_cast<const f32x4*>(L.nlse2 + q8 + 4 * t);
-                    const f32x4 nd = (PF && t == 0) ? nd0 : *reinterpret_cast<const f32x4*>(L.ndelta + q8 + 4 * t);
+                    const f32x4 nl = (PFI && t == 0) ? nl0 : *reinterpret_cast<const f32x4*>(L.nlse2 + q8 + 4 * t);
+                    const f32x4 nd = (PFI && t == 0) ? nd0 : *reinterpret_cast<const f32x4*>(L.ndelta + q8 + 4 * t);
                     f32x4 sacc = Elem<DT>::mfma16(aq, bk_now, nl);            // (S - lse) * log2e
                     const f32x4 pacc = Elem<DT>::mfma16(ado, w.bv[kt], nd);   // dP - delta
                     if (HAS_BIAS) {   // padded key rows of bias_t hold -inf
