@@ -14,6 +14,7 @@ ABI_VERSION = 2
 OK, ERR_INVALID_ARGUMENT, ERR_UNSUPPORTED, ERR_HIP, ERR_NO_DEVICE = range(5)
 F16, BF16, F32 = 0, 1, 2
 SCALE_DEFAULT, SCALE_TENSOR = 0, 1
+STATIC_SCRATCH_BYTES = 64 << 20     # FWA2_STATIC_SCRATCH_BYTES of include/fwa2.h
 
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libfwa2.so")
 
@@ -25,6 +26,7 @@ EXPORTS = (
     "fwa2_backward_workspace_bytes",
     "fwa2_forward",
     "fwa2_backward",
+    "fwa2_backward_static",
     "fwa2_cpb_bias_forward",
     "fwa2_cpb_bias_backward",
     "fwa2_set_kernel_events",
@@ -100,6 +102,8 @@ def load():
         lib.fwa2_forward.restype = ctypes.c_int
         lib.fwa2_backward.argtypes = [ctypes.POINTER(Problem)]
         lib.fwa2_backward.restype = ctypes.c_int
+        lib.fwa2_backward_static.argtypes = [ctypes.POINTER(Problem)]
+        lib.fwa2_backward_static.restype = ctypes.c_int
         lib.fwa2_cpb_bias_forward.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                               ctypes.c_void_p, ctypes.c_void_p]
         lib.fwa2_cpb_bias_forward.restype = ctypes.c_int

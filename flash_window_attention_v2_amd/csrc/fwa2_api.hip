@@ -2,6 +2,7 @@
 // validation, workspace sizing and dispatch to the gfx950 kernels.  Nothing
 // here allocates device memory or synchronises.
 #include <atomic>
+#include <mutex>
 #include <stdarg.h>
 #include <stdio.h>
 #include <stdlib.h>
@@ -55,14 +56,45 @@ int check_t4(const char* name, const fwa2_tensor4& t, int head_dim) {
 
 fwa2::T4 to_t4(const fwa2_tensor4& t) { return fwa2::T4{t.ptr, t.stride_bw, t.stride_h, t.stride_n}; }
 
+// Compute units of the CURRENT device, asked once per device (a property query: no device memory is touched and
+// nothing is launched).  Without a visible device the MI355X's 256 are assumed, so that a host-only caller of
+// fwa2_validate / fwa2_backward_workspace_bytes sees the sizes of the part this library is written for.
+constexpr int kMaxDevices = 64;
+std::atomic<int> g_cus[kMaxDevices];
 int cu_count() {
-    static int cus = [] {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) != hipSuccess) return 256;
-        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 256;
-        return n;
-    }();
-    return cus;
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256;
+    n = g_cus[dev].load(std::memory_order_relaxed);
+    if (n > 0) return n;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 256;
+    g_cus[dev].store(n, std::memory_order_relaxed);
+    return n;
+}
+
+// ---- scratch of the allocation-free backward entry point ----
+// One copy of this array exists on every GPU the library is loaded on and stays there until the process ends.
+// Host code never uses the array's name as an address: scratch_of_current_device() asks the runtime for the
+// address of the current device's copy, once per device, and every later use goes through that pointer.
+constexpr size_t kStaticScratchBytes = FWA2_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+std::mutex g_scratch_mu;
+void* g_scratch_ptr[kMaxDevices];
+
+int scratch_of_current_device(void** out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess) return fail(FWA2_ERR_NO_DEVICE, "fwa2_backward_static: no current device");
+    if (dev < 0 || dev >= kMaxDevices)
+        return fail(FWA2_ERR_UNSUPPORTED, "fwa2_backward_static: device index %d is beyond the %d this library tracks", dev, kMaxDevices);
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void* ptr = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || ptr == nullptr)
+            return fail(FWA2_ERR_HIP, "fwa2_backward_static: address of the scratch array on device %d: %s", dev, hipGetErrorString(e));
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return FWA2_OK;
 }
 
 int validate(const fwa2_problem* p, int backward) {
@@ -262,8 +294,7 @@ int fwa2_forward(const fwa2_problem* p) {
     return FWA2_OK;
 }
 
-int fwa2_backward(const fwa2_problem* p) {
-    g_err[0] = 0;
+static int run_backward(const fwa2_problem* p) {
     int rc = validate(p, 1);
     if (rc) return rc;
     if (fwa2::generic_problem(p->head_dim, p->n, p->n_keys > 0 ? p->n_keys : p->n)) {
@@ -296,6 +327,33 @@ int fwa2_backward(const fwa2_problem* p) {
                                          (hipStream_t)p->stream);
     if (e != hipSuccess) return fail(FWA2_ERR_HIP, "backward launch: %s", hipGetErrorString(e));
     return FWA2_OK;
+}
+
+int fwa2_backward(const fwa2_problem* p) {
+    g_err[0] = 0;
+    return run_backward(p);
+}
+
+int fwa2_backward_static(const fwa2_problem* p) {
+    g_err[0] = 0;
+    if (p == nullptr) return fail(FWA2_ERR_INVALID_ARGUMENT, "problem is null");
+    if (p->struct_bytes != sizeof(fwa2_problem) || p->abi_version != FWA2_ABI_VERSION)
+        return fail(FWA2_ERR_INVALID_ARGUMENT, "fwa2_problem layout mismatch: caller %u bytes / abi %u, library %zu bytes / abi %d",
+                    p->struct_bytes, p->abi_version, sizeof(fwa2_problem), FWA2_ABI_VERSION);
+    int rc = validate(p, 0);      // sizes and dtypes are sane before the workspace is sized from them
+    if (rc) return rc;
+    const size_t need = fwa2_backward_workspace_bytes(p);
+    if (need > kStaticScratchBytes)
+        return fail(FWA2_ERR_UNSUPPORTED,
+                    "fwa2_backward_static: this problem needs %zu bytes of scratch, the library's static buffer holds %zu; "
+                    "use fwa2_backward with a caller-owned workspace", need, kStaticScratchBytes);
+    void* ptr = nullptr;
+    rc = scratch_of_current_device(&ptr);
+    if (rc) return rc;
+    fwa2_problem q = *p;
+    q.workspace = ptr;
+    q.workspace_bytes = kStaticScratchBytes;
+    return run_backward(&q);
 }
 
 }  // extern "C"

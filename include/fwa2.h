@@ -150,10 +150,14 @@ int fwa2_abi_version(void);
 const char* fwa2_last_error(void);
 
 /*
- * Checks a problem description against the contract without touching the
- * device (shapes, dtypes, strides, NULL-ness, supported sizes).  `backward`
- * non-zero also checks the (bwd) fields.  Mirrors the assertions at
- * attn_kernel_forward.py:263-292 and attn_kernel_backward.py:571-579, 616-633.
+ * Checks a problem description against the contract (shapes, dtypes, strides,
+ * NULL-ness, supported sizes) without reading device memory or launching
+ * anything.  `backward` non-zero also checks the (bwd) fields, among them the
+ * workspace size, which depends on the compute-unit count of the CURRENT
+ * device: that one property is asked from the runtime (once per device); a
+ * process without a visible device gets the sizes of a 256-CU part (MI355X).
+ * Mirrors the assertions at attn_kernel_forward.py:263-292 and
+ * attn_kernel_backward.py:571-579, 616-633.
  */
 int fwa2_validate(const fwa2_problem* p, int backward);
 
@@ -170,9 +174,11 @@ int fwa2_mask_scan(const void* mask, int mask_dtype, int n_windows, int n, int64
                    uint8_t* live, void* stream);
 
 /*
- * Bytes of device scratch fwa2_backward needs for this problem (fp32
- * accumulators for dbias and dscale; the reference allocates these as
- * db_accum / dscale_accum, attn_kernel_backward.py:609-626).  0 if none.
+ * Bytes of device scratch fwa2_backward needs for this problem on the CURRENT
+ * device (fp32 accumulators for dbias and dscale; the reference allocates these
+ * as db_accum / dscale_accum, attn_kernel_backward.py:609-626).  0 if none.
+ * The figure grows with the device's compute-unit count (one partial dbias
+ * tile per persistent workgroup); see fwa2_validate.
  */
 size_t fwa2_backward_workspace_bytes(const fwa2_problem* p);
 
@@ -189,6 +195,25 @@ int fwa2_forward(const fwa2_problem* p);
  * copies and the clamp gate on dscale.
  */
 int fwa2_backward(const fwa2_problem* p);
+
+/*
+ * fwa2_backward for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc): the same kernels and results as fwa2_backward, but the scratch lives
+ * in a device array of FWA2_STATIC_SCRATCH_BYTES that the library holds on every GPU it is loaded on until the
+ * process ends; p->workspace and p->workspace_bytes are ignored.  The call allocates and frees nothing.
+ * Has no counterpart in the reference (whose launcher allocates dq_accum, db_accum, dscale_accum and delta with
+ * torch on every call, attn_kernel_backward.py:582-626).
+ *   - a problem whose fwa2_backward_workspace_bytes() exceeds FWA2_STATIC_SCRATCH_BYTES is refused with
+ *     FWA2_ERR_UNSUPPORTED (windows of 256 tokens with bias and mask fit up to about 10 workgroups per head
+ *     and launch; the 4 096-window benchmark shape does not: use fwa2_backward there);
+ *   - the device that is current at the call must be the one the tensors and the stream belong to; the address
+ *     of that device's copy of the array is looked up on the first call per device;
+ *   - every call on a GPU shares that GPU's array: calls that may overlap on one GPU (different streams, or
+ *     different threads without ordering) race on it.  Calls on one stream are ordered and safe.  Nothing in
+ *     the array needs clearing between calls: every kernel writes what a later kernel of the same call reads.
+ */
+#define FWA2_STATIC_SCRATCH_BYTES ((size_t)64 << 20)
+int fwa2_backward_static(const fwa2_problem* p);
 
 /*
  * Relative position bias of a window of wh x ww tokens (N = wh ww) from its table, for the caller of the

@@ -176,3 +176,17 @@ def test_header_compiles_as_c_and_cxx(tmp_path):
     cxx = tmp_path / "use_header.cpp"
     cxx.write_text('#include "fwa2.h"\nint main() { fwa2_problem p{}; return p.n; }\n')
     subprocess.run(["g++", "-std=c++17", "-Wall", "-Werror", "-I", inc, "-fsyntax-only", str(cxx)], check=True)
+
+
+def test_static_scratch_backward_refuses_oversize_without_a_device(lib):
+    """The allocation-free backward sizes the problem before it looks for a device: the benchmark shape needs
+    more scratch than the library's static buffer and is refused with the limit in the message."""
+    p = _good_problem(n=256, bw=4096, heads=3, backward=True)
+    p.bias.ptr, p.bias.stride_a, p.bias.stride_n = 0x10000, 256 * 256, 256
+    p.dbias = 0x10000
+    assert lib.fwa2_backward_workspace_bytes(p) > _abi.STATIC_SCRATCH_BYTES
+    assert lib.fwa2_backward_static(p) == _abi.ERR_UNSUPPORTED
+    msg = lib.fwa2_last_error().decode()
+    assert "static buffer holds" in msg and str(_abi.STATIC_SCRATCH_BYTES) in msg
+    header = open(os.path.join(ROOT, "include", "fwa2.h")).read()
+    assert re.search(r"#define FWA2_STATIC_SCRATCH_BYTES \(\(size_t\)64 << 20\)", header) and _abi.STATIC_SCRATCH_BYTES == 64 << 20
