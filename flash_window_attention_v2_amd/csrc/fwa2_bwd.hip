@@ -670,8 +670,17 @@ hipError_t launch_backward_fused(const BwdParams& p, int dtype, bool has_bias, i
 hipError_t launch_backward_dq_resident(const BwdParams& p, int dtype, bool has_bias, int mask_dt, hipStream_t st,
                                        int max_groups, int* ds_parts_out);
 
+// Largest set of score tables bwd_key_kernel may ask for (one 256 KB table per head and per (window, head) of a
+// masked call); calls beyond it stay on bwd_kernel, which streams bias and mask from key-major copies.
+constexpr size_t kTableBudget = (size_t)96 << 20;
+
+hipError_t launch_backward_key(const BwdParams& p, int dtype, bool has_bias, int mask_dt, hipStream_t st, int max_groups,
+                               int* groups_out);
+
 struct BwdPlan {
     int waves, groups, npk, r, nqb_t, kt, dq_waves, dq_chunks, ds_parts, dq_max_groups;
+    bool key256;    // 161 .. 256 tokens: bwd_key_kernel (fwa2_bwd_key.hip) is the key-side kernel
+    size_t off_tab;
     int n_chunks;   // > 1: windows of more than 256 tokens, cut into 256 x 256 or 192 x 192 super-tiles
     size_t off_dbias, off_dscale, off_bias_t, off_mask_t, off_delta, off_dk, off_dv, total;
     size_t smem;
@@ -681,6 +690,7 @@ static BwdPlan make_plan(int heads, int n, int bw, bool has_bias, bool has_mask,
     BwdPlan pl;
     const int nqb = (n + 31) / 32;
     pl.n_chunks = (n + 255) / 256;
+    pl.key256 = false;
     int wg_per_cu;
     if (pl.n_chunks > 1) {
         // every workgroup is a full super-tile kernel of 256 x 256, or of 192 x 192 where that pads the
@@ -705,6 +715,14 @@ static BwdPlan make_plan(int heads, int n, int bw, bool has_bias, bool has_mask,
         pl.waves = (n + 16 * pl.kt - 1) / (16 * pl.kt);
         pl.npk = pl.waves * 16 * pl.kt;
         wg_per_cu = pl.nqb_t == 2 ? 4 : (pl.nqb_t == 4 ? 2 : 1);
+        const size_t slots = (size_t)heads * (1 + (has_mask ? n_windows : 0));
+        if (pl.nqb_t == 8 && slots * 256 * 256 * 4 <= kTableBudget) {
+            // four wavefronts of four key tiles on 256 x 256 tiles whatever the window length
+            pl.key256 = true;
+            pl.kt = 4;
+            pl.waves = 4;
+            pl.npk = 256;
+        }
     }
     int groups = (cus * wg_per_cu) / (heads * pl.n_chunks * pl.n_chunks);
     if (groups < 1) groups = 1;
@@ -712,7 +730,8 @@ static BwdPlan make_plan(int heads, int n, int bw, bool has_bias, bool has_mask,
     pl.groups = groups;
     size_t off = 0;
     pl.off_dbias = off;
-    if (has_bias) off += align256((size_t)heads * 2 * groups * pl.npk * pl.r * 4);
+    // one partial tile per workgroup and launch: two launches (masked / unmasked units) except for bwd_key_kernel
+    if (has_bias) off += align256((size_t)heads * (pl.key256 ? 1 : 2) * groups * pl.npk * pl.r * 4);
     dq_geometry(n, &pl.dq_waves, &pl.dq_chunks);
     pl.ds_parts = bw * pl.dq_chunks;
     // the resident dq kernel writes one partial per workgroup: at most this many per head and launch
@@ -728,9 +747,11 @@ static BwdPlan make_plan(int heads, int n, int bw, bool has_bias, bool has_mask,
     pl.off_dv = off;
     if (pl.n_chunks > 1) off += align256((size_t)pl.n_chunks * bw * heads * pl.npk * 32 * 4);
     pl.off_bias_t = off;
-    if (has_bias) off += align256((size_t)heads * pl.npk * pl.r * 2);
+    if (has_bias && !pl.key256) off += align256((size_t)heads * pl.npk * pl.r * 2);
     pl.off_mask_t = off;
-    if (has_mask) off += align256((size_t)n_windows * pl.npk * pl.r * 4);
+    if (has_mask && !pl.key256) off += align256((size_t)n_windows * pl.npk * pl.r * 4);
+    pl.off_tab = off;
+    if (pl.key256) off += align256((size_t)heads * (1 + (has_mask ? n_windows : 0)) * 256 * 256 * 4);
     pl.total = off;
     pl.smem = 0;   // the kernels use static LDS
     return pl;
@@ -853,14 +874,15 @@ static hipError_t launch_bwd_dt(BwdParams p, bool has_bias, int mask_dt, hipStre
         }
         return ef;
     }
+    p.tab = reinterpret_cast<const float*>(ws + pl.off_tab);
     const dim3 tgrid(pl.r / 32, (pl.npk + 31) / 32, 1);
-    if (has_bias) {
+    if (has_bias && !pl.key256) {
         dim3 gr(tgrid.x, tgrid.y, p.heads);
         hipLaunchKernelGGL(transpose_pad_kernel<E>, gr, dim3(256), 0, st, reinterpret_cast<const E*>(p.bias), p.bias_sh,
                            p.bias_sn, p.n, pl.npk, pl.r, (const uint8_t*)nullptr,
                            reinterpret_cast<E*>(const_cast<void*>(p.bias_t)), -INFINITY);
     }
-    if (mask_dt >= 0) {
+    if (mask_dt >= 0 && !pl.key256) {
         dim3 gr(tgrid.x, tgrid.y, p.n_windows);
         if (mask_dt == FWA2_F32)
             hipLaunchKernelGGL(transpose_pad_kernel<float>, gr, dim3(256), 0, st, reinterpret_cast<const float*>(p.mask),
@@ -874,7 +896,9 @@ static hipError_t launch_bwd_dt(BwdParams p, bool has_bias, int mask_dt, hipStre
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     int gr_out[2] = {pl.groups, pl.groups};
-    if (has_bias) {
+    if (pl.key256) {
+        e = launch_backward_key(p, DT, has_bias, mask_dt, st, pl.groups, gr_out);
+    } else if (has_bias) {
         if (mask_dt < 0) e = launch_nqb<DT, true, -1>(p, pl, st, gr_out);
         else if (mask_dt == FWA2_F32) e = launch_nqb<DT, true, FWA2_F32>(p, pl, st, gr_out);
         else e = launch_nqb<DT, true, DT>(p, pl, st, gr_out);

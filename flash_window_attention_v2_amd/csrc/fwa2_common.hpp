@@ -339,6 +339,8 @@ struct BwdParams {
     bool side_vec;       // rows of bias and mask (query-major) may be read with 16-byte loads, n % 8 == 0
     const void* bias_t;  // [H, NP, NQ] input dtype: bias transposed to key-major, zero padded
     const void* mask_t;  // [nW, NP, NQ] mask dtype: mask transposed to key-major, zero padded
+    const float* tab;    // table mode of the key-side kernel: (bias + mask) * log2e in accumulator order, slot h for
+                         // head h alone and slot heads + w * heads + h for window w with a live mask
 };
 
 }  // namespace fwa2
