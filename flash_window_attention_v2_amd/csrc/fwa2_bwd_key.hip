@@ -435,8 +435,9 @@ __global__ void __launch_bounds__(key256::NT) bwd_key_kernel(const BwdParams p) 
                 if (kt == KT - 1 && qb + 1 < NQB) load_rows(qb + 1);
                 // everything read ahead is on its way before this tile's elementwise work starts
                 asm volatile("" : "+v"(sacc[0]), "+v"(sacc[1]) :: "memory");
-                // right behind a batch of table loads: a portion of the next unit's rows, and delta for the dq kernel
-                if (kt == 0 && qb < 7) fetch_rows(b_next, qb);
+                // right behind the block's last batch of table loads (which then never queue behind rows requested
+                // from HBM a moment ago): a portion of the next unit's rows; and once per unit delta for the dq kernel
+                if (kt == KT - 1 && qb < 7) fetch_rows(b_next, qb);
                 if (kt == 2 && qb == 3 && have_next) after = unit_at(nxt.t + p.groups);      // scalar work, off the critical path
                 if (kt == 1 && qb == 0) {
                     const int r = 64 * wave + lane;
