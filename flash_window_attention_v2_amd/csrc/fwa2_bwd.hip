@@ -49,7 +49,8 @@ template <int DT, int NQB, int KT>
 struct WaveRegs {
     float dbacc[NQB][KT][8];
     f32x4 dvacc[KT][2], dkacc[KT][2];
-    typename Elem<DT>::V8 bk[KT], bv[KT];
+    typename Elem<kScoreDT>::V8 bk[KT];
+    typename Elem<DT>::V8 bv[KT];
 };
 
 // LDS views of one workgroup.  The arrays behind them are separate __shared__ variables with
@@ -60,8 +61,10 @@ template <int DT, int NQB>
 struct BwdLds {
     typedef typename Elem<DT>::E E;
     static constexpr int R = 32 * NQB;
-    E* Qs;          // q_hat * s * log2e, row-major [query][kRow]
-    E* Ks;          // k_hat, [key][kRow]
+    // q_hat and k_hat are kept in the score type of the forward kernel (fp16 also for bf16 inputs), so that the
+    // recomputed scores round as the forward's did and P sums to 1 against the forward's lse
+    typename Elem<kScoreDT>::E* Qs;   // q_hat * s * log2e, row-major [query][kRow]
+    typename Elem<kScoreDT>::E* Ks;   // k_hat, [key][kRow]
     E* dOs;         // dO, [query][kRow]
     float* nlse2;   // -lse * log2e   (-inf for padded / fully masked rows)
     float* ndelta;  // -rowsum(o * dO)
@@ -91,6 +94,8 @@ __device__ __forceinline__ void unit_blocks(BwdLds<DT, NQB>& L, WaveRegs<DT, NQB
     typedef typename Elem<DT>::E E;
     typedef typename Elem<DT>::V8 V8;
     typedef typename Elem<DT>::V4 V4;
+    typedef typename Elem<kScoreDT>::E SE;
+    typedef typename Elem<kScoreDT>::V8 SV8;
     typedef ME MV4 __attribute__((ext_vector_type(4)));
     constexpr int R = 32 * NQB;
     const int SS = BIG ? side_stride_big : R;    // row stride of the key-major side tables
@@ -117,12 +122,13 @@ __device__ __forceinline__ void unit_blocks(BwdLds<DT, NQB>& L, WaveRegs<DT, NQB
     // not with one key tile per wavefront, where the budget is 128 registers and any of it would spill)
     constexpr bool PF = KT == 2;              // the two rows
     constexpr bool PFI = !MASKED && KT == 2;  // and the accumulator inits
-    V8 aq0, ado0;
+    SV8 aq0;
+    V8 ado0;
     f32x4 nl0, nd0;
     auto fetch_first = [&](int qbn) __attribute__((always_inline)) {
         if (!PF) return;
         const int rowq = 32 * qbn + 8 * (l16 >> 2) + (l16 & 3);
-        aq0 = ld8<V8>(L.Qs + rowq * kRow + 8 * g);
+        aq0 = ld8<SV8>(L.Qs + rowq * kRow + 8 * g);
         ado0 = ld8<V8>(L.dOs + rowq * kRow + 8 * g);
         if (PFI) {
             nl0 = *reinterpret_cast<const f32x4*>(L.nlse2 + 32 * qbn + 8 * g);
@@ -147,18 +153,19 @@ __device__ __forceinline__ void unit_blocks(BwdLds<DT, NQB>& L, WaveRegs<DT, NQB
             // ---- phase A, one key tile at a time ----
 #pragma unroll
             for (int kt = 0; kt < KT; kt++) {
-                V8 p8, z8;
+                V8 p8;
+                SV8 z8;     // dZ in the score type: its partner in the dK product is q_hat
                 // k_hat of the lane's key is re-read per block: 4 registers less per key tile than keeping it
-                const V8 bk_now = ld8<V8>(L.Ks + (key0 + 16 * kt) * kRow + 8 * g);
+                const SV8 bk_now = ld8<SV8>(L.Ks + (key0 + 16 * kt) * kRow + 8 * g);
 #pragma unroll
                 for (int t = 0; t < 2; t++) {
                     const int rowq = 32 * qb + 8 * (l16 >> 2) + 4 * t + (l16 & 3);
-                    const V8 aq = (PF && t == 0) ? aq0 : ld8<V8>(L.Qs + rowq * kRow + 8 * g);
+                    const SV8 aq = (PF && t == 0) ? aq0 : ld8<SV8>(L.Qs + rowq * kRow + 8 * g);
                     const V8 ado = (PF && t == 0) ? ado0 : ld8<V8>(L.dOs + rowq * kRow + 8 * g);
                     // accumulator inits: -lse*log2e and -delta of this lane's 4 queries
                     const f32x4 nl = (PFI && t == 0) ? nl0 : *reinterpret_cast<const f32x4*>(L.nlse2 + q8 + 4 * t);
                     const f32x4 nd = (PFI && t == 0) ? nd0 : *reinterpret_cast<const f32x4*>(L.ndelta + q8 + 4 * t);
-                    f32x4 sacc = Elem<DT>::mfma16(aq, bk_now, nl);            // (S - lse) * log2e
+                    f32x4 sacc = Elem<kScoreDT>::mfma16(aq, bk_now, nl);      // (S - lse) * log2e
                     const f32x4 pacc = Elem<DT>::mfma16(ado, w.bv[kt], nd);   // dP - delta
                     if (HAS_BIAS) {   // padded key rows of bias_t hold -inf
 #pragma unroll
@@ -180,7 +187,7 @@ __device__ __forceinline__ void unit_blocks(BwdLds<DT, NQB>& L, WaveRegs<DT, NQB
                         const float dz = pj * pacc[i];
                         if (HAS_BIAS) w.dbacc[qb][kt][4 * t + i] += dz;
                         p8[4 * t + i] = (E)pj;
-                        z8[4 * t + i] = (E)dz;
+                        z8[4 * t + i] = (SE)dz;
                     }
                 }
                 if (kt == KT - 1 && qb + 1 < NQB) fetch_first(qb + 1);   // the first tile's operands are dead by now
@@ -190,8 +197,8 @@ __device__ __forceinline__ void unit_blocks(BwdLds<DT, NQB>& L, WaveRegs<DT, NQB
                     const int off = (q8 + (l16 >> 2)) * kRow + 8 * (l16 & 3) + 4 * dt;
                     const V8 a_do = lds_tr8<DT>(L.dOs + off, L.dOs + off + 4 * kRow);
                     w.dvacc[kt][dt] = Elem<DT>::mfma16(a_do, p8, w.dvacc[kt][dt]);
-                    const V8 a_q = lds_tr8<DT>(L.Qs + off, L.Qs + off + 4 * kRow);
-                    w.dkacc[kt][dt] = Elem<DT>::mfma16(a_q, z8, w.dkacc[kt][dt]);
+                    const SV8 a_q = lds_tr8<kScoreDT>(L.Qs + off, L.Qs + off + 4 * kRow);
+                    w.dkacc[kt][dt] = Elem<kScoreDT>::mfma16(a_q, z8, w.dkacc[kt][dt]);
                 }
             }
             fetch_side(qb + 1 < nqb ? qb + 1 : 0);
@@ -239,8 +246,11 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
     const int NPk_tot = BIG ? p.npk_tot : NPk;
     const int nqb = (N + 31) >> 5;         // query blocks of 32 that hold real rows
 
-    __shared__ __attribute__((aligned(16))) E lds_Qs[R * kRow];
-    __shared__ __attribute__((aligned(16))) E lds_Ks[R * kRow];
+    typedef typename Elem<kScoreDT>::E SE;
+    typedef typename Elem<kScoreDT>::V8 SV8;
+    typedef typename Elem<kScoreDT>::V4 SV4;
+    __shared__ __attribute__((aligned(16))) SE lds_Qs[R * kRow];
+    __shared__ __attribute__((aligned(16))) SE lds_Ks[R * kRow];
     __shared__ __attribute__((aligned(16))) E lds_dOs[R * kRow];
     __shared__ __attribute__((aligned(16))) float lds_nlse2[R];
     __shared__ __attribute__((aligned(16))) float lds_ndelta[R];
@@ -428,11 +438,11 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
                 for (int j = 0; j < 8; j++) { sq += xq[j] * xq[j]; sk += xk[j] * xk[j]; dl += xo[j] * xd[j]; }
                 sq = quad_add(sq); sk = quad_add(sk); dl = quad_add(dl);
                 const float iq = inv_norm(sq) * scale2, ik = inv_norm(sk);
-                V8 qn, kn;
+                SV8 qn, kn;
 #pragma unroll
-                for (int j = 0; j < 8; j++) { qn[j] = (E)(xq[j] * iq); kn[j] = (E)(xk[j] * ik); }
-                st8<V8>(L.Qs + r * kRow + dc, qn);
-                st8<V8>(L.Ks + r * kRow + dc, kn);
+                for (int j = 0; j < 8; j++) { qn[j] = (SE)(xq[j] * iq); kn[j] = (SE)(xk[j] * ik); }
+                st8<SV8>(L.Qs + r * kRow + dc, qn);
+                st8<SV8>(L.Ks + r * kRow + dc, kn);
                 st8<V8>(L.dOs + r * kRow + dc, do8);
                 if ((st & 3) == 0) {
                     L.ndelta[r] = -dl;
@@ -457,7 +467,7 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
         for (int kt = 0; kt < KT; kt++) w.bv[kt] = ld8<V8>(L.rawV + (key0 + 16 * kt) * 32 + 8 * g);
         __syncthreads();   // tiles complete; the landing area is free again
 #pragma unroll
-        for (int kt = 0; kt < KT; kt++) w.bk[kt] = ld8<V8>(L.Ks + (key0 + 16 * kt) * kRow + 8 * g);
+        for (int kt = 0; kt < KT; kt++) w.bk[kt] = ld8<SV8>(L.Ks + (key0 + 16 * kt) * kRow + 8 * g);
 #pragma unroll
         for (int kt = 0; kt < KT; kt++)
 #pragma unroll
@@ -492,7 +502,7 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
             float dot = 0.f;
 #pragma unroll
             for (int dt = 0; dt < 2; dt++) {
-                const V4 k4 = *reinterpret_cast<const V4*>(L.Ks + key * kRow + 8 * g + 4 * dt);
+                const SV4 k4 = *reinterpret_cast<const SV4*>(L.Ks + key * kRow + 8 * g + 4 * dt);
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     x[4 * dt + i] = (float)k4[i];

@@ -28,12 +28,16 @@ __global__ void __launch_bounds__(512) bwd_dq_kernel(const BwdParams p) {
     typedef typename Elem<DT>::V8 V8;
     typedef typename Elem<DT>::V4 V4;
     typedef typename MaskElem<DT, MASK_DT>::E ME;
+    // q_hat and k_hat in the score type of the forward kernel (fp16 also for bf16 inputs): the recomputed scores
+    // then round as the forward's did; dZ takes the same type, its partner in the dQ product being k_hat
+    typedef typename Elem<kScoreDT>::E SE;
+    typedef typename Elem<kScoreDT>::V8 SV8;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     const int N = p.n;
     const int chunk_rows = (min(N, kKeyChunk) + 63) & ~63;
-    E* Ks = reinterpret_cast<E*>(smem_raw);
-    E* Vs = Ks + chunk_rows * kLdsStride;
+    SE* Ks = reinterpret_cast<SE*>(smem_raw);
+    E* Vs = reinterpret_cast<E*>(Ks + chunk_rows * kLdsStride);
     float* red = reinterpret_cast<float*>(Vs + chunk_rows * kLdsStride);   // [8]
 
     const int tid = threadIdx.x;
@@ -73,7 +77,8 @@ __global__ void __launch_bounds__(512) bwd_dq_kernel(const BwdParams p) {
     const bool wave_live = q0 < N;
 
     // ---- per-query operands: q_hat * s * log2e, dO (both as B operands), delta, lse ----
-    V8 bq0 = zero8<V8>(), bq1 = zero8<V8>(), bd0 = zero8<V8>(), bd1 = zero8<V8>();
+    SV8 bq0 = zero8<SV8>(), bq1 = zero8<SV8>();
+    V8 bd0 = zero8<V8>(), bd1 = zero8<V8>();
     float nlse2 = -INFINITY, ndelta = 0.f;
     if (wave_live) {
         V8 a = zero8<V8>(), c = zero8<V8>(), o0 = zero8<V8>(), o1 = zero8<V8>();
@@ -100,7 +105,7 @@ __global__ void __launch_bounds__(512) bwd_dq_kernel(const BwdParams p) {
         ndelta = -xor32_add(dl);
         const float sc = scale2 * inv_norm(ss);
 #pragma unroll
-        for (int j = 0; j < 8; j++) { bq0[j] = (E)(xa[j] * sc); bq1[j] = (E)(xc[j] * sc); }
+        for (int j = 0; j < 8; j++) { bq0[j] = (SE)(xa[j] * sc); bq1[j] = (SE)(xc[j] * sc); }
     }
 
     const E* bias_row = nullptr;
@@ -136,10 +141,10 @@ __global__ void __launch_bounds__(512) bwd_dq_kernel(const BwdParams p) {
             for (int j = 0; j < 8; j++) ss += x[j] * x[j];
             ss = quad_add(ss);
             const float inv = inv_norm(ss);
-            V8 kn;
+            SV8 kn;
 #pragma unroll
-            for (int j = 0; j < 8; j++) kn[j] = (E)(x[j] * inv);
-            st8<V8>(Ks + r * kLdsStride + dch, kn);
+            for (int j = 0; j < 8; j++) kn[j] = (SE)(x[j] * inv);
+            st8<SV8>(Ks + r * kLdsStride + dch, kn);
             st8<V8>(Vs + r * kLdsStride + dch, vv);
         }
         __syncthreads();
@@ -151,13 +156,13 @@ __global__ void __launch_bounds__(512) bwd_dq_kernel(const BwdParams p) {
             const int kbase = c0 + kt * 32;
             // register i <-> key kbase + 16(i/8) + 8hf + i%8
             const int row = (kt * 32 + swap_bits23(col)) * kLdsStride + 8 * hf;
-            const V8 k0 = ld8<V8>(Ks + row), k1 = ld8<V8>(Ks + row + 16);
+            const SV8 k0 = ld8<SV8>(Ks + row), k1 = ld8<SV8>(Ks + row + 16);
             const V8 v0 = ld8<V8>(Vs + row), v1 = ld8<V8>(Vs + row + 16);
             f32x16 sacc, pacc;
 #pragma unroll
             for (int i = 0; i < 16; i++) { sacc[i] = nlse2; pacc[i] = ndelta; }
-            sacc = Elem<DT>::mfma32(k0, bq0, sacc);
-            sacc = Elem<DT>::mfma32(k1, bq1, sacc);      // (S - lse) * log2e
+            sacc = Elem<kScoreDT>::mfma32(k0, bq0, sacc);
+            sacc = Elem<kScoreDT>::mfma32(k1, bq1, sacc);      // (S - lse) * log2e
             pacc = Elem<DT>::mfma32(v0, bd0, pacc);
             pacc = Elem<DT>::mfma32(v1, bd1, pacc);      // dP - delta
             if (HAS_BIAS) {
@@ -190,12 +195,12 @@ __global__ void __launch_bounds__(512) bwd_dq_kernel(const BwdParams p) {
             // ---- dZ^T = P^T (dP^T - delta); dQ_hat^T += K_hat^T dZ^T, 16 keys per MFMA ----
 #pragma unroll
             for (int mm = 0; mm < 2; mm++) {
-                V8 bz;
+                SV8 bz;
 #pragma unroll
-                for (int j = 0; j < 8; j++) bz[j] = (E)(fast_exp2(sacc[8 * mm + j]) * pacc[8 * mm + j]);
-                const E* klo = Ks + (kt * 32 + 16 * mm + 8 * hf + (li >> 2)) * kLdsStride + 16 * blk1 + 4 * (li & 3);
-                const V8 ak = lds_tr8<DT>(klo, klo + 4 * kLdsStride);
-                dqacc = Elem<DT>::mfma32(ak, bz, dqacc);
+                for (int j = 0; j < 8; j++) bz[j] = (SE)(fast_exp2(sacc[8 * mm + j]) * pacc[8 * mm + j]);
+                const SE* klo = Ks + (kt * 32 + 16 * mm + 8 * hf + (li >> 2)) * kLdsStride + 16 * blk1 + 4 * (li & 3);
+                const SV8 ak = lds_tr8<kScoreDT>(klo, klo + 4 * kLdsStride);
+                dqacc = Elem<kScoreDT>::mfma32(ak, bz, dqacc);
             }
         }
     }

@@ -11,20 +11,61 @@ from .kernels import (_DTYPES, _check_inputs, _describe, _flags_for, _flash_attn
                       _kernel_ready, _on_device, _rows_16b_aligned, _set_t4, mask_window_flags, tensor_version)
 
 
+def _scale_argument(logit_scale, device):
+    """(tensor for the saved-tensor slot, scale_type) as the reference derives them
+    (flash_window_attention_v2.py:9-17)."""
+    if logit_scale is not None:
+        assert isinstance(logit_scale, torch.Tensor), \
+            "Make sure logit_scale is a tensor if defined in the paramaters."
+        return (logit_scale if logit_scale.is_contiguous() else logit_scale.contiguous()), "tensor"
+    # placeholder for the saved-tensor slot (the reference keeps 1/sqrt(d) there); the kernels derive the
+    # default scale from head_dim, and filling a device scalar from the host would synchronise and break
+    # stream capture
+    return torch.empty((), device=device), "scalar"
+
+
+def _packed_forward(q, k, v, units, logit_scale, bias, mask, scale_type, window_map=None):
+    """Forward of the two packed Functions: q, k, v are [B, H, L, d] views of one qkv buffer, `units` the
+    (number of windows, tokens per window) the library sees.  Returns out [B, L, H, d], lse and the mask's
+    per-window flags (kept for backward)."""
+    b, heads, length, d = q.shape
+    bw, n = units
+    lse = torch.empty((bw, heads, (n + 63) // 64 * 64), device=q.device, dtype=torch.float32)
+    out = torch.empty((b, length, heads, d), device=q.device, dtype=q.dtype)
+    mask_live = mask_window_flags(mask) if mask is not None else None
+    p = _describe(q, k, v, out.transpose(1, 2), lse, logit_scale, bias, mask, mask_live, scale_type, window_map)
+    with _on_device(q.device) as stream:
+        p.stream = stream
+        _abi.check(_abi.load().fwa2_forward(p), "fwa2_forward")
+    return out, lse, mask_live
+
+
+def _packed_backward(qkv, q, k, v, out, lse, logit_scale, bias, mask, mask_live, scale_type, do, window_map=None):
+    """Backward of the two packed Functions: dq, dk, dv land in one buffer shaped like qkv."""
+    dqkv = torch.empty_like(qkv)
+    dq, dk, dv = (dqkv[:, :, i].transpose(1, 2) for i in range(3))
+    dscale = torch.empty_like(logit_scale, memory_format=torch.contiguous_format) if scale_type == "tensor" else None
+    db = torch.empty_like(bias, memory_format=torch.contiguous_format) if bias is not None else None
+    lib = _abi.load()
+    p = _describe(q, k, v, out.transpose(1, 2), lse, logit_scale, bias, mask, mask_live, scale_type, window_map)
+    _set_t4(p.d_o, do); _set_t4(p.dq, dq); _set_t4(p.dk, dk); _set_t4(p.dv, dv)
+    if db is not None:
+        p.dbias = db.data_ptr()
+    if dscale is not None:
+        p.dscale = dscale.data_ptr()
+    with _on_device(qkv.device) as stream:
+        need = lib.fwa2_backward_workspace_bytes(p)
+        ws = torch.empty(max(need, 1), dtype=torch.uint8, device=qkv.device)
+        p.workspace, p.workspace_bytes = ws.data_ptr(), need
+        p.stream = stream
+        _abi.check(lib.fwa2_backward(p), "fwa2_backward")
+    return dqkv, dscale, db
+
+
 class FlashWindowAttentionV2(torch.autograd.Function):
     @staticmethod
     def forward(ctx, q, k, v, logit_scale=None, bias=None, mask=None):
-        if logit_scale is not None:
-            assert isinstance(logit_scale, torch.Tensor), \
-                "Make sure logit_scale is a tensor if defined in the paramaters."
-            scale_type = "tensor"
-            logit_scale = logit_scale if logit_scale.stride(-1) == 1 else logit_scale.contiguous()
-        else:
-            scale_type = "scalar"
-            # placeholder for the saved-tensor slot (the reference keeps 1/sqrt(d) there, fn.py:15-17); the
-            # kernels derive the default scale from head_dim, and filling a device scalar from the host
-            # would synchronise and break stream capture
-            logit_scale = torch.empty((), device=q.device)
+        logit_scale, scale_type = _scale_argument(logit_scale, q.device)
 
         # unit inner stride is the reference's requirement (flash_window_attention_v2.py:20), 16-byte-aligned
         # rows this library's: copy only when either fails
@@ -64,17 +105,7 @@ class FlashWindowAttentionV2QKVPacked(torch.autograd.Function):
         if not (_rows_16b_aligned(qkv) and qkv.is_contiguous()):
             qkv = qkv.contiguous()
         q, k, v = (qkv[:, :, i].transpose(1, 2) for i in range(3))       # [BW, H, N, d] views
-        if logit_scale is not None:
-            assert isinstance(logit_scale, torch.Tensor), \
-                "Make sure logit_scale is a tensor if defined in the paramaters."
-            scale_type = "tensor"
-            logit_scale = logit_scale.contiguous()
-        else:
-            scale_type = "scalar"
-            # placeholder for the saved-tensor slot (the reference keeps 1/sqrt(d) there, fn.py:15-17); the
-            # kernels derive the default scale from head_dim, and filling a device scalar from the host
-            # would synchronise and break stream capture
-            logit_scale = torch.empty((), device=q.device)
+        logit_scale, scale_type = _scale_argument(logit_scale, q.device)
         _check_inputs(q, k, v, logit_scale, bias, mask, scale_type)
         if bias is not None and bias.stride(-1) != 1:
             bias = bias.contiguous()
@@ -82,14 +113,7 @@ class FlashWindowAttentionV2QKVPacked(torch.autograd.Function):
             mask = mask.contiguous()
 
         bw, heads, n, d = q.shape
-        lib = _abi.load()
-        lse = torch.empty((bw, heads, (n + 63) // 64 * 64), device=q.device, dtype=torch.float32)
-        out = torch.empty((bw, n, heads, d), device=q.device, dtype=q.dtype)
-        mask_live = mask_window_flags(mask) if mask is not None else None
-        p = _describe(q, k, v, out.transpose(1, 2), lse, logit_scale, bias, mask, mask_live, scale_type)
-        with _on_device(q.device) as stream:
-            p.stream = stream
-            _abi.check(lib.fwa2_forward(p), "fwa2_forward")
+        out, lse, mask_live = _packed_forward(q, k, v, (bw, n), logit_scale, bias, mask, scale_type)
 
         ctx.save_for_backward(qkv, out, lse, logit_scale, bias, mask)
         ctx.scale_type = scale_type
@@ -104,24 +128,7 @@ class FlashWindowAttentionV2QKVPacked(torch.autograd.Function):
         do = dout.transpose(1, 2)                                          # [BW, H, N, d] view
         if not _rows_16b_aligned(do):
             do = do.contiguous()
-        dqkv = torch.empty_like(qkv)
-        dq, dk, dv = (dqkv[:, :, i].transpose(1, 2) for i in range(3))
-        dscale = torch.empty_like(logit_scale, memory_format=torch.contiguous_format) if scale_type == "tensor" else None
-        db = torch.empty_like(bias, memory_format=torch.contiguous_format) if bias is not None else None
-
-        lib = _abi.load()
-        p = _describe(q, k, v, out.transpose(1, 2), lse, logit_scale, bias, mask, ctx.mask_live, scale_type)
-        _set_t4(p.d_o, do); _set_t4(p.dq, dq); _set_t4(p.dk, dk); _set_t4(p.dv, dv)
-        if db is not None:
-            p.dbias = db.data_ptr()
-        if dscale is not None:
-            p.dscale = dscale.data_ptr()
-        with _on_device(qkv.device) as stream:
-            need = lib.fwa2_backward_workspace_bytes(p)
-            ws = torch.empty(max(need, 1), dtype=torch.uint8, device=qkv.device)
-            p.workspace, p.workspace_bytes = ws.data_ptr(), need
-            p.stream = stream
-            _abi.check(lib.fwa2_backward(p), "fwa2_backward")
+        dqkv, dscale, db = _packed_backward(qkv, q, k, v, out, lse, logit_scale, bias, mask, ctx.mask_live, scale_type, do)
         return dqkv, dscale, db, None
 
 
@@ -146,17 +153,7 @@ class FlashWindowAttentionV2Grid(torch.autograd.Function):
         if not (_rows_16b_aligned(qkv) and qkv.is_contiguous()):
             qkv = qkv.contiguous()
         q, k, v = (qkv[:, :, i].transpose(1, 2) for i in range(3))       # [B, H, L, d] views
-        if logit_scale is not None:
-            assert isinstance(logit_scale, torch.Tensor), \
-                "Make sure logit_scale is a tensor if defined in the paramaters."
-            scale_type = "tensor"
-            logit_scale = logit_scale.contiguous()
-        else:
-            scale_type = "scalar"
-            # placeholder for the saved-tensor slot (the reference keeps 1/sqrt(d) there, fn.py:15-17); the
-            # kernels derive the default scale from head_dim, and filling a device scalar from the host
-            # would synchronise and break stream capture
-            logit_scale = torch.empty((), device=q.device)
+        logit_scale, scale_type = _scale_argument(logit_scale, q.device)
         b, heads, length, d = q.shape
         n, nw = wh * ww, (gh // wh) * (gw // ww)
         assert d <= 128, "FlashAttention only support head dimensions up to 128"
@@ -174,15 +171,8 @@ class FlashWindowAttentionV2Grid(torch.autograd.Function):
             if mask.stride(-1) != 1:
                 mask = mask.contiguous()
 
-        lib = _abi.load()
-        lse = torch.empty((b * nw, heads, (n + 63) // 64 * 64), device=q.device, dtype=torch.float32)
-        out = torch.empty((b, length, heads, d), device=q.device, dtype=q.dtype)
-        mask_live = mask_window_flags(mask) if mask is not None else None
         window_map = ((gh, gw), (wh, ww), (sh % gh, sw % gw))
-        p = _describe(q, k, v, out.transpose(1, 2), lse, logit_scale, bias, mask, mask_live, scale_type, window_map)
-        with _on_device(q.device) as stream:
-            p.stream = stream
-            _abi.check(lib.fwa2_forward(p), "fwa2_forward")
+        out, lse, mask_live = _packed_forward(q, k, v, (b * nw, n), logit_scale, bias, mask, scale_type, window_map)
 
         ctx.save_for_backward(qkv, out, lse, logit_scale, bias, mask)
         ctx.scale_type = scale_type
@@ -198,25 +188,8 @@ class FlashWindowAttentionV2Grid(torch.autograd.Function):
         do = dout.transpose(1, 2)                                          # [B, H, L, d] view
         if not _rows_16b_aligned(do):
             do = do.contiguous()
-        dqkv = torch.empty_like(qkv)
-        dq, dk, dv = (dqkv[:, :, i].transpose(1, 2) for i in range(3))
-        dscale = torch.empty_like(logit_scale, memory_format=torch.contiguous_format) if scale_type == "tensor" else None
-        db = torch.empty_like(bias, memory_format=torch.contiguous_format) if bias is not None else None
-
-        lib = _abi.load()
-        p = _describe(q, k, v, out.transpose(1, 2), lse, logit_scale, bias, mask, ctx.mask_live, scale_type,
-                      ctx.window_map)
-        _set_t4(p.d_o, do); _set_t4(p.dq, dq); _set_t4(p.dk, dk); _set_t4(p.dv, dv)
-        if db is not None:
-            p.dbias = db.data_ptr()
-        if dscale is not None:
-            p.dscale = dscale.data_ptr()
-        with _on_device(qkv.device) as stream:
-            need = lib.fwa2_backward_workspace_bytes(p)
-            ws = torch.empty(max(need, 1), dtype=torch.uint8, device=qkv.device)
-            p.workspace, p.workspace_bytes = ws.data_ptr(), need
-            p.stream = stream
-            _abi.check(lib.fwa2_backward(p), "fwa2_backward")
+        dqkv, dscale, db = _packed_backward(qkv, q, k, v, out, lse, logit_scale, bias, mask, ctx.mask_live, scale_type, do,
+                                            ctx.window_map)
         return dqkv, None, None, None, dscale, db, None
 
 

@@ -74,11 +74,16 @@ def tensor_version(t):
 
 def mask_window_flags(mask):
     """uint8[nW]: 1 where a window's mask has a non-zero entry (device tensor).
-    Cached on the mask tensor object and refreshed if the tensor is modified in place (a mask created under
-    torch.inference_mode tracks no modifications: edit such a mask by making a new tensor)."""
-    cached = getattr(mask, "_fwa2_live", None)
+    Cached on the mask tensor object, keyed by its storage address and in-place modification counter, so a
+    mask edited in place or re-pointed at other memory (`mask.data = ...`) is scanned again.  Two cases are
+    never cached and scan on every call: a mask created under torch.inference_mode, which tracks no
+    modifications, and a first scan made while a graph is being captured, whose flags live in the graph's
+    own memory pool and must not be handed to eager calls (scan once eagerly before capturing to avoid the
+    extra node)."""
     version = tensor_version(mask)
-    if cached is not None and cached[0] == version and cached[1].device == mask.device:
+    key = (version, mask.data_ptr(), mask.device)
+    cached = getattr(mask, "_fwa2_live", None)
+    if version is not None and cached is not None and cached[0] == key:
         return cached[1]
     lib = _abi.load()
     live = torch.empty(mask.shape[0], dtype=torch.uint8, device=mask.device)
@@ -86,10 +91,11 @@ def mask_window_flags(mask):
         st = lib.fwa2_mask_scan(mask.data_ptr(), _DTYPES[mask.dtype], mask.shape[0], mask.shape[1], mask.stride(0),
                                 mask.stride(1), live.data_ptr(), stream)
     _abi.check(st, "fwa2_mask_scan")
-    try:
-        mask._fwa2_live = (version, live)
-    except Exception:
-        pass
+    if version is not None and not torch.cuda.is_current_stream_capturing():
+        try:
+            mask._fwa2_live = (key, live)
+        except Exception:
+            pass
     return live
 
 

@@ -190,3 +190,22 @@ def test_static_scratch_backward_refuses_oversize_without_a_device(lib):
     assert "static buffer holds" in msg and str(_abi.STATIC_SCRATCH_BYTES) in msg
     header = open(os.path.join(ROOT, "include", "fwa2.h")).read()
     assert re.search(r"#define FWA2_STATIC_SCRATCH_BYTES \(\(size_t\)64 << 20\)", header) and _abi.STATIC_SCRATCH_BYTES == 64 << 20
+
+
+def test_problem_filled_the_way_a_binding_fills_it(lib):
+    """A struct built by keyword, as a ctypes binding of the reference's forward call site would build it
+    (flash_win_attn_v2/flash_window_attention_v2.py:22-24), passes validation with the version the library
+    reports and is refused with any other."""
+    bw, h, n, d, nw = 8, 3, 64, 32, 4
+    t4 = lambda: _abi.Tensor4(0x10000, h * n * d, n * d, d)
+    t3 = lambda: _abi.Tensor3(0x10000, n * n, n)
+    fields = dict(struct_bytes=ctypes.sizeof(_abi.Problem), dtype=_abi.BF16, mask_dtype=_abi.BF16,
+                  scale_kind=_abi.SCALE_TENSOR, bw=bw, heads=h, n=n, head_dim=d, n_windows=nw,
+                  q=t4(), k=t4(), v=t4(), o=t4(), logit_scale=0x10000, bias=t3(), mask=t3(), lse=0x10000,
+                  lse_stride_bw=h * n, lse_stride_h=n, stream=None)
+    p = _abi.Problem(abi_version=lib.fwa2_abi_version(), **fields)
+    assert lib.fwa2_abi_version() == 2
+    assert lib.fwa2_validate(ctypes.byref(p), 0) == _abi.OK, lib.fwa2_last_error()
+    p = _abi.Problem(abi_version=1, **fields)
+    assert lib.fwa2_validate(ctypes.byref(p), 0) == _abi.ERR_INVALID_ARGUMENT
+    assert b"abi 1, library 456 bytes / abi 2" in lib.fwa2_last_error()

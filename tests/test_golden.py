@@ -70,14 +70,19 @@ def test_kernels_against_fixture(case):
             t[name].requires_grad_(True)
     o = flash_win_attn_v2_func(t["q"], t["k"], t["v"], t.get("logit_scale"), t.get("bias"), t.get("mask"))
     o.backward(t["do"])
-    # A head past the clamp runs at s = 100, where rounding q_hat.k_hat to the input dtype moves the
-    # logits by up to 100 * 2^-9 (bf16): such heads are held to a loose sanity bound, the others to
-    # the stated tolerances.  The clamped head's logit-scale gradient must be exactly zero.
+    # A head past the clamp runs at s = 100, where rounding q_hat.k_hat moves the logits by up to
+    # 100 * 2^-9 in bf16: such a head is held to what the eager classic path reaches in the same dtype on the
+    # same inputs, the others to the stated tolerances.  The clamped head's logit-scale gradient must be exactly zero.
     heads = t["q"].shape[1]
     clamped = [bool(t["logit_scale"][h] > 4.6051) for h in range(heads)] if "logit_scale" in t else [False] * heads
-    o_err = (o.detach().float().cpu() - torch.from_numpy(fx["o"])).abs()
+    cpu = {k: v.detach().cpu() for k, v in t.items()}
+    eager = classic_fwd_bwd(cpu["q"], cpu["k"], cpu["v"], cpu.get("logit_scale"), cpu.get("bias"), cpu.get("mask"), cpu["do"],
+                            dtype=dtype)
+    o_ref = torch.from_numpy(fx["o"])
+    o_err = (o.detach().float().cpu() - o_ref).abs()
+    eager_err = (eager["o"].float() - o_ref).abs()
     for h in range(heads):
-        assert float(o_err[:, h].max()) <= (0.5 if clamped[h] else tol_o), f"o head {h}"
+        assert float(o_err[:, h].max()) <= (float(eager_err[:, h].max()) if clamped[h] else tol_o), f"o head {h}"
     for gname, tname in (("dq", "q"), ("dk", "k"), ("dv", "v"), ("dbias", "bias"), ("dscale", "logit_scale")):
         if gname not in fx:
             continue
@@ -90,4 +95,7 @@ def test_kernels_against_fixture(case):
                 assert float(g.abs().max()) == 0.0 and float(r.abs().max()) == 0.0
                 continue
             rel = float((g - r).abs().max() / r.abs().max())
-            assert rel <= (0.5 if clamped[h] else tol_g), f"{gname} head {h}: {rel}"
+            bound = tol_g
+            if clamped[h]:
+                bound = float((eager[gname].float().select(axis, h) - r).abs().max() / r.abs().max())
+            assert rel <= bound, f"{gname} head {h}: {rel} (bound {bound})"

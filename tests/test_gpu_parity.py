@@ -117,13 +117,23 @@ def test_more_windows_than_the_flag_cache_and_no_flags(monkeypatch):
     inp["mask"] = mask.to(torch.bfloat16)
     _run_and_check(inp, torch.bfloat16, tag="1040 windows")
 
-    # (b) a caller that never scanned the mask: the flag pointer stays NULL
-    import flash_window_attention_v2_amd.flash_window_attention_v2 as fw
-    monkeypatch.setattr(fw, "mask_window_flags", lambda mask: None)
-    for n_, res, win, shift in ((64, 32, 8, 4), (256, 64, 16, 8)):
+    # (b) a caller that never scanned the mask: the flag pointer stays NULL in every problem the launchers describe
+    from flash_window_attention_v2_amd import kernels
+    monkeypatch.setattr(kernels, "_flags_for", lambda mask: None)
+    described = []
+    describe = kernels._describe
+
+    def spy(*args, **kwargs):
+        prob = describe(*args, **kwargs)
+        described.append(prob.mask_live)
+        return prob
+
+    monkeypatch.setattr(kernels, "_describe", spy)
+    for n_, res, win, shift in ((64, 32, 8, 4), (256, 64, 16, 8), (576, 48, 24, 12)):
         inp = make_inputs(batch=2, n_windows=(res // win) ** 2, heads=3, n=n_, dtype=torch.bfloat16, seed=23,
                           resolution=res, window=win, shift=shift)
         _run_and_check(inp, torch.bfloat16, tag=f"no flags N={n_}")
+    assert len(described) == 6 and all(ptr is None for ptr in described), described
 
 
 @pytest.mark.parametrize("n", [1, 7, 17, 31, 33, 47, 63, 65, 100, 129, 200, 255])
@@ -178,19 +188,29 @@ def test_fully_masked_rows_and_clamped_scale():
         assert torch.isfinite(dev[t].grad).all(), t
     assert float(dev["logit_scale"].grad[0]) == 0.0 and float(dev["logit_scale"].grad[1]) != 0.0
     # against the float64 oracle, which shares the zero-row convention.  Head 1 (s = 10) is held to
-    # the benchmark tolerances; head 0 runs at the clamp, s = 100, where the rounding of the
-    # normalised vectors is amplified ten times more, so it only gets a sanity bound.
+    # the benchmark tolerances.  Head 0 runs at the clamp, s = 100, where the rounding of the normalised
+    # vectors is amplified ten times more: it is held to what the eager classic path reaches in the same
+    # dtype on the same inputs.  The eager path turns the fully masked row into NaN, so its error is
+    # measured on the units of window 0 (even b), which have no such row, and bounds the others too.
     f64 = lambda x: None if x is None else x.double().numpy()
     oo, lse = wa.forward(f64(inp["q"]), f64(inp["k"]), f64(inp["v"]), f64(inp["logit_scale"]), f64(inp["bias"]),
                          f64(inp["mask"]))
-    err = np.abs(o.detach().float().cpu().numpy() - oo)
-    assert float(err[:, 1].max()) <= 2e-2 and float(err[:, 0].max()) <= 2e-1
     gr = wa.backward(f64(inp["q"]), f64(inp["k"]), f64(inp["v"]), f64(inp["do"]), f64(inp["logit_scale"]),
                      f64(inp["bias"]), f64(inp["mask"]))
+    even = {k: (v[0::2] if k in ("q", "k", "v", "do") else v) for k, v in inp.items()}
+    even["mask"] = inp["mask"][:1]
+    eager = classic_fwd_bwd(even["q"], even["k"], even["v"], even["logit_scale"], even["bias"], even["mask"], even["do"],
+                            dtype=dtype)
+    err = np.abs(o.detach().float().cpu().numpy() - oo)
+    eager_o = float(np.abs(eager["o"].float().numpy()[:, 0] - oo[0::2, 0]).max())
+    assert float(err[:, 1].max()) <= 2e-2
+    assert float(err[0::2, 0].max()) <= eager_o and float(err[1::2, 0].max()) <= 1.5 * eager_o, (err[:, 0].max(), eager_o)
     for gname, tname in (("dq", "q"), ("dk", "k"), ("dv", "v")):
         ref = torch.from_numpy(gr[gname])
         assert _rel(dev[tname].grad[:, 1], ref[:, 1]) <= 5e-2, gname
-        assert _rel(dev[tname].grad[:, 0], ref[:, 0]) <= 5e-1, gname
+        eager_g = _rel(eager[gname][:, 0], ref[0::2, 0])
+        assert _rel(dev[tname].grad[0::2, 0], ref[0::2, 0]) <= eager_g, (gname, eager_g)
+        assert _rel(dev[tname].grad[1::2, 0], ref[1::2, 0]) <= 1.5 * eager_g, (gname, eager_g)
     assert _rel(dev["bias"].grad[1], torch.from_numpy(gr["dbias"])[1]) <= 5e-2
     # dlogit_scale is a signed sum of BW*N^2 terms that nearly cancels at this tiny size: hold the
     # error against the larger of |ref| and 2 % of the sum of absolute terms
@@ -346,7 +366,7 @@ def test_recompute_under_checkpoint():
     assert _rel(dev["q"].grad, ref["dq"]) <= 5e-2 and _rel(dev["bias"].grad, ref["dbias"]) <= 5e-2
 
 
-@pytest.mark.parametrize("n,dtype", [(576, torch.bfloat16), (1024, torch.bfloat16), (320, torch.float16),
+@pytest.mark.parametrize("n,dtype", [(576, torch.bfloat16), (1024, torch.bfloat16), (1024, torch.float16), (320, torch.float16),
                                      (784, torch.bfloat16), (530, torch.float16)])
 def test_large_windows(n, dtype):
     """N = 576 and 1024 (windows 24 and 32 of the sweep), 784 = 28 x 28 and the ragged 320 and 530: several
@@ -408,14 +428,28 @@ def test_full_benchmark_shapes(cfg):
     assert float(cosq.max()) < 2e-2 and float(cosk.max()) < 2e-2
     db = dev["bias"].grad.float()
     assert float(db.sum(-1).abs().max()) <= 2e-2 * float(db.abs().max()) * math.sqrt(db.shape[-1])
-    # no worse than the eager classic path run in the same low precision (proxy for the reference's claim)
-    with torch.no_grad():
-        sl = slice(0, 256)
-        low = win_attention_classic(plain["q"][sl], plain["k"][sl], plain["v"][sl], plain["logit_scale"], plain["bias"],
-                                    plain["mask"])
-        err_low = float((low.float() - ref["o"][sl]).abs().max())
-        err_hip = float((o.detach()[sl].float() - ref["o"][sl]).abs().max())
-    assert err_hip <= max(err_low, 2e-2)
+    # No worse than the eager classic path run in the same low precision, output and every gradient: the
+    # reference states its error as "the same level as torch.compile" of that path (README.md:28) and gives no
+    # number.  Both are run on the first 4 images (256 units) and held against the fp32 path on the same units.
+    sl = slice(0, 256)
+    part = {k: (v[sl] if k in ("q", "k", "v", "do") else v) for k, v in plain.items()}
+    ref_s = classic_fwd_bwd(part["q"], part["k"], part["v"], part["logit_scale"], part["bias"], part["mask"], part["do"])
+    low = classic_fwd_bwd(part["q"], part["k"], part["v"], part["logit_scale"], part["bias"], part["mask"], part["do"],
+                          dtype=dtype)
+    dev_s = {k: (None if v is None else v.clone()) for k, v in part.items()}
+    for name in ("q", "k", "v", "bias", "logit_scale"):
+        dev_s[name].requires_grad_(True)
+    o_s = _func()(dev_s["q"], dev_s["k"], dev_s["v"], dev_s["logit_scale"], dev_s["bias"], dev_s["mask"])
+    o_s.backward(dev_s["do"])
+    rows = [("o", float((o_s.detach().float() - ref_s["o"]).abs().max()), float((low["o"].float() - ref_s["o"]).abs().max()))]
+    for gname, tname in GRADS:
+        scale = float(ref_s[gname].abs().max())
+        rows.append((gname, float((dev_s[tname].grad.float() - ref_s[gname]).abs().max()) / scale,
+                     float((low[gname].float() - ref_s[gname]).abs().max()) / scale))
+    print(f"\n{cfg}: error against fp32 classic, this library / eager classic in bf16: " +
+          ", ".join(f"{n} {a:.2e} / {b:.2e}" for n, a, b in rows))
+    for name, err_hip, err_low in rows:
+        assert err_hip <= err_low, f"{cfg} {name}: {err_hip} against {err_low} of the eager path"
 
 
 def test_launchers_under_the_reference_names():
@@ -479,3 +513,36 @@ def test_empty_batch():
         assert float(a.abs().sum()) == 0.0
         if b is not None:
             assert torch.equal(a.float(), b.float())
+
+
+@pytest.mark.parametrize("n", [64, 256])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_heads_at_the_clamp_are_no_worse_than_eager(n, dtype):
+    """Trained Swin V2 heads reach the clamp (s = 100), where the rounding of the normalised vectors moves a
+    logit by up to 100 * 2^-9 in bf16.  The kernels score from fp16 q_hat / k_hat in the forward and in both
+    backward kernels, so they must not lose to the eager classic path run in the same dtype: output and every
+    gradient, against the fp32 classic path on the same inputs.  Head 0 sits past the clamp (its logit-scale
+    gradient is exactly zero), head 1 just below it."""
+    win = 8 if n == 64 else 16
+    inp = make_inputs(batch=2, n_windows=4, heads=2, n=n, dtype=dtype, seed=40 + n, resolution=2 * win, window=win,
+                      shift=win // 2)
+    inp["logit_scale"] = torch.tensor([5.0, 4.59375]).view(2, 1, 1).to(dtype)
+    ref = classic_fwd_bwd(inp["q"], inp["k"], inp["v"], inp["logit_scale"], inp["bias"], inp["mask"], inp["do"])
+    low = classic_fwd_bwd(inp["q"], inp["k"], inp["v"], inp["logit_scale"], inp["bias"], inp["mask"], inp["do"], dtype=dtype)
+    dev = _to_dev(inp)
+    o = _func()(dev["q"], dev["k"], dev["v"], dev["logit_scale"], dev["bias"], dev["mask"])
+    o.backward(dev["do"])
+    torch.cuda.synchronize()
+    assert float(dev["logit_scale"].grad[0]) == 0.0 and float(dev["logit_scale"].grad[1]) != 0.0
+    err_hip = float((o.detach().float().cpu() - ref["o"]).abs().max())
+    err_low = float((low["o"].float() - ref["o"]).abs().max())
+    assert err_hip <= err_low, f"o: {err_hip} against {err_low} of the eager path"
+    for gname, tname in GRADS[:4]:
+        a, b = _rel(dev[tname].grad, ref[gname]), _rel(low[gname], ref[gname])
+        assert a <= b, f"{gname}: {a} against {b} of the eager path"
+    # the logit-scale gradient of head 1 is a signed sum of BW * N^2 terms that nearly cancels, so which of two
+    # roundings lands closer is chance: it is held to the eager error or to 5 % of the larger of |ref| and
+    # 2 % of the sum of the absolute terms, whichever is larger
+    want = float(ref["dscale"][1])
+    a, b = abs(float(dev["logit_scale"].grad[1]) - want), abs(float(low["dscale"][1]) - want)
+    assert a <= max(b, 5e-2 * max(abs(want), 0.02 * float(ref["dscale_l1"][1]))), f"dscale: {a} against {b}"

@@ -74,3 +74,28 @@ def test_scale_gate():
     # without a tensor scale there is no scale gradient and no bias gradient without bias
     g2 = wa.backward(q, k, v, do, None, None, mask)
     assert g2["dscale"] is None and g2["dbias"] is None
+
+
+def test_dscale_l1_is_the_sum_of_absolute_terms():
+    """`dscale_l1`, the yardstick the GPU tests hold the logit-scale gradient against, recomputed from first
+    principles with numpy: P from the logits, dZ = P (dP - delta), then sum |dZ c| per head.  The signed sum
+    of the same terms times s must give back dscale itself (for heads below the clamp), which ties the
+    yardstick to the gradient it measures."""
+    q, k, v, do, ls, bias, mask = _rand(15, bw=4, nw=2, h=3, n=7, d=4)
+    ls = ls.copy()
+    ls[2] = 5.0                                                   # one clamped head: s = 100, dscale = 0
+    ref = classic_fwd_bwd(*(torch.from_numpy(x) for x in (q, k, v, ls, bias, mask, do)), dtype=torch.float64)
+    z, c, s = wa.logits(q, k, ls, bias, mask)
+    p = np.exp(z - z.max(-1, keepdims=True))
+    p /= p.sum(-1, keepdims=True)
+    dp = np.einsum("bhid,bhjd->bhij", do, v)
+    delta = np.einsum("bhij,bhij->bhi", p, dp)[..., None]
+    dz = p * (dp - delta)
+    s = np.asarray(s).reshape(-1)
+    np.testing.assert_allclose(s, [math.exp(ls[0, 0, 0]), math.exp(ls[1, 0, 0]), 100.0], rtol=1e-12)
+    # the helper differentiates with respect to the cosine scores, so each term carries the factor s once
+    l1 = np.abs(dz * c).sum(axis=(0, 2, 3)) * s
+    np.testing.assert_allclose(ref["dscale_l1"].numpy(), l1, rtol=1e-9)
+    signed = (dz * c).sum(axis=(0, 2, 3)) * s
+    np.testing.assert_allclose(ref["dscale"].numpy().reshape(-1)[:2], signed[:2], rtol=1e-9)
+    assert float(ref["dscale"].reshape(-1)[2]) == 0.0 and np.all(l1 >= np.abs(signed) - 1e-12)
