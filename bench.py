@@ -8,7 +8,11 @@ synthetic batch (benchmark configuration 3: B=64 images x 64 windows of N=256 to
 logit_scale = ln 10), inputs already resident in HBM.  One JSON line goes to
 stdout; progress goes to stderr.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extras]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extras] [--sweep]
+
+`extras` carries the forward-only and N = 64 figures, peak memory, the window-size sweep of the reference's
+operator benchmark as HIP graph replays and one end-to-end model step; `--sweep` prints the sweep alone, with
+the eager timings beside the replays.
 """
 import argparse
 import ctypes
@@ -126,42 +130,63 @@ def cpu_baseline(cfg, torch):
     }
 
 
-def window_sweep(torch, steps, warmup):
+class L2Flush:
+    """Overwrites a buffer larger than every cache level between timed calls (the 8 x 4 MB L2s and the
+    256 MB memory-side cache), as triton.testing.do_bench does for the reference's own operator benchmark
+    (benchmark/bench_attn.py:93): small shapes are then timed from HBM, not from a warm cache."""
+
+    def __init__(self, torch, nbytes=512 << 20):
+        self.buf = torch.empty(nbytes // 4, dtype=torch.int32, device="cuda")
+
+    def __call__(self):
+        self.buf.zero_()
+
+
+def timed_calls(torch, fn, steps, warmup, flush=None):
+    """One event pair per call (recorded on torch's current stream, which is where `fn` enqueues), an optional
+    cache flush before each call outside the pair.  Returns (median ms, mean ms)."""
+    for _ in range(warmup):
+        fn()
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    for e0, e1 in pairs:
+        if flush is not None:
+            flush()
+        e0.record()
+        fn()
+        e1.record()
+    torch.cuda.synchronize()
+    ms = sorted(e0.elapsed_time(e1) for e0, e1 in pairs)
+    return ms[len(ms) // 2], sum(ms) / len(ms)
+
+
+def captured(torch, fn):
+    """`fn` as one HIP graph: warmed up on a side stream, captured once; returns the replay callable."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            fn()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        fn()
+    return graph.replay
+
+
+def window_sweep(torch, steps, warmup, eager=True, windows=(64, 144, 256, 576, 1024)):
     """The reference's window-size sweep (benchmark/config.py: B16 x 16 windows, H6, d32, windows of 8, 12, 16, 24
     and 32 tokens a side, bias = 16 sigmoid(randn), tensor logit scale ln 10, no mask) in bf16 and fp16, forward
-    and forward + backward.  Every case is timed twice: as eager calls, and as one captured HIP graph replayed
-    `steps` times, which takes the host out of the figure (at 1 536 units the eager calls are bound by it up to
-    256 tokens).  TFLOP/s count the matrix products only (4 N^2 d forward, 14 N^2 d forward + backward)."""
+    and forward + backward.  Every case is timed as one captured HIP graph replayed `steps` times, which takes the
+    host out of the figure (at 1 536 units the eager calls are bound by it up to 256 tokens), each replay from
+    flushed caches; with `eager` also as plain calls.  Median and mean per call; TFLOP/s (of the median) count the
+    matrix products only (4 N^2 d forward, 14 N^2 d forward + backward)."""
     from flash_window_attention_v2_amd import flash_win_attn_v2_func
 
-    def timed(fn):
-        for _ in range(warmup):
-            fn()
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(steps):
-            fn()
-        e1.record()
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) / steps
-
-    def captured(fn):
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
-            for _ in range(3):
-                fn()
-        torch.cuda.current_stream().wait_stream(side)
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            fn()
-        return graph.replay
-
+    flush = L2Flush(torch)
     bw, heads, d = 16 * 16, 6, 32
     rows = []
     for dtype in (torch.bfloat16, torch.float16):
-        for n in (64, 144, 256, 576, 1024):
+        for n in windows:
             g = torch.Generator(device="cpu").manual_seed(0)
             q, k, v, do = (torch.randn(bw, heads, n, d, generator=g).to(dtype).cuda() for _ in range(4))
             bias = (16 * torch.sigmoid(torch.randn(heads, n, n, generator=g))).to(dtype).cuda()
@@ -183,16 +208,59 @@ def window_sweep(torch, steps, warmup):
             fl_all = flops_matmul(bw, heads, n, d)
             row = {"dtype": str(dtype).split(".")[-1], "n": n}
             for tag, fn, f in (("fwd", fwd, fl), ("fwd_bwd", fwd_bwd, fl_all)):
-                ms_e = timed(fn)
-                ms_g = timed(captured(fn))
-                row[tag + "_ms"] = round(ms_e, 4)
-                row[tag + "_tflops"] = round(f / ms_e * 1e-9, 1)
-                row[tag + "_graph_ms"] = round(ms_g, 4)
-                row[tag + "_graph_tflops"] = round(f / ms_g * 1e-9, 1)
+                if eager:
+                    med, mean = timed_calls(torch, fn, steps, warmup, flush)
+                    row[tag + "_eager_ms"] = [round(med, 4), round(mean, 4)]
+                    row[tag + "_eager_tflops"] = round(f / med * 1e-9, 1)
+                med, mean = timed_calls(torch, captured(torch, fn), steps, warmup, flush)
+                row[tag + "_ms"] = [round(med, 4), round(mean, 4)]
+                row[tag + "_tflops"] = round(f / med * 1e-9, 1)
+                row[tag + "_pct_peak"] = round(f / med * 1e-9 / MFMA_BF16_PEAK_TFLOPS * 100, 2)
             log(f"[bench] sweep {row}")
             rows.append(row)
-    return {"sweep": "B16 x 16 windows, H6, d32, bias, tensor scale, no mask; TFLOP/s of the matrix products",
+    return {"sweep": "B16 x 16 windows, H6, d32, bias, tensor scale, no mask; one HIP graph replay per call, caches "
+                     "flushed before each; *_ms = [median, mean]; TFLOP/s of the matrix products at the median; "
+                     "pct_peak against 2.5 PFLOP/s (bf16 and fp16 dense)",
             "steps": steps, "warmup": warmup, "rows": rows}
+
+
+def model_step(torch, steps, warmup, batch=64):
+    """The end-to-end case (Swin V2-T layout: 256 x 256 images, patch 4, depths 2/2/6/2, heads 3/6/12/24, windows
+    of 16 x 16 tokens, bf16, batch 64) timed the way the reference times its model (benchmark/bench_model.py:23-38:
+    zero_grad, forward, cross-entropy, backward, Adam step; peak memory of the loop), with this library's operator
+    and with the classic one.  Median and mean of per-step event pairs."""
+    from flash_window_attention_v2_amd import SwinTransformerV2
+
+    out = {"config": f"img 256, patch 4, embed 96, depths 2/2/6/2, heads 3/6/12/24, window 16, bf16, batch {batch}, "
+                     "random weights and images; training step with Adam; *_ms = [median, mean]"}
+    g = torch.Generator(device="cpu").manual_seed(0)
+    x = torch.randn(batch, 3, 256, 256, generator=g).to(torch.bfloat16).cuda()
+    y = torch.randint(0, 1000, (batch,), generator=g).cuda()
+    for tag, flash in (("flash", True), ("classic", False)):
+        torch.manual_seed(0)
+        model = SwinTransformerV2(img_size=256, patch_size=4, embed_dim=96, depths=[2, 2, 6, 2], num_heads=[3, 6, 12, 24],
+                                  window_size=16, is_flash=flash).to(dtype=torch.bfloat16, device="cuda")
+        opt = torch.optim.Adam(model.parameters(), lr=1e-4)
+
+        def step():
+            opt.zero_grad()
+            loss = torch.nn.functional.cross_entropy(model(x), y)
+            loss.backward()
+            opt.step()
+
+        step()
+        torch.cuda.synchronize(); torch.cuda.empty_cache(); torch.cuda.reset_peak_memory_stats()
+        med, mean = timed_calls(torch, step, steps, warmup)
+        out[tag + "_step_ms"] = [round(med, 3), round(mean, 3)]
+        out[tag + "_peak_mem_gb"] = round(torch.cuda.max_memory_allocated() / 2**30, 3)
+        with torch.no_grad():
+            med, mean = timed_calls(torch, lambda: model(x), steps, warmup)
+        out[tag + "_fwd_ms"] = [round(med, 3), round(mean, 3)]
+        log(f"[bench] model {tag}: step {out[tag + '_step_ms']} ms, {out[tag + '_peak_mem_gb']} GB")
+        del model, opt
+        torch.cuda.empty_cache()
+    out["step_speedup"] = round(out["classic_step_ms"][0] / out["flash_step_ms"][0], 3)
+    return out
 
 
 def main():
@@ -220,7 +288,7 @@ def main():
     lib = _abi.load()
     torch.cuda.set_device(0)
     if args.sweep:
-        print(json.dumps(window_sweep(torch, args.steps, args.warmup)), flush=True)
+        print(json.dumps(window_sweep(torch, min(args.steps, 30), min(args.warmup, 5))), flush=True)
         return
 
     def setup(cfg):
@@ -266,7 +334,7 @@ def main():
         "config": {"workload": "C3: B64 x 64 windows, H3, N256, d32, bf16, shift-8 mask, fwd+bwd", "bw": bw,
                    "heads": cfg["heads"], "n": cfg["n"], "head_dim": cfg["d"]},
         "pct_mfma_peak": round(100 * tflops / MFMA_BF16_PEAK_TFLOPS, 2),
-        "roofline": {"bound": "mfma", "kernel": "bwd_kernel (dk, dv, dbias; both launches)", "achieved": round(achieved, 2),
+        "roofline": {"bound": "mfma", "kernel": "bwd_key_kernel (dk, dv, dbias, delta; one launch)", "achieved": round(achieved, 2),
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": BWD_KERNEL_TRAFFIC_BYTES,
                      "kernel_ms": round(kern_avg, 4),
@@ -316,6 +384,11 @@ def main():
         extras["c2_hbm_frac"] = round(extras["c2_hbm_gbs"] / HBM_PEAK_GBS, 4)
         extras["c2_tflops"] = round(flops_matmul(bw2, c2["heads"], c2["n"], c2["d"]) / ms2 * 1e-9, 2)
         del dev2
+        torch.cuda.empty_cache()
+        log("[bench] window-size sweep as graph replays")
+        extras["window_sweep"] = window_sweep(torch, 10, 2, eager=False)
+        log("[bench] end-to-end model step")
+        extras["model"] = model_step(torch, 8, 2)
         result["extras"] = extras
 
     if args.copy_bytes:

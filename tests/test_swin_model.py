@@ -293,15 +293,13 @@ def test_block_window_map_matches_partition_gpu(window, shift):
         assert rel(grads_a[n], p.grad) < 2e-2, n
 
 
-@pytest.mark.gpu
-def test_model_flash_matches_classic_gpu():
-    """Whole-model step at a reduced width: bf16 model on the fused kernels against the same weights
-    on the classic path in fp32, LayerNorms away from their zero initialisation and no stochastic
-    depth so both runs are deterministic functions of the weights."""
+def _model_step_against_classic(kw, batch, classes):
+    """One training step of the bf16 model on the fused kernels, of the same weights on the classic path
+    in fp32 and in bf16: LayerNorms away from their zero initialisation and no stochastic depth, so all
+    three runs are deterministic functions of the weights.  Returns the losses and, per run, the worst
+    relative gradient error over the parameters against the fp32 run."""
     torch.manual_seed(0)
     dev = torch.device("cuda")
-    kw = dict(img_size=64, patch_size=2, embed_dim=96, depths=[2, 2], num_heads=[3, 6], window_size=8,
-              num_classes=10, drop_path_rate=0.0)
     ref = swin.SwinTransformerV2(is_flash=False, **kw)
     _randomise_norms(ref)
     ref = ref.to(dev)
@@ -312,8 +310,8 @@ def test_model_flash_matches_classic_gpu():
     eager.load_state_dict(ref.state_dict())
     eager = eager.to(torch.bfloat16)
 
-    x = torch.randn(4, 3, 64, 64, device=dev)
-    labels = torch.randint(0, 10, (4,), device=dev)
+    x = torch.randn(batch, 3, kw["img_size"], kw["img_size"], device=dev)
+    labels = torch.randint(0, classes, (batch,), device=dev)
     losses, grads = {}, {}
     for name, model, inp in (("ref", ref, x), ("fused", fused, x.bfloat16()), ("eager", eager, x.bfloat16())):
         logits = model(inp)
@@ -321,14 +319,42 @@ def test_model_flash_matches_classic_gpu():
         loss.backward()
         losses[name] = float(loss)
         grads[name] = {k: p.grad.float() for k, p in model.named_parameters()}
-    assert abs(losses["fused"] - losses["ref"]) < 3e-2
+        assert all(torch.isfinite(g).all() for g in grads[name].values()), name
 
     def worst(name):
         return max(float((grads[name][k] - grads["ref"][k]).abs().max() / (grads["ref"][k].abs().max() + 1e-6))
                    for k in grads["ref"])
 
+    return losses, worst("fused"), worst("eager"), fused
+
+
+@pytest.mark.gpu
+def test_model_flash_matches_classic_gpu():
+    """Whole-model step at a reduced width (two stages, 64 x 64 images, windows of 64 tokens)."""
+    kw = dict(img_size=64, patch_size=2, embed_dim=96, depths=[2, 2], num_heads=[3, 6], window_size=8,
+              num_classes=10, drop_path_rate=0.0)
+    losses, fused, eager, _ = _model_step_against_classic(kw, batch=4, classes=10)
+    assert abs(losses["fused"] - losses["ref"]) < 3e-2
     # the fused path in bf16 must be about as close to fp32 as the eager bf16 model is
-    assert worst("fused") < max(2.0 * worst("eager"), 5e-2)
+    assert fused < max(2.0 * eager, 5e-2)
+
+
+@pytest.mark.gpu
+def test_model_of_the_end_to_end_benchmark_gpu():
+    """The model the reference times end to end (benchmark/bench_swin.py:110-131: 256 x 256 images,
+    patch 4, depths 2/2/6/2, heads 3/6/12/24, windows of 16 x 16 tokens, which the last stage's 8 x 8 grid
+    cuts down to 8 x 8) at a reduced batch: every stage's kernels, both window sizes, shifted and
+    unshifted blocks, patch merging and the head in one step."""
+    kw = dict(img_size=256, patch_size=4, embed_dim=96, depths=[2, 2, 6, 2], num_heads=[3, 6, 12, 24],
+              window_size=16, num_classes=1000, drop_path_rate=0.0)
+    losses, fused, eager, model = _model_step_against_classic(kw, batch=4, classes=1000)
+    windows = [blk.attn.window_size for layer in model.layers for blk in layer.blocks]
+    shifts = [blk.shift_size for layer in model.layers for blk in layer.blocks]
+    assert windows[:10] == [(16, 16)] * 10 and windows[10:] == [(8, 8)] * 2
+    assert shifts == [0, 8, 0, 8] + [0] * 8          # the 16 x 16 and 8 x 8 grids are one window: no shift
+    assert abs(losses["fused"] - losses["ref"]) < 3e-2
+    assert abs(losses["fused"] - losses["ref"]) <= max(2.0 * abs(losses["eager"] - losses["ref"]), 1e-2)
+    assert fused < max(2.0 * eager, 5e-2), (fused, eager)
 
 
 @pytest.mark.gpu
