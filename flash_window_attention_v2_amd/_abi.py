@@ -9,12 +9,13 @@ import ctypes
 import os
 import threading
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 OK, ERR_INVALID_ARGUMENT, ERR_UNSUPPORTED, ERR_HIP, ERR_NO_DEVICE = range(5)
 F16, BF16, F32 = 0, 1, 2
 SCALE_DEFAULT, SCALE_TENSOR = 0, 1
 STATIC_SCRATCH_BYTES = 64 << 20     # FWA2_STATIC_SCRATCH_BYTES of include/fwa2.h
+MASK_REGION_BYTES = 272             # FWA2_MASK_REGION_BYTES of include/fwa2.h
 
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libfwa2.so")
 
@@ -23,6 +24,7 @@ EXPORTS = (
     "fwa2_last_error",
     "fwa2_validate",
     "fwa2_mask_scan",
+    "fwa2_mask_scan_regions",
     "fwa2_backward_workspace_bytes",
     "fwa2_forward",
     "fwa2_backward",
@@ -61,6 +63,7 @@ class Problem(ctypes.Structure):
         ("win_h", ctypes.c_int32), ("win_w", ctypes.c_int32),
         ("shift_h", ctypes.c_int32), ("shift_w", ctypes.c_int32),
         ("n_keys", ctypes.c_int32), ("reserved0", ctypes.c_int32),
+        ("mask_regions", ctypes.c_void_p),
     ]
 
 
@@ -96,6 +99,9 @@ def load():
         lib.fwa2_mask_scan.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int64,
                                        ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]
         lib.fwa2_mask_scan.restype = ctypes.c_int
+        lib.fwa2_mask_scan_regions.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int64,
+                                               ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
+        lib.fwa2_mask_scan_regions.restype = ctypes.c_int
         lib.fwa2_backward_workspace_bytes.argtypes = [ctypes.POINTER(Problem)]
         lib.fwa2_backward_workspace_bytes.restype = ctypes.c_size_t
         lib.fwa2_forward.argtypes = [ctypes.POINTER(Problem)]

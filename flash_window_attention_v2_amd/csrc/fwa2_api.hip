@@ -13,7 +13,8 @@
 namespace fwa2 {
 hipError_t launch_forward(FwdParams p, int dtype, bool has_bias, int mask_dt, hipStream_t st);
 hipError_t launch_mask_scan(const void* mask, int mask_dt, int64_t sw, int64_t sn, int n, int n_windows,
-                            uint8_t* live, hipStream_t st);
+                            uint8_t* live, uint8_t* regions, hipStream_t st);
+static_assert(sizeof(RegionRecord) == FWA2_MASK_REGION_BYTES, "the header states the size of a region record");
 hipError_t launch_backward(const BwdParams& p, int dtype, bool has_bias, int mask_dt, hipStream_t st);
 size_t backward_workspace_bytes(int heads, int n, int bw, bool has_bias, bool has_mask, int n_windows, int cus);
 bool generic_problem(int d, int n, int nk);
@@ -219,16 +220,30 @@ size_t fwa2_backward_workspace_bytes(const fwa2_problem* p) {
                                           p->n_windows, cu_count());
 }
 
-int fwa2_mask_scan(const void* mask, int mask_dtype, int n_windows, int n, int64_t stride_w, int64_t stride_n,
-                   uint8_t* live, void* stream) {
+static int mask_scan(const char* what, const void* mask, int mask_dtype, int n_windows, int n, int64_t stride_w,
+                     int64_t stride_n, uint8_t* live, void* regions, bool want_regions, void* stream) {
     g_err[0] = 0;
-    if (mask == nullptr || live == nullptr || n_windows <= 0 || n <= 0)
-        return fail(FWA2_ERR_INVALID_ARGUMENT, "fwa2_mask_scan: bad argument");
+    if (mask == nullptr || live == nullptr || n_windows <= 0 || n <= 0 || (want_regions && regions == nullptr))
+        return fail(FWA2_ERR_INVALID_ARGUMENT, "%s: bad argument", what);
+    if (want_regions && ((uintptr_t)regions & 15))
+        return fail(FWA2_ERR_INVALID_ARGUMENT, "%s: regions must be 16-byte aligned", what);
     if (mask_dtype != FWA2_F16 && mask_dtype != FWA2_BF16 && mask_dtype != FWA2_F32)
-        return fail(FWA2_ERR_INVALID_ARGUMENT, "fwa2_mask_scan: bad mask dtype");
-    hipError_t e = fwa2::launch_mask_scan(mask, mask_dtype, stride_w, stride_n, n, n_windows, live, (hipStream_t)stream);
+        return fail(FWA2_ERR_INVALID_ARGUMENT, "%s: bad mask dtype", what);
+    hipError_t e = fwa2::launch_mask_scan(mask, mask_dtype, stride_w, stride_n, n, n_windows, live, (uint8_t*)regions,
+                                          (hipStream_t)stream);
     if (e != hipSuccess) return fail(FWA2_ERR_HIP, "mask scan launch: %s", hipGetErrorString(e));
     return FWA2_OK;
+}
+
+int fwa2_mask_scan(const void* mask, int mask_dtype, int n_windows, int n, int64_t stride_w, int64_t stride_n,
+                   uint8_t* live, void* stream) {
+    return mask_scan("fwa2_mask_scan", mask, mask_dtype, n_windows, n, stride_w, stride_n, live, nullptr, false, stream);
+}
+
+int fwa2_mask_scan_regions(const void* mask, int mask_dtype, int n_windows, int n, int64_t stride_w, int64_t stride_n,
+                           uint8_t* live, void* regions, void* stream) {
+    return mask_scan("fwa2_mask_scan_regions", mask, mask_dtype, n_windows, n, stride_w, stride_n, live, regions, true,
+                     stream);
 }
 
 static int check_cpb(const char* what, const void* a, const void* b, const void* c, int dtype, int heads, int wh, int ww) {
@@ -281,6 +296,7 @@ int fwa2_forward(const fwa2_problem* p) {
     k.mask = p->mask.ptr; k.mask_sw = p->mask.stride_a; k.mask_sn = p->mask.stride_n;
     // the kernels keep the per-window flags in LDS; beyond that many windows they go without
     k.mask_live = (p->mask.ptr && p->n_windows <= fwa2::kLiveCache) ? p->mask_live : nullptr;
+    k.regions = k.mask_live ? (const uint8_t*)p->mask_regions : nullptr;
     k.lse = p->lse; k.lse_sb = p->lse_stride_bw; k.lse_sh = p->lse_stride_h;
     k.bw = p->bw; k.heads = p->heads; k.n = p->n; k.n_windows = p->mask.ptr ? p->n_windows : 1;
     k.scale_kind = p->scale_kind;
@@ -312,6 +328,7 @@ static int run_backward(const fwa2_problem* p) {
     k.mask = p->mask.ptr; k.mask_sw = p->mask.stride_a; k.mask_sn = p->mask.stride_n;
     // the kernels keep the per-window flags in LDS; beyond that many windows they go without
     k.mask_live = (p->mask.ptr && p->n_windows <= fwa2::kLiveCache) ? p->mask_live : nullptr;
+    k.regions = k.mask_live ? (const uint8_t*)p->mask_regions : nullptr;
     k.lse = p->lse; k.lse_sb = p->lse_stride_bw; k.lse_sh = p->lse_stride_h;
     k.bw = p->bw; k.heads = p->heads; k.n = p->n; k.n_windows = p->mask.ptr ? p->n_windows : 1;
     k.scale_kind = p->scale_kind;

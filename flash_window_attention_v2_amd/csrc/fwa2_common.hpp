@@ -89,6 +89,26 @@ __device__ __forceinline__ typename Elem<DT>::V8 lds_tr8(const typename Elem<DT>
     return r;
 }
 
+// ---- global -> LDS copies that bypass the registers, issued by hand ---------------------------------------
+// The builtin form of these loads makes the compiler guard LDS reads it cannot tell apart from the landing area
+// with a wait for ALL outstanding vector-memory operations, which stalls a kernel that fetches the next unit while
+// it computes on the current one.  Written as inline assembly the copies are invisible to that bookkeeping: the
+// kernel waits for them itself (s_waitcnt vmcnt) before it reads a landing area.  Each lane reads 16 (or 4) bytes
+// at its own address; lane i lands at lds + 16 i (4 i), lds being uniform over the wavefront.  The waits the
+// hardware asks for around M0 are part of the sequence.
+__device__ __forceinline__ uint32_t lds_address(const void* p) {     // of a wavefront-uniform pointer, as a scalar
+    return __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)p);
+}
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+__device__ __forceinline__ void dma16_to_lds(const void* src, uint32_t lds) {      // non-temporal: streamed rows
+    asm volatile("s_nop 3\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off nt" ::"v"(src), "s"(lds) : "memory", "m0");
+}
+__device__ __forceinline__ void dma4_to_lds(const void* src, uint32_t lds) {
+    asm volatile("s_nop 3\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(src), "s"(lds) : "memory", "m0");
+}
+#pragma clang diagnostic pop
+
 // ---- cross-lane helpers (wave64) -------------------------------------------
 // Value held by the lane 32 away, combined with the own value by max / add.
 __device__ __forceinline__ float xor32_max(float x) {
@@ -174,6 +194,45 @@ __device__ __forceinline__ float wave_sum(float x) {
 // ---- helpers of the kernels that keep the bias tile resident in registers ----
 constexpr int kLiveCache = 1024;    // windows whose mask flags are cached in LDS
 constexpr float kGapLimit = 96.f;   // largest tolerated (row bound - largest logit), log2 domain
+
+// A window whose mask is exactly value * [id_i != id_j] (see mask_scan_kernel) is described by this record
+// instead of its N x N entries.  The kernels add the term on the matrix pipe: one more (small) MFMA per score
+// tile whose query-side operand holds value * log2e, split into two fp16 terms, in the k-slot of the query's
+// id, and whose key-side operand holds 1 in every slot but the key's own id.
+constexpr int kMaxRegions = 8;
+constexpr float kMaxRegionValue2 = 30000.f;     // |value * log2e| must stay inside fp16 with room to spare
+struct RegionRecord {
+    float value;
+    int count;
+    int pad[2];
+    uint8_t id[256];
+};
+static_assert(sizeof(RegionRecord) == 272, "RegionRecord is part of the C ABI (FWA2_MASK_REGION_BYTES)");
+// The region product is a 16 x 16 x 16 fp16 MFMA whose 16 k-slots are (8 ids) x (value * log2e split into two
+// fp16 terms).  Lane (g, l16) of an operand holds slots 4g .. 4g+3: ids 4 (g & 1) .. 4 (g & 1) + 3, first term for
+// g < 2, second term for g >= 2.  `key_side` is the M operand (rows = keys), `query_side` the N operand.
+__device__ __forceinline__ f32x4 region_mfma(f16x4 key_side, f16x4 query_side, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x16f16(key_side, query_side, c, 0, 0, 0);
+}
+// Query-side operand of this lane for a query with region id `id`: value2 = value * log2e.
+__device__ __forceinline__ f16x4 region_query_operand(float value2, int id, int g) {
+    const _Float16 hi = (_Float16)value2;
+    const _Float16 lo = (_Float16)(value2 - (float)hi);
+    const _Float16 term = g < 2 ? hi : lo;
+    const int rel = id - 4 * (g & 1);
+    f16x4 r;
+#pragma unroll
+    for (int j = 0; j < 4; j++) r[j] = j == rel ? term : (_Float16)0.f;
+    return r;
+}
+// Key-side table entry of a key with region id `id`: 1 in every id slot but its own (8 halves, ids 0 .. 7); a lane
+// reads the four halves at 4 (g & 1).
+__device__ __forceinline__ f16x8 region_key_entry(int id) {
+    f16x8 r;
+#pragma unroll
+    for (int j = 0; j < 8; j++) r[j] = j == id ? (_Float16)0.f : (_Float16)1.f;
+    return r;
+}
 
 __device__ __forceinline__ float xor16_max(float x) {
     u32x2 r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
@@ -284,8 +343,10 @@ struct FwdParams {
     const void* mask;
     int64_t mask_sw, mask_sn;
     const uint8_t* mask_live;  // [n_windows] flags from the mask scan (0 = window's mask is all zero, bit 0 =
-                               // it has a non-zero entry, bit 1 = all entries <= 0 and every row keeps a 0);
+                               // it has a non-zero entry, bit 1 = all entries <= 0 and every row keeps a 0,
+                               // bit 2 = the window has a RegionRecord);
                                // nullptr = assume every window live and nothing known about it
+    const uint8_t* regions;    // [n_windows] RegionRecord, or nullptr
     float* lse;
     int64_t lse_sb, lse_sh;
     int bw, heads, n, n_windows;
@@ -307,6 +368,7 @@ struct BwdParams {
     const void* mask;
     int64_t mask_sw, mask_sn;
     const uint8_t* mask_live;
+    const uint8_t* regions;    // [n_windows] RegionRecord, or nullptr
     const float* lse;
     int64_t lse_sb, lse_sh;
     int bw, heads, n, n_windows;

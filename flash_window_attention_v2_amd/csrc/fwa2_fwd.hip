@@ -249,26 +249,91 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdParams p) {
 // One byte of flags per window.  0: the [N, N] mask is all zero.  Bit 0: it holds a non-zero entry.
 // Bit 1 (with bit 0): no entry is positive (or NaN) and every row keeps at least one exact zero, so
 // the mask can only remove keys and never removes all of a row.
+// Bit 2 (with bits 0 and 1, only when `regions` is given and n <= 256): the mask is EXACTLY
+// c * [id_i != id_j] for one finite c < 0 and a labelling of the tokens with at most kMaxRegions ids, which
+// is what the shifted-window construction produces (swin_transformer_v2.py:386-405 of the reference: ids
+// painted on the rolled grid, -100 where they differ).  The window's record in `regions` then holds c and
+// the ids (RegionRecord); every entry of the mask has been compared with that form, so a kernel may rebuild
+// the window's mask from the record instead of reading it.
 template <class ME>
 __global__ void __launch_bounds__(256) mask_scan_kernel(const ME* mask, int64_t sw, int64_t sn, int n,
-                                                        uint8_t* live) {
+                                                        uint8_t* live, uint8_t* regions) {
     const int w = blockIdx.x;
     const ME* m = mask + w * sw;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    __shared__ int lds_rep[256];          // first column of the row that holds an exact zero (n if none)
+    __shared__ float lds_lo[256], lds_hi[256];
+    __shared__ uint8_t lds_id[256];
+    const bool want = regions != nullptr && n <= 256;
     int any = 0, unsafe = 0;
+    float lo = INFINITY, hi = -INFINITY;  // range of the non-zero entries this thread saw
     for (int r = wave; r < n; r += 4) {       // one wavefront per row, coalesced along the row
-        int zero = 0;
+        int first = n;
         for (int c = lane; c < n; c += 64) {
             const float v = (float)m[r * sn + c];
             any |= (v != 0.f);
             unsafe |= !(v <= 0.f);
-            zero |= (v == 0.f);
+            if (v == 0.f) first = min(first, c);
+            else { lo = fminf(lo, v); hi = fmaxf(hi, v); }
         }
-        if (!__any(zero)) unsafe = 1;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) first = min(first, __shfl_xor(first, off));
+        if (first == n) unsafe = 1;
+        if (want && lane == 0) lds_rep[r] = first;
     }
     any = __syncthreads_or(any);
     unsafe = __syncthreads_or(unsafe);
-    if (threadIdx.x == 0) live[w] = any ? (unsafe ? 1 : 3) : 0;
+    uint8_t flags = any ? (unsafe ? 1 : 3) : 0;
+    if (want && flags == 3) {
+        // the one non-zero value
+        lds_lo[tid] = lo;
+        lds_hi[tid] = hi;
+        __syncthreads();
+        for (int off = 128; off > 0; off >>= 1) {
+            if (tid < off) {
+                lds_lo[tid] = fminf(lds_lo[tid], lds_lo[tid + off]);
+                lds_hi[tid] = fmaxf(lds_hi[tid], lds_hi[tid + off]);
+            }
+            __syncthreads();
+        }
+        const float cval = lds_lo[0];
+        int bad = !(cval == lds_hi[0]) || !(cval < 0.f) || !(cval * kLog2e > -kMaxRegionValue2);
+        // tokens of a region all see their first zero at the region's smallest token: that token stands for
+        // the region, and ids number the regions in the order of those tokens
+        int id = 0, reps = 0;
+        if (tid < n) {
+            const int rep = lds_rep[tid];
+            bad |= rep > tid;                            // the diagonal must be zero
+            for (int j = 0; j < n; j++) {
+                const int is_rep = lds_rep[j] == j;
+                reps += is_rep;
+                id += is_rep && j < rep;
+            }
+            bad |= reps > kMaxRegions;
+            lds_id[tid] = (uint8_t)(id & 255);
+        }
+        bad = __syncthreads_or(bad);
+        if (!bad) {
+            // every entry against the form
+            for (int r = wave; r < n; r += 4) {
+                const int idr = lds_id[r];
+                for (int c = lane; c < n; c += 64) {
+                    const float v = (float)m[r * sn + c];
+                    const float want_v = (lds_id[c] != idr) ? cval : 0.f;
+                    bad |= !(v == want_v);
+                }
+            }
+            bad = __syncthreads_or(bad);
+        }
+        if (!bad) {
+            flags |= 4;
+            RegionRecord* rec = reinterpret_cast<RegionRecord*>(regions + (size_t)w * sizeof(RegionRecord));
+            if (tid == 0) { rec->value = cval; rec->count = reps; rec->pad[0] = 0; rec->pad[1] = 0; }
+            rec->id[tid] = tid < n ? lds_id[tid] : 0;
+        }
+    }
+    if (tid == 0) live[w] = flags;
 }
 
 template <int DT, bool HAS_BIAS, int MASK_DT>
@@ -309,14 +374,14 @@ hipError_t launch_forward(FwdParams p, int dtype, bool has_bias, int mask_dt, hi
 }
 
 hipError_t launch_mask_scan(const void* mask, int mask_dt, int64_t sw, int64_t sn, int n, int n_windows,
-                            uint8_t* live, hipStream_t st) {
+                            uint8_t* live, uint8_t* regions, hipStream_t st) {
     dim3 grid(n_windows), block(256);
     if (mask_dt == FWA2_F32)
-        hipLaunchKernelGGL(mask_scan_kernel<float>, grid, block, 0, st, (const float*)mask, sw, sn, n, live);
+        hipLaunchKernelGGL(mask_scan_kernel<float>, grid, block, 0, st, (const float*)mask, sw, sn, n, live, regions);
     else if (mask_dt == FWA2_BF16)
-        hipLaunchKernelGGL(mask_scan_kernel<__bf16>, grid, block, 0, st, (const __bf16*)mask, sw, sn, n, live);
+        hipLaunchKernelGGL(mask_scan_kernel<__bf16>, grid, block, 0, st, (const __bf16*)mask, sw, sn, n, live, regions);
     else
-        hipLaunchKernelGGL(mask_scan_kernel<_Float16>, grid, block, 0, st, (const _Float16*)mask, sw, sn, n, live);
+        hipLaunchKernelGGL(mask_scan_kernel<_Float16>, grid, block, 0, st, (const _Float16*)mask, sw, sn, n, live, regions);
     return hipGetLastError();
 }
 

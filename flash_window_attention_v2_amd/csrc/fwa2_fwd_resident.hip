@@ -58,6 +58,14 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
     __shared__ __attribute__((aligned(16))) E lds_V[2][ROWS * S];
     __shared__ __attribute__((aligned(16))) E lds_rawK[ROWS * 32];   // landing area: unpadded 64-byte rows
     __shared__ __attribute__((aligned(16))) E lds_rawV[ROWS * 32];
+    __shared__ __attribute__((aligned(16))) E lds_rawQ[ROWS * 32];   // the wavefront's own 16 query rows
+    // REGIONS: the plain launch also takes the windows whose mask has region form (RegionRecord): their mask term
+    // comes out of one more MFMA per score tile, query-side operand in registers, key-side operand in lds_kop
+    constexpr bool REGIONS = MASK_DT >= 0 && !MASKED;
+    static_assert(kLdsStride >= 40 && kScoreDT == FWA2_F16,
+                  "the key-side entries of the region product live in the 8 spare fp16 columns of the staged K rows");
+    // landing area of the region record: per wavefront the ids of its 16 rows, then the record's value
+    __shared__ __attribute__((aligned(16))) uint8_t lds_rawid[REGIONS ? ROWS * 2 : 32];
     __shared__ uint8_t lds_live[kLiveCache];       // copy of the per-window mask flags
     __shared__ uint16_t lds_list[kLiveCache];      // windows of this launch's class, ascending
     __shared__ int lds_count;
@@ -66,7 +74,7 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
     const int tid = threadIdx.x;
     const int nthreads = blockDim.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);      // uniform: lives in a scalar register
     const int l16 = lane & 15;       // query column inside the wavefront's 16 rows
     const int g = lane >> 4;         // accumulator rows 4g .. 4g+3, operand k-slots 8g .. 8g+7
 
@@ -81,6 +89,35 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
         scale2 = p.default_scale * kLog2e;
     }
 
+    // ---- which units belong to this launch.  With the mask flags at hand the windows of this
+    // launch's class (mask live or not) are listed once.
+    //   plain launch: the units of the listed windows (all units without a mask) are dealt out by
+    //     their rank, so every workgroup of the head gets the same number of them;
+    //   MASKED launch: the head's workgroups are dealt out over the listed windows (several per
+    //     window, which then share its images, or several windows per workgroup in turn), and the
+    //     tile is rebuilt with the window's mask whenever a workgroup moves on to another window. ----
+    const int nw = MASK_DT >= 0 ? p.n_windows : 1;
+    const bool listed = MASK_DT >= 0 && p.mask_live != nullptr;      // the host drops the flags beyond kLiveCache
+    if (listed) {
+        for (int i = tid; i < nw; i += nthreads) lds_live[i] = p.mask_live[i];
+        __syncthreads();
+        if (wave == 0) {
+            int c = 0;
+            for (int base = 0; base < nw; base += 64) {
+                const int w = base + lane;
+                // a live window goes to the MASKED launch unless its region record serves it here
+                const bool in = w < nw && ((lds_live[w] != 0 && !(p.regions != nullptr && (lds_live[w] & 4))) == MASKED);
+                const unsigned long long bal = __ballot(in);
+                if (in) lds_list[c + __popcll(bal & ((1ull << lane) - 1ull))] = (uint16_t)w;
+                c += __popcll(bal);
+            }
+            if (lane == 0) lds_count = c;
+        }
+        __syncthreads();
+    }
+    const int cnt = listed ? __builtin_amdgcn_readfirstlane(lds_count) : nw;    // windows of this class
+    if (cnt == 0) return;                  // nothing for this launch (every live window has region form, say)
+
     // rows of the staging buffers that no unit ever writes must read as zeros
     for (int i = tid; i < 2 * ROWS * S / 8; i += nthreads) {
         st8<SV8>(&lds_K[0][0] + i * 8, zero8<SV8>());
@@ -89,6 +126,7 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
     for (int i = tid; i < ROWS * 32 / 8; i += nthreads) {
         st8<V8>(lds_rawK + i * 8, zero8<V8>());
         st8<V8>(lds_rawV + i * 8, zero8<V8>());
+        st8<V8>(lds_rawQ + i * 8, zero8<V8>());
     }
 
     const int qi = wave * 16 + l16;
@@ -102,6 +140,7 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
     // of every logit of the row; the key that attains the maximum scores at least m_fixed - 2 s log2e. ----
     f32x4 acc0[NT];
     float m_fixed = 0.f;
+    float bias_range = 0.f;      // largest minus smallest bias (log2 domain) of this lane's row
     auto build_tile = [&](int w) __attribute__((always_inline)) {
         // lane-derived offsets are re-materialised per call: hoisted out of the unit loop, the row
         // addresses of every key group would stay alive (and spilled) across all units
@@ -113,7 +152,7 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
         const ME* mrow = nullptr;
         if (HAS_BIAS) brow = reinterpret_cast<const E*>(p.bias) + h * p.bias_sh + (int64_t)qrow * p.bias_sn;
         if (MASKED) mrow = reinterpret_cast<const ME*>(p.mask) + w * p.mask_sw + (int64_t)qrow * p.mask_sn;
-        float mb = -INFINITY;
+        float mb = -INFINITY, mn = INFINITY;
 #pragma unroll
         for (int kp = 0; kp < NT / 2; kp++) {
             float v[8];
@@ -133,9 +172,11 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
             for (int j = 0; j < 8; j++) {
                 acc0[2 * kp + (j >> 2)][j & 3] = v[j];
                 mb = fmaxf(mb, v[j]);
+                if (REGIONS && v[j] > -INFINITY) mn = fminf(mn, v[j]);
             }
         }
         mb = col_max(mb);
+        if (REGIONS) bias_range = mb - (-col_max(-mn));
         if (!(mb > -INFINITY)) mb = 0.f;        // every key of the row removed: nothing to bound
         m_fixed = mb + scale2;
 #pragma unroll
@@ -147,32 +188,6 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
     // largest logit (the same for every row of the head)
     const bool fast = (DT == FWA2_BF16) && (2.f * scale2 <= kGapLimit);
 
-    // ---- which units belong to this launch.  With the mask flags at hand the windows of this
-    // launch's class (mask live or not) are listed once.
-    //   plain launch: the units of the listed windows (all units without a mask) are dealt out by
-    //     their rank, so every workgroup of the head gets the same number of them;
-    //   MASKED launch: the head's workgroups are dealt out over the listed windows (several per
-    //     window, which then share its images, or several windows per workgroup in turn), and the
-    //     tile is rebuilt with the window's mask whenever a workgroup moves on to another window. ----
-    const int nw = MASK_DT >= 0 ? p.n_windows : 1;
-    const bool listed = MASK_DT >= 0 && p.mask_live != nullptr;      // the host drops the flags beyond kLiveCache
-    if (listed) {
-        for (int i = tid; i < nw; i += nthreads) lds_live[i] = p.mask_live[i];
-        __syncthreads();
-        if (wave == 0) {
-            int c = 0;
-            for (int base = 0; base < nw; base += 64) {
-                const int w = base + lane;
-                const bool in = w < nw && ((lds_live[w] != 0) == MASKED);
-                const unsigned long long bal = __ballot(in);
-                if (in) lds_list[c + __popcll(bal & ((1ull << lane) - 1ull))] = (uint16_t)w;
-                c += __popcll(bal);
-            }
-            if (lane == 0) lds_count = c;
-        }
-        __syncthreads();
-    }
-    const int cnt = listed ? __builtin_amdgcn_readfirstlane(lds_count) : nw;    // windows of this class
     const int n_img = p.bw / nw;
     auto window_at = [&](int wi) -> int {
         return listed ? __builtin_amdgcn_readfirstlane((int)lds_list[wi]) : wi;
@@ -212,12 +227,19 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
         return c;
     };
     auto unit_of = [&](const Cursor& c) -> int { return c.img * nw + window_at(c.wi); };
+    // the region record of the cursor's window, or nullptr when the window has none (uniform)
+    auto record_of = [&](const Cursor& c) -> const RegionRecord* {
+        if (!REGIONS || p.regions == nullptr) return nullptr;
+        const int w = window_at(c.wi);
+        if (!(lds_live[w] & 4)) return nullptr;
+        return reinterpret_cast<const RegionRecord*>(p.regions) + w;
+    };
 
     // ---- per-unit fetch: every wavefront brings in the 16 K and V rows it will stage (lane i lands
     // at 16 i bytes from the wavefront's base) and its own 16 query rows ----
     const int frow = wave * 16 + (lane >> 2);      // K / V row of this lane
     const int fc8 = (lane & 3) * 8;
-    auto fetch = [&](int b, V8& qq) __attribute__((always_inline)) {
+    auto fetch = [&](int b, const RegionRecord* rec) __attribute__((always_inline)) {
         // lane-derived offsets are re-materialised here: hoisted out of the unit loop they would be
         // spilled, and the reload would sit in front of every fetch
         int ln = lane;
@@ -225,20 +247,28 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
         const int frow = wave * 16 + (ln >> 2);
         const int fc8 = (ln & 3) * 8;
         if (frow < N) {
-            const E* kp = row_ptr<MAPPED, E>(p.k, p.map, b, h, frow, fc8);
-            const E* vp = row_ptr<MAPPED, E>(p.v, p.map, b, h, frow, fc8);
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)kp,
-                                             (__attribute__((address_space(3))) void*)(lds_rawK + wave * 16 * 32), 16, 0, kStreamPolicy);
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)vp,
-                                             (__attribute__((address_space(3))) void*)(lds_rawV + wave * 16 * 32), 16, 0, kStreamPolicy);
+            dma16_to_lds(row_ptr<MAPPED, E>(p.k, p.map, b, h, frow, fc8), lds_address(lds_rawK + wave * 16 * 32));
+            dma16_to_lds(row_ptr<MAPPED, E>(p.v, p.map, b, h, frow, fc8), lds_address(lds_rawV + wave * 16 * 32));
+            dma16_to_lds(row_ptr<MAPPED, E>(p.q, p.map, b, h, frow, fc8), lds_address(lds_rawQ + wave * 16 * 32));
         }
-        qq = zero8<V8>();
-        const int fq = wave * 16 + (ln & 15);
-        if (fq < N) qq = ld8<V8>(row_ptr<MAPPED, E>(p.q, p.map, b, h, fq, 8 * (ln >> 4)));
+        if (REGIONS && rec != nullptr && ln < 5) {    // the ids of this wavefront's 16 rows (lanes 0 .. 3), the value (lane 4)
+            const void* src = ln < 4 ? (const void*)(rec->id + wave * 16 + 4 * ln) : (const void*)&rec->value;
+            dma4_to_lds(src, lds_address(lds_rawid + wave * 32));
+        }
     };
     // landing area -> tiles: K normalised and rounded to fp16, V as is (rows >= n stay zero)
-    auto stage = [&](int buf) __attribute__((always_inline)) {
+    f16x4 qop = {0, 0, 0, 0};   // query-side operand of the region product for the unit staged last
+    auto stage = [&](int buf, const RegionRecord* rec) __attribute__((always_inline)) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");    // this wavefront's rows have landed
+        if (REGIONS && rec != nullptr) {
+            int ln = lane;
+            asm volatile("" : "+v"(ln));
+            const float value = *reinterpret_cast<const float*>(lds_rawid + wave * 32 + 16);
+            qop = region_query_operand(value * kLog2e, lds_rawid[wave * 32 + (ln & 15)], ln >> 4);
+            if ((ln & 3) == 0)
+                st8<f16x8>(reinterpret_cast<_Float16*>(&lds_K[buf][(wave * 16 + (ln >> 2)) * S + 32]),
+                           region_key_entry(lds_rawid[wave * 32 + (ln >> 2)]));
+        }
         const V8 kk = ld8<V8>(lds_rawK + frow * 32 + fc8);
         const V8 vv = ld8<V8>(lds_rawV + frow * 32 + fc8);
         float x[8];
@@ -257,12 +287,15 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
 
     __syncthreads();                       // zero fill done
     Cursor c = first();
-    V8 qq = zero8<V8>();
     int tile_wi = -1;                      // window index the resident tile was built for
     if (!MASKED) build_tile(0);
+    // a region unit may skip the running maximum only if the row bound, which ignores the mask, cannot be
+    // further from the largest logit than the gap limit: the key with the largest bias may be one the mask removes
+    bool fast_reg = fast;
+    if (REGIONS && p.regions != nullptr) fast_reg = fast && !__syncthreads_or(2.f * scale2 + bias_range > kGapLimit);
     if (valid(c)) {
-        fetch(unit_of(c), qq);
-        stage(0);
+        fetch(unit_of(c), record_of(c));
+        stage(0, record_of(c));
     }
     __syncthreads();
     int cur = 0;
@@ -278,6 +311,8 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
         // ---- Q operand: normalise, fold s log2e, round to fp16 ----
         SV8 bq;
         {
+            // the rows landed before the previous unit's barrier (the first unit's before the one above)
+            const V8 qq = ld8<V8>(lds_rawQ + (wave * 16 + l16) * 32 + 8 * g);
             float x[8];
             unpack8(qq, x);
             float ss = 0.f;
@@ -288,7 +323,10 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
 #pragma unroll
             for (int j = 0; j < 8; j++) bq[j] = (SE)(x[j] * sc);
         }
-        if (more) fetch(unit_of(cn), qq);      // in flight while this unit is computed
+        const RegionRecord* rec = record_of(c);
+        const RegionRecord* rec_next = more ? record_of(cn) : nullptr;
+        const bool reg = REGIONS && rec != nullptr;
+        if (more) fetch(unit_of(cn), rec_next);      // in flight while this unit is computed
 
         const SE* Kb = &lds_K[cur][0];
         const E* Vb = &lds_V[cur][0];
@@ -301,12 +339,28 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
 
         // scores of keys 32 kp .. 32 kp + 31: MFMA tile A holds keys 8r/4 + r%4 in its rows r, tile B
         // the keys 4 further on, so that this lane's 8 values are keys 8g .. 8g+7 of the group
-        auto scores = [&](int kp, f32x4& s0, f32x4& s1) __attribute__((always_inline)) {
+        auto scores = [&](int kp, f32x4& s0, f32x4& s1, bool with_regions) __attribute__((always_inline)) {
             const int krow = 32 * kp + 8 * (l16 >> 2) + (l16 & 3);
             const SV8 a0 = ld8<SV8>(Kb + krow * S + 8 * g);
             const SV8 a1 = ld8<SV8>(Kb + (krow + 4) * S + 8 * g);
             s0 = Elem<kScoreDT>::mfma16(a0, bq, acc0[2 * kp]);
             s1 = Elem<kScoreDT>::mfma16(a1, bq, acc0[2 * kp + 1]);
+            if (REGIONS && with_regions) {
+                // the lane's offset is derived again here: hoisted out of the unit loop, the eight addresses
+                // (one per key group) would be spilled
+                int ln = lane;
+                asm volatile("" : "+v"(ln));
+                const _Float16* ko = reinterpret_cast<const _Float16*>(Kb) +
+                                     (32 * kp + 2 * (ln & 12) + (ln & 3)) * S + 32 + ((ln >> 2) & 4);
+                // read by hand: the compiler cannot tell these reads from the landing areas the fetch of the next
+                // unit is still writing, and would wait for that fetch in front of every one of them
+                f16x4 k0, k1;
+                asm volatile("ds_read_b64 %0, %2\n\tds_read_b64 %1, %2 offset:%3\n\ts_waitcnt lgkmcnt(0)"
+                             : "=&v"(k0), "=&v"(k1)
+                             : "v"((uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)ko), "n"(4 * S * 2));
+                s0 = region_mfma(k0, qop, s0);
+                s1 = region_mfma(k1, qop, s1);
+            }
         };
         // FAST: the row sum comes out of a third MFMA against a tile of ones, i.e. it sums the
         // ROUNDED P~ values that also enter the product with V: o is then an exact convex
@@ -331,52 +385,58 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
             }
         };
 
-        if (fast) {
+        // the loop in two copies, so that units without a region record run exactly the code they would run
+        // if there were no such units
+        auto tiles = [&](bool use_fast, bool with_regions) __attribute__((always_inline)) {
+            if (use_fast) {
 #pragma unroll
-            for (int kp = 0; kp < NT / 2; kp++) {
-                if (32 * kp < N) {
-                    f32x4 s0, s1;
-                    scores(kp, s0, s1);
+                for (int kp = 0; kp < NT / 2; kp++) {
+                    if (32 * kp < N) {
+                        f32x4 s0, s1;
+                        scores(kp, s0, s1, with_regions);
 #pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        s0[i] = fast_exp2(s0[i]);
-                        s1[i] = fast_exp2(s1[i]);
+                        for (int i = 0; i < 4; i++) {
+                            s0[i] = fast_exp2(s0[i]);
+                            s1[i] = fast_exp2(s1[i]);
+                        }
+                        pv(kp, s0, s1, true);
                     }
-                    pv(kp, s0, s1, true);
                 }
-            }
-        } else {
-            // fp16 (P would underflow against a mere bound) or a very large scale: the exact row maximum
-            // first, from a pass of score products alone; the matrix pipe has the room, and the second pass
-            // then needs no running maximum, no rescaling of o and no VALU row sum
-            float bm = -INFINITY;
+            } else {
+                // fp16 (P would underflow against a mere bound) or a very large scale: the exact row maximum
+                // first, from a pass of score products alone; the matrix pipe has the room, and the second pass
+                // then needs no running maximum, no rescaling of o and no VALU row sum
+                float bm = -INFINITY;
 #pragma unroll
-            for (int kp = 0; kp < NT / 2; kp++) {
-                if (32 * kp < N) {
-                    f32x4 s0, s1;
-                    scores(kp, s0, s1);
-                    bm = fmaxf(bm, fmaxf(fmaxf(s0[0], s0[1]), fmaxf(s0[2], s0[3])));
-                    bm = fmaxf(bm, fmaxf(fmaxf(s1[0], s1[1]), fmaxf(s1[2], s1[3])));
-                }
-            }
-            m_run = col_max(bm);
-            const float m_use = (m_run == -INFINITY) ? 0.f : m_run;
-#pragma unroll
-            for (int kp = 0; kp < NT / 2; kp++) {
-                if (32 * kp < N) {
-                    f32x4 s0, s1;
-                    scores(kp, s0, s1);
-#pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        s0[i] = fast_exp2(s0[i] - m_use);
-                        s1[i] = fast_exp2(s1[i] - m_use);
+                for (int kp = 0; kp < NT / 2; kp++) {
+                    if (32 * kp < N) {
+                        f32x4 s0, s1;
+                        scores(kp, s0, s1, with_regions);
+                        bm = fmaxf(bm, fmaxf(fmaxf(s0[0], s0[1]), fmaxf(s0[2], s0[3])));
+                        bm = fmaxf(bm, fmaxf(fmaxf(s1[0], s1[1]), fmaxf(s1[2], s1[3])));
                     }
-                    pv(kp, s0, s1, true);
+                }
+                m_run = col_max(bm);
+                const float m_use = (m_run == -INFINITY) ? 0.f : m_run;
+#pragma unroll
+                for (int kp = 0; kp < NT / 2; kp++) {
+                    if (32 * kp < N) {
+                        f32x4 s0, s1;
+                        scores(kp, s0, s1, with_regions);
+#pragma unroll
+                        for (int i = 0; i < 4; i++) {
+                            s0[i] = fast_exp2(s0[i] - m_use);
+                            s1[i] = fast_exp2(s1[i] - m_use);
+                        }
+                        pv(kp, s0, s1, true);
+                    }
                 }
             }
-        }
+        };
+        if (REGIONS && reg) tiles(fast_reg, true);
+        else tiles(fast, false);
 
-        if (more) stage(cur ^ 1);     // before the stores below, so the wait covers only the fetch
+        if (more) stage(cur ^ 1, rec_next);     // before the stores below, so the wait covers only the fetch
         // ---- normalise, write o (input dtype) and lse (natural log, fp32) ----
         const float l_tot = lacc[0];
         const float inv_l = l_tot > 0.f ? 1.0f / l_tot : 0.f;
@@ -406,6 +466,8 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
 int forward_resident_supported(int n) { return n >= 1 && n <= 256; }
 #endif
 
+constexpr int kRegionMaxImages = 32;     // images per window up to which region records are used (see launch_map)
+
 template <class K>
 static int resident_fit(K kern, int threads) {
     int n = 0;
@@ -426,6 +488,11 @@ static hipError_t launch_map(FwdParams p, hipStream_t st) {
         if (groups > p.bw) groups = p.bw;
         return groups;
     };
+    // Windows whose mask has region form can ride in the first launch, which saves the second launch its tile
+    // rebuilds and its uneven split of few units: measured on the 256-token benchmark shape that is 25 % of the
+    // forward time at 2 images per window, 8 % at 8, nothing at 32 and a loss of 3 % at 64, where the second
+    // launch has enough units per workgroup to hide both.
+    if (p.regions != nullptr && p.bw / p.n_windows > kRegionMaxImages) p.regions = nullptr;
     // units with an all-zero mask (or every unit when there is no mask) ...
     if (MASK_DT < 0 || p.mask_live != nullptr) {
         p.groups = groups_for(fit_plain);

@@ -73,7 +73,11 @@ def tensor_version(t):
 
 
 def mask_window_flags(mask):
-    """uint8[nW]: 1 where a window's mask has a non-zero entry (device tensor).
+    """uint8[nW] device tensor of per-window flags: 0 where a window's mask is all zero, bit 0 where it has a
+    non-zero entry, bit 1 where it only removes keys and never a whole row, bit 2 where it is exactly
+    c * [id_i != id_j] (what the reference's builder produces, swin_transformer_v2.py:386-405).  For the last
+    kind the scan also fills one record per window (c and the N ids), kept on the returned tensor as
+    `_fwa2_regions` and handed to the library with the flags.
     Cached on the mask tensor object, keyed by its storage address and in-place modification counter, so a
     mask edited in place or re-pointed at other memory (`mask.data = ...`) is scanned again.  Two cases are
     never cached and scan on every call: a mask created under torch.inference_mode, which tracks no
@@ -87,10 +91,12 @@ def mask_window_flags(mask):
         return cached[1]
     lib = _abi.load()
     live = torch.empty(mask.shape[0], dtype=torch.uint8, device=mask.device)
+    regions = torch.empty(mask.shape[0] * _abi.MASK_REGION_BYTES, dtype=torch.uint8, device=mask.device)
     with _on_device(mask.device) as stream:
-        st = lib.fwa2_mask_scan(mask.data_ptr(), _DTYPES[mask.dtype], mask.shape[0], mask.shape[1], mask.stride(0),
-                                mask.stride(1), live.data_ptr(), stream)
-    _abi.check(st, "fwa2_mask_scan")
+        st = lib.fwa2_mask_scan_regions(mask.data_ptr(), _DTYPES[mask.dtype], mask.shape[0], mask.shape[1],
+                                        mask.stride(0), mask.stride(1), live.data_ptr(), regions.data_ptr(), stream)
+    _abi.check(st, "fwa2_mask_scan_regions")
+    live._fwa2_regions = regions
     if version is not None and not torch.cuda.is_current_stream_capturing():
         try:
             mask._fwa2_live = (key, live)
@@ -123,6 +129,9 @@ def _describe(q, k, v, o, lse, logit_scale, bias, mask, mask_live, scale_type, w
         p.mask_dtype = _DTYPES[mask.dtype]
         if mask_live is not None:
             p.mask_live = mask_live.data_ptr()
+            regions = getattr(mask_live, "_fwa2_regions", None)
+            if regions is not None:
+                p.mask_regions = regions.data_ptr()
     else:
         p.mask_dtype = p.dtype
     p.lse = lse.data_ptr()

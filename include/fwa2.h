@@ -40,7 +40,7 @@
 extern "C" {
 #endif
 
-#define FWA2_ABI_VERSION 2
+#define FWA2_ABI_VERSION 3
 
 typedef enum fwa2_status {
     FWA2_OK = 0,
@@ -141,6 +141,12 @@ typedef struct fwa2_problem {
      */
     int32_t n_keys;
     int32_t reserved0;       /* must be 0 */
+
+    const void* mask_regions;/* optional [nW] records of FWA2_MASK_REGION_BYTES each from fwa2_mask_scan_regions,
+                                given together with the mask_live it filled; NULL = none.  A window flagged there
+                                as having region form is then computed from its record (N bytes) instead of its
+                                N x N mask entries, by the kernels for windows of up to 256 tokens at head
+                                dimension 32; everywhere else the record is ignored and the mask is read */
 } fwa2_problem;
 
 /* Library / ABI identification.  Returns FWA2_ABI_VERSION. */
@@ -172,6 +178,20 @@ int fwa2_validate(const fwa2_problem* p, int backward);
  */
 int fwa2_mask_scan(const void* mask, int mask_dtype, int n_windows, int n, int64_t stride_w, int64_t stride_n,
                    uint8_t* live, void* stream);
+
+/*
+ * fwa2_mask_scan that also recognises the form the reference's mask builder produces
+ * (flash_win_attn_v2/swin_transformer_v2.py:386-405: region ids painted on the shifted grid, then
+ * mask[w][i][j] = -100 where id_i != id_j, 0 elsewhere).  For a window of n <= 256 tokens whose mask is EXACTLY
+ * c * [id_i != id_j] for one finite c < 0 and at most 8 distinct ids (every entry is compared), bit 2 of live[w]
+ * is set as well and regions[w] receives c and the n ids; such a window is then attended from those n bytes
+ * (see fwa2_problem.mask_regions).  Any other mask keeps bit 2 clear and is read entry by entry as before, so the
+ * result is the same for every mask.  `regions` is device memory of n_windows * FWA2_MASK_REGION_BYTES bytes,
+ * 16-byte aligned; its layout is private to the library.  Has no counterpart in the reference.
+ */
+#define FWA2_MASK_REGION_BYTES 272
+int fwa2_mask_scan_regions(const void* mask, int mask_dtype, int n_windows, int n, int64_t stride_w, int64_t stride_n,
+                           uint8_t* live, void* regions, void* stream);
 
 /*
  * Bytes of device scratch fwa2_backward needs for this problem on the CURRENT
