@@ -55,6 +55,8 @@ __global__ void __launch_bounds__(64 * NT / SUB) bwd_dq_resident_kernel(const Bw
     __shared__ __attribute__((aligned(16))) E lds_rawV[ROWS * 32];
     __shared__ __attribute__((aligned(16))) E lds_rawQ[ROWS * 32];   // this wavefront's 16 query rows
     __shared__ __attribute__((aligned(16))) E lds_rawDO[ROWS * 32];
+    __shared__ __attribute__((aligned(16))) float lds_rawLse[ROWS];  // lse and delta of the same rows
+    __shared__ __attribute__((aligned(16))) float lds_rawDelta[ROWS];
     __shared__ uint8_t lds_live[kLiveCache];
     __shared__ uint16_t lds_list[kLiveCache];
     __shared__ int lds_count;
@@ -64,7 +66,7 @@ __global__ void __launch_bounds__(64 * NT / SUB) bwd_dq_resident_kernel(const Bw
     const int tid = threadIdx.x;
     const int nthreads = blockDim.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);      // uniform: lives in a scalar register
     const int l16 = lane & 15;
     const int g = lane >> 4;
 
@@ -215,12 +217,12 @@ __global__ void __launch_bounds__(64 * NT / SUB) bwd_dq_resident_kernel(const Bw
 
     // ---- per-unit fetch: the wavefront's WR rows of k, v (which it will stage) and of q, dO (its own
     // queries) by DMA, 16 rows per instruction; lse and delta of its queries in registers ----
-    struct Row { float lse[SUB], delta[SUB]; };
+    // issued by hand (see dma16_to_lds): the compiler would otherwise wait for the whole fetch in front of the
+    // first transposing LDS read of every unit, which it cannot tell from the landing areas
     auto dma16 = [&](const E* src, E* lds_wave_base) __attribute__((always_inline)) {
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                         (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, kStreamPolicy);
+        dma16_to_lds(src, lds_address(lds_wave_base));
     };
-    auto fetch = [&](int b, Row& r) __attribute__((always_inline)) {
+    auto fetch = [&](int b) __attribute__((always_inline)) {
         // lane-derived offsets are re-materialised here: hoisted out of the unit loop they would occupy
         // a dozen registers for the whole kernel
         int ln = lane;
@@ -237,12 +239,12 @@ __global__ void __launch_bounds__(64 * NT / SUB) bwd_dq_resident_kernel(const Bw
                 dma16(row_ptr<MAPPED, E>(p.d_o, p.map, b, h, frow, fc8),
                       lds_rawDO + row0 * 32);
             }
-            const int q = row0 + (ln & 15);
-            r.lse[u] = -INFINITY; r.delta[u] = 0.f;
-            if (q < N) {
-                r.lse[u] = p.lse[b * p.lse_sb + h * p.lse_sh + q];
-                r.delta[u] = p.delta[((int64_t)b * p.heads + h) * p.delta_stride + q];
-            }
+        }
+        // lse and delta of the wavefront's rows, one row per lane
+        const int q = wave * WR + ln;
+        if (ln < WR && q < N) {
+            dma4_to_lds(p.lse + b * p.lse_sb + h * p.lse_sh + q, lds_address(lds_rawLse + wave * WR));
+            dma4_to_lds(p.delta + ((int64_t)b * p.heads + h) * p.delta_stride + q, lds_address(lds_rawDelta + wave * WR));
         }
     };
     auto stage = [&](int buf) __attribute__((always_inline)) {
@@ -272,11 +274,8 @@ __global__ void __launch_bounds__(64 * NT / SUB) bwd_dq_resident_kernel(const Bw
     Cursor c = first();
     int tile_wi = -1;                      // window index the resident tile was built for
     if (!MASKED) build_tile(0);
-    Row row;
-#pragma unroll
-    for (int u = 0; u < SUB; u++) { row.lse[u] = -INFINITY; row.delta[u] = 0.f; }
     if (valid(c)) {
-        fetch(unit_of(c), row);
+        fetch(unit_of(c));
         stage(0);
     }
     __syncthreads();
@@ -302,6 +301,8 @@ __global__ void __launch_bounds__(64 * NT / SUB) bwd_dq_resident_kernel(const Bw
             // the rows landed before the previous unit's barrier (the first unit's before the one above)
             const V8 qcur = ld8<V8>(lds_rawQ + (wave * WR + 16 * u + l16) * 32 + 8 * g);
             const V8 docur = ld8<V8>(lds_rawDO + (wave * WR + 16 * u + l16) * 32 + 8 * g);
+            const float lse_q = qv[u] ? lds_rawLse[wave * WR + 16 * u + l16] : -INFINITY;
+            const float delta_q = qv[u] ? lds_rawDelta[wave * WR + 16 * u + l16] : 0.f;
             float x[8];
             unpack8(qcur, x);
             float ss = 0.f;
@@ -313,22 +314,22 @@ __global__ void __launch_bounds__(64 * NT / SUB) bwd_dq_resident_kernel(const Bw
 #pragma unroll
             for (int j = 0; j < 8; j++) bq[u][j] = (SE)(x[j] * sc);
             // fully masked row (lse = -inf): P = 0
-            nl[u] = (row.lse[u] == -INFINITY) ? -INFINITY : m_fixed[u] - row.lse[u] * kLog2e;
+            nl[u] = (lse_q == -INFINITY) ? -INFINITY : m_fixed[u] - lse_q * kLog2e;
             float nd;
             if (fold) {
                 const float w = fast_exp2(nl[u]);
 #pragma unroll
                 for (int j = 0; j < 8; j++) bd[u][j] = (E)((float)docur[j] * w);
-                nd = -row.delta[u] * w;
+                nd = -delta_q * w;
                 nl[u] = 0.f;
             } else {
                 bd[u] = docur;
-                nd = -row.delta[u];
+                nd = -delta_q;
             }
 #pragma unroll
             for (int i = 0; i < 4; i++) { dqacc[u][0][i] = 0.f; dqacc[u][1][i] = 0.f; ndv[u][i] = nd; }
         }
-        if (more) fetch(unit_of(cn), row);      // in flight while this unit is computed
+        if (more) fetch(unit_of(cn));      // in flight while this unit is computed
 
         const SE* Kb = &lds_K[cur][0];
         const E* Vb = &lds_V[cur][0];
