@@ -62,7 +62,7 @@ class Problem(ctypes.Structure):
         ("grid_h", ctypes.c_int32), ("grid_w", ctypes.c_int32),
         ("win_h", ctypes.c_int32), ("win_w", ctypes.c_int32),
         ("shift_h", ctypes.c_int32), ("shift_w", ctypes.c_int32),
-        ("n_keys", ctypes.c_int32), ("reserved0", ctypes.c_int32),
+        ("n_keys", ctypes.c_int32), ("scale_head_dim", ctypes.c_int32),
         ("mask_regions", ctypes.c_void_p),
     ]
 

@@ -131,7 +131,9 @@ int validate(const fwa2_problem* p, int backward) {
                 return fail(FWA2_ERR_UNSUPPORTED, "a unit spans more than 2^31 bytes (rows %lld, row stride %lld)", (long long)rows,
                             (long long)ts[i]->stride_n);
     }
-    if (p->n_keys < 0 || p->reserved0 != 0) return fail(FWA2_ERR_INVALID_ARGUMENT, "n_keys must not be negative, reserved0 must be 0");
+    if (p->n_keys < 0) return fail(FWA2_ERR_INVALID_ARGUMENT, "n_keys must not be negative");
+    if (p->scale_head_dim < 0 || p->scale_head_dim > p->head_dim)
+        return fail(FWA2_ERR_INVALID_ARGUMENT, "scale_head_dim must be 0 or a dimension up to head_dim (rows padded with zeros)");
     const int nk = p->n_keys > 0 ? p->n_keys : p->n;
     if (p->bias.ptr && p->bias.stride_n < nk)
         return fail(FWA2_ERR_INVALID_ARGUMENT, "bias: row stride %lld < number of keys", (long long)p->bias.stride_n);
@@ -300,7 +302,7 @@ int fwa2_forward(const fwa2_problem* p) {
     k.lse = p->lse; k.lse_sb = p->lse_stride_bw; k.lse_sh = p->lse_stride_h;
     k.bw = p->bw; k.heads = p->heads; k.n = p->n; k.n_windows = p->mask.ptr ? p->n_windows : 1;
     k.scale_kind = p->scale_kind;
-    k.default_scale = 1.0f / sqrtf((float)p->head_dim);
+    k.default_scale = 1.0f / sqrtf((float)(p->scale_head_dim > 0 ? p->scale_head_dim : p->head_dim));
     k.side_vec = (!p->bias.ptr || row_vec_ok(p->bias.ptr, p->bias.stride_a, p->bias.stride_n, p->n)) &&
                  (!p->mask.ptr || row_vec_ok(p->mask.ptr, p->mask.stride_a, p->mask.stride_n, p->n));
     k.cus = cu_count();
@@ -332,7 +334,7 @@ static int run_backward(const fwa2_problem* p) {
     k.lse = p->lse; k.lse_sb = p->lse_stride_bw; k.lse_sh = p->lse_stride_h;
     k.bw = p->bw; k.heads = p->heads; k.n = p->n; k.n_windows = p->mask.ptr ? p->n_windows : 1;
     k.scale_kind = p->scale_kind;
-    k.default_scale = 1.0f / sqrtf((float)p->head_dim);
+    k.default_scale = 1.0f / sqrtf((float)(p->scale_head_dim > 0 ? p->scale_head_dim : p->head_dim));
     k.dbias = p->dbias; k.dscale = p->dscale;
     k.side_vec = (!p->bias.ptr || row_vec_ok(p->bias.ptr, p->bias.stride_a, p->bias.stride_n, p->n)) &&
                  (!p->mask.ptr || row_vec_ok(p->mask.ptr, p->mask.stride_a, p->mask.stride_n, p->n));

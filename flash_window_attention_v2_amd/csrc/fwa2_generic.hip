@@ -726,7 +726,7 @@ hipError_t launch_generic(const fwa2_problem* pr, bool backward) {
     }
     p.logit_scale = pr->logit_scale;
     p.scale_kind = pr->scale_kind;
-    p.default_scale = 1.0f / sqrtf((float)pr->head_dim);
+    p.default_scale = 1.0f / sqrtf((float)(pr->scale_head_dim > 0 ? pr->scale_head_dim : pr->head_dim));
     p.bias = pr->bias.ptr; p.bias_sh = pr->bias.stride_a; p.bias_sn = pr->bias.stride_n;
     p.mask = pr->mask.ptr; p.mask_sw = pr->mask.stride_a; p.mask_sn = pr->mask.stride_n;
     p.mask_f32 = pr->mask.ptr && pr->mask_dtype == FWA2_F32;

@@ -105,9 +105,10 @@ def mask_window_flags(mask):
     return live
 
 
-def _describe(q, k, v, o, lse, logit_scale, bias, mask, mask_live, scale_type, window_map=None):
+def _describe(q, k, v, o, lse, logit_scale, bias, mask, mask_live, scale_type, window_map=None, scale_dim=0):
     bw, heads, n, d = q.shape
     p = _abi.new_problem()
+    p.scale_head_dim = scale_dim
     if window_map is not None:
         # q, k, v, o are token grids [B, H, gh * gw, d]; the library partitions them into windows
         (gh, gw), (wh, ww), (sh, sw) = window_map
@@ -163,10 +164,22 @@ def _check_inputs(q, k, v, logit_scale, bias, mask, scale_type):
             "mask must be [nW, N, N_k] with BW % nW == 0"
 
 
-def _flash_attn_forward(q, k, v, logit_scale, bias=None, mask=None, scale_type="scalar"):
+def _pad8(x):
+    """Rows padded with zeros to the next multiple of 8 elements (a new contiguous tensor)."""
+    return torch.nn.functional.pad(x, (0, -x.shape[-1] % 8))
+
+
+def _flash_attn_forward(q, k, v, logit_scale, bias=None, mask=None, scale_type="scalar", _scale_dim=0):
     """(o, lse, logit_scale) as the reference's launcher returns them (attn_kernel_forward.py:261-345):
-    o like q, lse fp32 [BW, H, ceil(N / 64) * 64] holding the natural-log normaliser of every query row."""
+    o like q, lse fp32 [BW, H, ceil(N / 64) * 64] holding the natural-log normaliser of every query row.
+    A head dimension that is not a multiple of 8 runs on zero-padded copies (the reference pads inside its
+    kernels, attn_kernel_forward.py:267,298): zero columns change neither the norms nor the products, and the
+    default scale keeps referring to the true dimension."""
     _check_inputs(q, k, v, logit_scale, bias, mask, scale_type)
+    d = q.shape[-1]
+    if d % 8:
+        o, lse, logit_scale = _flash_attn_forward(_pad8(q), _pad8(k), _pad8(v), logit_scale, bias, mask, scale_type, d)
+        return o[..., :d].contiguous(), lse, logit_scale
     q, k, v = (_kernel_ready(x) for x in (q, k, v))
     if scale_type == "tensor" and not logit_scale.is_contiguous():
         logit_scale = logit_scale.contiguous()
@@ -183,7 +196,7 @@ def _flash_attn_forward(q, k, v, logit_scale, bias=None, mask=None, scale_type="
         return o, lse, logit_scale
     if not _rows_16b_aligned(o):
         o = torch.empty(q.shape, device=q.device, dtype=q.dtype)
-    p = _describe(q, k, v, o, lse, logit_scale, bias, mask, _flags_for(mask), scale_type)
+    p = _describe(q, k, v, o, lse, logit_scale, bias, mask, _flags_for(mask), scale_type, scale_dim=_scale_dim)
     with _on_device(q.device) as stream:
         p.stream = stream
         _abi.check(lib.fwa2_forward(p), "fwa2_forward")
@@ -191,13 +204,22 @@ def _flash_attn_forward(q, k, v, logit_scale, bias=None, mask=None, scale_type="
 
 
 def _flash_attn_backward(do, q, k, v, logit_scale, o, lse, dq, dk, dv, dscale, db, bias=None, mask=None,
-                         scale_type="scalar"):
+                         scale_type="scalar", _scale_dim=0):
     """Fills dq, dk, dv (and dscale, db when given) in place, as the reference's launcher does
     (attn_kernel_backward.py:567-711); dscale already carries the clamp mask (l <= ln 100)."""
     if q.shape[0] == 0:     # an empty batch: the sums over units are empty
         for t in (db, dscale):
             if t is not None:
                 t.zero_()
+        return
+    d = q.shape[-1]
+    if d % 8:               # zero-padded copies, as in the forward; the gradients of the pad columns are dropped
+        padded = [_pad8(x) for x in (do, q, k, v, o)]
+        grads = [torch.empty_like(padded[i]) for i in (1, 2, 3)]
+        _flash_attn_backward(padded[0], padded[1], padded[2], padded[3], logit_scale, padded[4], lse, *grads, dscale, db,
+                             bias=bias, mask=mask, scale_type=scale_type, _scale_dim=d)
+        for given, used in zip((dq, dk, dv), grads):
+            given.copy_(used[..., :d])
         return
     do, q, k, v, o = (_kernel_ready(x) for x in (do, q, k, v, o))
     if bias is not None and bias.stride(-1) != 1:
@@ -213,7 +235,7 @@ def _flash_attn_backward(do, q, k, v, logit_scale, o, lse, dq, dk, dv, dscale, d
     ds_k = dscale if dscale is None or dscale.is_contiguous() else torch.empty(dscale.shape, device=dscale.device,
                                                                                dtype=dscale.dtype)
     lib = _abi.load()
-    p = _describe(q, k, v, o, lse, logit_scale, bias, mask, _flags_for(mask), scale_type)
+    p = _describe(q, k, v, o, lse, logit_scale, bias, mask, _flags_for(mask), scale_type, scale_dim=_scale_dim)
     _set_t4(p.d_o, do); _set_t4(p.dq, outs[0]); _set_t4(p.dk, outs[1]); _set_t4(p.dv, outs[2])
     if db_k is not None:
         p.dbias = db_k.data_ptr()

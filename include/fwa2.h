@@ -90,7 +90,7 @@ typedef struct fwa2_problem {
     int32_t bw;              /* batch * windows-per-image */
     int32_t heads;
     int32_t n;               /* tokens per window (queries == keys) */
-    int32_t head_dim;        /* multiple of 8, at most 128; 32 runs on the tuned kernels */
+    int32_t head_dim;        /* multiple of 8, at most 128 (see scale_head_dim for others); 32 runs on the tuned kernels */
     int32_t n_windows;       /* leading extent of mask; window of row b is b % n_windows; 1 if no mask */
 
     fwa2_tensor4 q, k, v;    /* inputs */
@@ -140,7 +140,13 @@ typedef struct fwa2_problem {
      * kernels that also serve head dimensions other than 32; not combined with a window map.
      */
     int32_t n_keys;
-    int32_t reserved0;       /* must be 0 */
+    /*
+     * Head dimension the default scale 1/sqrt(d) refers to, for rows that were zero-padded up to a multiple of 8
+     * (the reference pads to the next power of two inside its kernels and keeps 1/sqrt(d) of the true d,
+     * attn_kernel_forward.py:267,298; flash_window_attention_v2.py:14-17); 0 = head_dim.  Zero columns change
+     * neither the normalised vectors nor the products, so a caller may pad q, k, v, d_o and slice o, dq, dk, dv.
+     */
+    int32_t scale_head_dim;
 
     const void* mask_regions;/* optional [nW] records of FWA2_MASK_REGION_BYTES each from fwa2_mask_scan_regions,
                                 given together with the mask_live it filled; NULL = none.  A window flagged there

@@ -86,8 +86,10 @@ def test_validate_accepts_and_rejects(lib):
     p.bw = 8
     assert lib.fwa2_validate(p, 0) == _abi.ERR_UNSUPPORTED and b"window map" in lib.fwa2_last_error()
     p = _good_problem()
-    p.reserved0 = 1
-    assert lib.fwa2_validate(p, 0) == _abi.ERR_INVALID_ARGUMENT
+    p.scale_head_dim = 20       # rows of 20 elements padded with zeros to 32: legal
+    assert lib.fwa2_validate(p, 0) == _abi.OK
+    p.scale_head_dim = 40       # more than the rows hold
+    assert lib.fwa2_validate(p, 0) == _abi.ERR_INVALID_ARGUMENT and b"scale_head_dim" in lib.fwa2_last_error()
 
     p = _good_problem()
     p.q = _abi.Tensor4(0x10002, 4096, 2048, 32)  # rows not 16-byte aligned

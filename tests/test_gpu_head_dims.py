@@ -43,11 +43,25 @@ def test_head_dim_64_ragged_window_fp32_mask_and_clamped_scale():
     _run_and_check(inp, torch.bfloat16, tag="ragged", dscale_l1_frac=0.1)
 
 
-def test_head_dim_must_be_a_multiple_of_8():
-    from flash_window_attention_v2_amd import flash_win_attn_v2_func
-    q = torch.randn(2, 2, 16, 20, device="cuda", dtype=torch.bfloat16)
-    with pytest.raises(NotImplementedError, match="multiples of 8"):
-        flash_win_attn_v2_func(q, q, q)
+@pytest.mark.parametrize("d,with_scale", [(20, True), (20, False), (12, False), (36, True), (100, False), (5, True)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_head_dims_that_are_not_multiples_of_8(d, with_scale, dtype):
+    """Any head dimension up to 128 (attn_kernel_forward.py:267, 298): the launchers run these on zero-padded
+    rows.  Without a logit scale the default 1/sqrt(d) must keep referring to the true d, not to the padded one
+    (d = 12 padded to 16 would otherwise be off by 13 % in every logit)."""
+    inp = make_inputs(batch=2, n_windows=4, heads=2, n=64, d=d, dtype=dtype, seed=d, resolution=16, window=8, shift=4,
+                      with_scale=with_scale)
+    _run_and_check(inp, dtype, tag=f"d{d}")
+
+
+def test_the_library_itself_takes_multiples_of_8_only():
+    """Below the Python launchers the C ABI refuses such a head dimension instead of reading past the rows."""
+    from flash_window_attention_v2_amd import _abi
+    from tests.test_abi import _good_problem
+    lib = _abi.load()
+    p = _good_problem()
+    p.head_dim = 20
+    assert lib.fwa2_validate(p, 0) == _abi.ERR_UNSUPPORTED and b"multiples of 8" in lib.fwa2_last_error()
 
 
 @pytest.mark.parametrize("nq,nk,d", [(64, 96, 32), (100, 49, 32), (49, 128, 64), (300, 64, 32), (37, 290, 16)])
