@@ -215,10 +215,11 @@ __device__ __forceinline__ void unit_blocks(BwdLds<DT, NQB>& L, WaveRegs<DT, NQB
 // a workgroup then belongs to one (head, query chunk, key chunk), reads only those rows, keeps that
 // tile of dbias in registers and writes its share of dk / dv (already taken back through the
 // normalisation, which is linear) as fp32 partials that dkv_reduce_kernel sums over the query chunks.
-// MAPPED: rows are addressed through the window map (cyclic shift + window partition done here; not with BIG).
+// MAPPED: rows are addressed through the window map (cyclic shift + window partition done here).  BIG decides that
+// at run time (p.map.nw > 0): its row fetches are a small part of a super-tile's work.
 template <int DT, bool HAS_BIAS, int MASK_DT, int NQB, int KT, int MODE, bool BIG, bool MAPPED = false>
 __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) {
-    static_assert(!(MAPPED && BIG), "the window map is limited to windows one workgroup holds");
+    static_assert(!(MAPPED && BIG), "with BIG the map is a run-time property (p.map.nw > 0)");
     typedef typename Elem<DT>::E E;
     typedef typename Elem<DT>::V8 V8;
     typedef typename Elem<DT>::V4 V4;
@@ -375,6 +376,19 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
                 }
                 continue;
             }
+            if constexpr (BIG) {
+                if (p.map.nw > 0) {
+                    if (r < N) {
+                        const int pos = unit_row<true>(p.map, b, q_off + r);
+                        async_row_chunk(row_at(unit_ptr<true, E>(p.q, p.map, b, h), pos, p.q.sn, dc), L.rawQ + row0 * 32);
+                        async_row_chunk(row_at(unit_ptr<true, E>(p.d_o, p.map, b, h), pos, p.d_o.sn, dc), L.rawDO + row0 * 32);
+                        async_row_chunk(row_at(unit_ptr<true, E>(p.o, p.map, b, h), pos, p.o.sn, dc), L.rawO + row0 * 32);
+                    }
+                    if (r < NK)
+                        async_row_chunk(row_ptr<true, E>(p.k, p.map, b, h, k_off + r, dc), L.rawK + row0 * 32);
+                    continue;
+                }
+            }
             if (r < N) {
                 async_row_chunk(row_at(qptr, r, p.q.sn, dc), L.rawQ + row0 * 32);
                 async_row_chunk(row_at(doptr, r, p.d_o.sn, dc), L.rawDO + row0 * 32);
@@ -390,6 +404,12 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
             if constexpr (MAPPED) {
                 if (r < NK) async_row_chunk(row_ptr<true, E>(p.v, p.map, b, h, r, dc), L.rawV + row0 * 32);
                 continue;
+            }
+            if constexpr (BIG) {
+                if (p.map.nw > 0) {
+                    if (r < NK) async_row_chunk(row_ptr<true, E>(p.v, p.map, b, h, k_off + r, dc), L.rawV + row0 * 32);
+                    continue;
+                }
             }
             if (r < NK) async_row_chunk(row_at(vptr, r, p.v.sn, dc), L.rawV + row0 * 32);
         }
@@ -659,8 +679,8 @@ __global__ void __launch_bounds__(256) dkv_reduce_kernel(const BwdParams p) {
     V8 ok, ov;
 #pragma unroll
     for (int j = 0; j < 8; j++) { ok[j] = (E)sk[j]; ov[j] = (E)sv[j]; }
-    st8<V8>(reinterpret_cast<E*>(const_cast<void*>(p.dk.ptr)) + b * p.dk.sb + h * p.dk.sh + (int64_t)key * p.dk.sn + c8, ok);
-    st8<V8>(reinterpret_cast<E*>(const_cast<void*>(p.dv.ptr)) + b * p.dv.sb + h * p.dv.sh + (int64_t)key * p.dv.sn + c8, ov);
+    st8<V8>(reinterpret_cast<E*>(const_cast<void*>(p.dk.ptr)) + row_off_any(p.dk, p.map, (int)b, h, key) + c8, ok);
+    st8<V8>(reinterpret_cast<E*>(const_cast<void*>(p.dv.ptr)) + row_off_any(p.dv, p.map, (int)b, h, key) + c8, ov);
 }
 
 // ---- host side -----------------------------------------------------------------
@@ -833,9 +853,10 @@ static hipError_t launch_main(BwdParams p, const BwdPlan& pl, hipStream_t st, in
 
 template <int DT, bool HAS_BIAS, int MASK_DT>
 static hipError_t launch_nqb(const BwdParams& p, const BwdPlan& pl, hipStream_t st, int* groups_out) {
-    if (p.map.nw > 0) {
-        // windows of up to 64 tokens with a map go to the fused kernel, longer than 256 are refused earlier
-        if (pl.n_chunks > 1 || pl.nqb_t == 2) return hipErrorInvalidValue;
+    if (p.map.nw > 0 && pl.n_chunks == 1) {
+        // windows of up to 64 tokens with a map go to the fused kernel; those of more than 256 run on the
+        // super-tiled form below, which reads the map at run time
+        if (pl.nqb_t == 2) return hipErrorInvalidValue;
         if (pl.nqb_t == 4) return launch_main<DT, HAS_BIAS, MASK_DT, 4, 1, false, true>(p, pl, st, groups_out);
         if (pl.kt == 1) return launch_main<DT, HAS_BIAS, MASK_DT, 5, 1, false, true>(p, pl, st, groups_out);
         return launch_main<DT, HAS_BIAS, MASK_DT, 8, 2, false, true>(p, pl, st, groups_out);

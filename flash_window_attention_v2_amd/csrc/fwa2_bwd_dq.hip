@@ -55,12 +55,13 @@ __global__ void __launch_bounds__(512) bwd_dq_kernel(const BwdParams p) {
     const int h = idx % p.heads;
     const int b = idx / p.heads;
 
-    const E* qptr = reinterpret_cast<const E*>(p.q.ptr) + b * p.q.sb + h * p.q.sh;
-    const E* kptr = reinterpret_cast<const E*>(p.k.ptr) + b * p.k.sb + h * p.k.sh;
-    const E* vptr = reinterpret_cast<const E*>(p.v.ptr) + b * p.v.sb + h * p.v.sh;
-    const E* optr = reinterpret_cast<const E*>(p.o.ptr) + b * p.o.sb + h * p.o.sh;
-    const E* doptr = reinterpret_cast<const E*>(p.d_o.ptr) + b * p.d_o.sb + h * p.d_o.sh;
-    E* dqptr = reinterpret_cast<E*>(const_cast<void*>(p.dq.ptr)) + b * p.dq.sb + h * p.dq.sh;
+    // rows are addressed through the window map when there is one (cyclic shift + window partition done here)
+    const E* qbase = reinterpret_cast<const E*>(p.q.ptr);
+    const E* kbase = reinterpret_cast<const E*>(p.k.ptr);
+    const E* vbase = reinterpret_cast<const E*>(p.v.ptr);
+    const E* obase = reinterpret_cast<const E*>(p.o.ptr);
+    const E* dobase = reinterpret_cast<const E*>(p.d_o.ptr);
+    E* dqbase = reinterpret_cast<E*>(const_cast<void*>(p.dq.ptr));
 
     float s_true;
     if (p.scale_kind == FWA2_SCALE_TENSOR) {
@@ -83,12 +84,15 @@ __global__ void __launch_bounds__(512) bwd_dq_kernel(const BwdParams p) {
     if (wave_live) {
         V8 a = zero8<V8>(), c = zero8<V8>(), o0 = zero8<V8>(), o1 = zero8<V8>();
         if (qv) {
-            a = ld8<V8>(qptr + (int64_t)qi * p.q.sn + 8 * hf);
-            c = ld8<V8>(qptr + (int64_t)qi * p.q.sn + 16 + 8 * hf);
-            bd0 = ld8<V8>(doptr + (int64_t)qi * p.d_o.sn + 8 * hf);
-            bd1 = ld8<V8>(doptr + (int64_t)qi * p.d_o.sn + 16 + 8 * hf);
-            o0 = ld8<V8>(optr + (int64_t)qi * p.o.sn + 8 * hf);
-            o1 = ld8<V8>(optr + (int64_t)qi * p.o.sn + 16 + 8 * hf);
+            const E* qrow = qbase + row_off_any(p.q, p.map, b, h, qi);
+            const E* dorow = dobase + row_off_any(p.d_o, p.map, b, h, qi);
+            const E* orow = obase + row_off_any(p.o, p.map, b, h, qi);
+            a = ld8<V8>(qrow + 8 * hf);
+            c = ld8<V8>(qrow + 16 + 8 * hf);
+            bd0 = ld8<V8>(dorow + 8 * hf);
+            bd1 = ld8<V8>(dorow + 16 + 8 * hf);
+            o0 = ld8<V8>(orow + 8 * hf);
+            o1 = ld8<V8>(orow + 16 + 8 * hf);
             const float l = p.lse[b * p.lse_sb + h * p.lse_sh + qi];
             nlse2 = (l == -INFINITY) ? -INFINITY : -l * kLog2e;   // fully masked row: P = 0
         }
@@ -131,8 +135,8 @@ __global__ void __launch_bounds__(512) bwd_dq_kernel(const BwdParams p) {
             const int dch = (tid & 3) * 8;
             V8 kk = zero8<V8>(), vv = zero8<V8>();
             if (r < rows) {
-                kk = ld8<V8>(kptr + (int64_t)(c0 + r) * p.k.sn + dch);
-                vv = ld8<V8>(vptr + (int64_t)(c0 + r) * p.v.sn + dch);
+                kk = ld8<V8>(kbase + row_off_any(p.k, p.map, b, h, c0 + r) + dch);
+                vv = ld8<V8>(vbase + row_off_any(p.v, p.map, b, h, c0 + r) + dch);
             }
             float x[8];
             unpack8(kk, x);
@@ -215,7 +219,7 @@ __global__ void __launch_bounds__(512) bwd_dq_kernel(const BwdParams p) {
             V4 q4;
 #pragma unroll
             for (int j = 0; j < 4; j++) q4[j] = 0;
-            if (qv) q4 = *reinterpret_cast<const V4*>(qptr + (int64_t)qi * p.q.sn + 8 * c + 4 * hf);
+            if (qv) q4 = *reinterpret_cast<const V4*>(qbase + row_off_any(p.q, p.map, b, h, qi) + 8 * c + 4 * hf);
 #pragma unroll
             for (int j = 0; j < 4; j++) { x[4 * c + j] = (float)q4[j]; ss += x[4 * c + j] * x[4 * c + j]; }
         }
@@ -233,7 +237,7 @@ __global__ void __launch_bounds__(512) bwd_dq_kernel(const BwdParams p) {
                 V4 o4;
 #pragma unroll
                 for (int j = 0; j < 4; j++) o4[j] = (E)(f * (dqacc[4 * c + j] - x[4 * c + j] * proj));
-                *reinterpret_cast<V4*>(dqptr + (int64_t)qi * p.dq.sn + 8 * c + 4 * hf) = o4;
+                *reinterpret_cast<V4*>(dqbase + row_off_any(p.dq, p.map, b, h, qi) + 8 * c + 4 * hf) = o4;
             }
         }
         if (!qv || hf != 0) dot = 0.f;

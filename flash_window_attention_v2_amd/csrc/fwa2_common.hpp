@@ -265,7 +265,7 @@ __device__ __forceinline__ auto load_raw8(const T* row, int c0, int n, float pad
 // not push the bias / mask tables (re-read by every unit) out of the L2.
 constexpr int kStreamPolicy = 2;
 
-constexpr int kMapMaxN = 256;    // largest window the kernels address through a window map (the resident-tile ones)
+constexpr int kMapMaxN = 1024;   // largest window addressed through a window map: row * win_w must stay below 65536
 constexpr int kKeyChunk = 256;   // keys staged in LDS at a time by the query-owning kernels
 constexpr int kLdsStride = 40;   // elements per staged row (32 + 8 pad): 80-byte rows
 
@@ -297,6 +297,12 @@ __device__ __forceinline__ int64_t row_off(const T4& t, const WinMap& m, int b, 
     y -= y >= m.gh ? m.gh : 0;
     x -= x >= m.gw ? m.gw : 0;
     return img * t.sb + h * t.sh + (int64_t)(y * m.gw + x) * t.sn;
+}
+
+// The same with the map decided at run time, for the kernels that stream long windows: a few address
+// computations per key chunk, so the branch costs nothing there.
+__device__ __forceinline__ int64_t row_off_any(const T4& t, const WinMap& m, int b, int h, int row) {
+    return m.nw > 0 ? row_off<true>(t, m, b, h, row) : row_off<false>(t, m, b, h, row);
 }
 
 // Row `row` of a tensor whose unit starts at `unit` (a wavefront-uniform pointer): one full-rate 24-bit

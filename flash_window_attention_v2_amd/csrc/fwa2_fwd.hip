@@ -60,10 +60,11 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdParams p) {
     const int h = idx % p.heads;
     const int b = idx / p.heads;
 
-    const E* qptr = reinterpret_cast<const E*>(p.q.ptr) + b * p.q.sb + h * p.q.sh;
-    const E* kptr = reinterpret_cast<const E*>(p.k.ptr) + b * p.k.sb + h * p.k.sh;
-    const E* vptr = reinterpret_cast<const E*>(p.v.ptr) + b * p.v.sb + h * p.v.sh;
-    E* optr = reinterpret_cast<E*>(const_cast<void*>(p.o.ptr)) + b * p.o.sb + h * p.o.sh;
+    // rows are addressed through the window map when there is one (cyclic shift + window partition done here)
+    const E* qbase = reinterpret_cast<const E*>(p.q.ptr);
+    const E* kbase = reinterpret_cast<const E*>(p.k.ptr);
+    const E* vbase = reinterpret_cast<const E*>(p.v.ptr);
+    E* obase = reinterpret_cast<E*>(const_cast<void*>(p.o.ptr));
 
     float scale2;
     if (p.scale_kind == FWA2_SCALE_TENSOR) {
@@ -83,8 +84,9 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdParams p) {
     if (wave_live) {
         V8 a = zero8<V8>(), c = zero8<V8>();
         if (qv) {
-            a = ld8<V8>(qptr + qi * p.q.sn + 8 * hf);
-            c = ld8<V8>(qptr + qi * p.q.sn + 16 + 8 * hf);
+            const E* qrow = qbase + row_off_any(p.q, p.map, b, h, qi);
+            a = ld8<V8>(qrow + 8 * hf);
+            c = ld8<V8>(qrow + 16 + 8 * hf);
         }
         float xa[8], xc[8];
         unpack8(a, xa);
@@ -123,8 +125,8 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdParams p) {
             const int dch = (tid & 3) * 8;
             V8 kk = zero8<V8>(), vv = zero8<V8>();
             if (r < rows) {
-                kk = ld8<V8>(kptr + (int64_t)(c0 + r) * p.k.sn + dch);
-                vv = ld8<V8>(vptr + (int64_t)(c0 + r) * p.v.sn + dch);
+                kk = ld8<V8>(kbase + row_off_any(p.k, p.map, b, h, c0 + r) + dch);
+                vv = ld8<V8>(vbase + row_off_any(p.v, p.map, b, h, c0 + r) + dch);
             }
             float x[8];
             unpack8(kk, x);
@@ -237,7 +239,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdParams p) {
             V4 ov;
 #pragma unroll
             for (int j = 0; j < 4; j++) ov[j] = (E)(oacc[4 * c + j] * inv_l);
-            *reinterpret_cast<V4*>(optr + (int64_t)qi * p.o.sn + 8 * c + 4 * hf) = ov;
+            *reinterpret_cast<V4*>(obase + row_off_any(p.o, p.map, b, h, qi) + 8 * c + 4 * hf) = ov;
         }
         if (hf == 0) {
             const float lse = l_tot > 0.f ? (m_run + fast_log2(l_tot)) * kLn2 : -INFINITY;

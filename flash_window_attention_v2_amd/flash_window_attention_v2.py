@@ -132,7 +132,7 @@ class FlashWindowAttentionV2QKVPacked(torch.autograd.Function):
         return dqkv, dscale, db, None
 
 
-MAPPED_MAX_N = 256      # largest window the library addresses through a window map
+MAPPED_MAX_N = 1024     # largest window the library addresses through a window map
 
 
 class FlashWindowAttentionV2Grid(torch.autograd.Function):

@@ -127,7 +127,7 @@ typedef struct fwa2_problem {
      * nW = (grid_h / win_h) (grid_w / win_w), window = wy (grid_w / win_w) + wx; its row n = r win_w + c is the
      * token at ((wy win_h + r + shift_h) mod grid_h, (wx win_w + c + shift_w) mod grid_w).  n must equal
      * win_h win_w and bw must equal B nW; lse, bias, mask, dbias are indexed as without a map (mask: nW == n_windows).
-     * Supported for n <= 256 and win_w <= 64 (FWA2_ERR_UNSUPPORTED otherwise).
+     * Supported for n <= 1024 and win_w <= 64 (FWA2_ERR_UNSUPPORTED otherwise).
      */
     int32_t grid_h, grid_w;
     int32_t win_h, win_w;

@@ -60,6 +60,9 @@ CASES = [
     (1, (20, 40), (10, 20), (5, 10), 2, True),      # 200 tokens, not a multiple of 16
     (2, (16, 24), (8, 12), (4, 6), 3, True),        # 96 tokens
     (2, (22, 11), (11, 11), (5, 5), 2, True),       # 121 tokens, odd
+    (2, (36, 18), (18, 18), (9, 9), 2, True),       # 324 tokens: the streaming kernels, two key-side super-tiles
+    (1, (24, 48), (24, 24), (12, 12), 3, True),     # 576 tokens
+    (1, (32, 64), (32, 32), (16, 16), 2, False),    # 1024 tokens, the largest mapped window
 ]
 
 
@@ -88,7 +91,7 @@ def test_grid_matches_partitioned_call(case, dtype):
     assert torch.equal(scale_a.grad, scale_b.grad)
 
 
-@pytest.mark.parametrize("case", [CASES[2], CASES[7]], ids=["w4x8", "w16x16"])
+@pytest.mark.parametrize("case", [CASES[2], CASES[7], CASES[13]], ids=["w4x8", "w16x16", "w18x18"])
 def test_grid_against_the_classic_oracle(case):
     """The grid operator held directly against the fp32 classic path applied to rolled and partitioned copies
     made on the CPU (roll, window_partition, attention, window_reverse, roll back, as the reference's block
@@ -138,13 +141,13 @@ def test_grid_with_other_head_dimensions(case, d):
     assert torch.equal(bias_a.grad, bias_b.grad) and torch.equal(scale_a.grad, scale_b.grad)
 
 
-def test_grid_rejects_windows_longer_than_256_tokens():
-    """Windows of more than 256 tokens run on the streaming kernels, which take no map: the library must
-    say so instead of computing on wrong addresses."""
+def test_grid_rejects_windows_longer_than_1024_tokens():
+    """The map's row arithmetic covers windows of up to 1024 tokens: beyond that the library must say so
+    instead of computing on wrong addresses."""
     from flash_window_attention_v2_amd import flash_win_attn_v2_grid_func
-    qkv, scale, bias, mask, _ = _inputs(1, (36, 18), (18, 18), 2, 32, torch.bfloat16, 12, True)
+    qkv, scale, bias, mask, _ = _inputs(1, (36, 72), (36, 36), 2, 32, torch.bfloat16, 12, False)
     with pytest.raises(NotImplementedError, match="window map"):
-        flash_win_attn_v2_grid_func(qkv, (36, 18), (18, 18), (9, 9), scale, bias, mask)
+        flash_win_attn_v2_grid_func(qkv, (36, 72), (36, 36), (18, 18), scale, bias, mask)
 
 
 def test_grid_argument_errors():

@@ -259,16 +259,16 @@ def test_fused_position_bias_gpu(window, dtype):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("window,shift", [(8, 0), (8, 4), (16, 8)])
-def test_block_window_map_matches_partition_gpu(window, shift):
+@pytest.mark.parametrize("window,shift,res", [(8, 0, 32), (8, 4, 32), (16, 8, 32), (24, 12, 48)])
+def test_block_window_map_matches_partition_gpu(window, shift, res):
     """SwinTransformerBlock with the roll / partition / reverse done by the kernels' addressing against the
     same block doing them as the reference does (swin_transformer_v2.py:419-441).  The attention kernels see
     the same values either way; the projections run on differently ordered rows, hence a tolerance of a few ulp."""
     torch.manual_seed(3)
     dev = torch.device("cuda")
-    blk = swin.SwinTransformerBlock(96, (32, 32), 3, window_size=window, shift_size=shift, is_flash=True).to(dev).bfloat16()
-    x = torch.randn(2, 32 * 32, 96, device=dev).bfloat16()
-    g = torch.randn(2, 32 * 32, 96, device=dev).bfloat16()
+    blk = swin.SwinTransformerBlock(96, (res, res), 3, window_size=window, shift_size=shift, is_flash=True).to(dev).bfloat16()
+    x = torch.randn(2, res * res, 96, device=dev).bfloat16()
+    g = torch.randn(2, res * res, 96, device=dev).bfloat16()
 
     assert blk.attn.grid_ready(x)
     xa = x.clone().requires_grad_()
