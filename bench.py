@@ -29,10 +29,10 @@ if ROOT not in sys.path:
 METRIC = "fwd+bwd ms & TFLOPS (% MFMA peak), B64 nW64 H3 d32 N256 bf16, 1 GPU"
 MFMA_BF16_PEAK_TFLOPS = 2500.0     # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0              # MI355X HBM3E
-# HBM bytes per launch of the backward kernel at the benchmark shape, from
+# HBM bytes per launch of the key-side backward kernel at the benchmark shape, from
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a copy kernel of known size
-# (profiles/kernels_C3_fwd_bwd.txt: FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, both launches).
-BWD_KERNEL_TRAFFIC_BYTES = 1.640e9
+# (profiles/kernels_C3_fwd_bwd.txt: FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0).
+BWD_KERNEL_TRAFFIC_BYTES = 1.631e9
 
 
 def log(*a):
