@@ -104,10 +104,35 @@ __device__ __forceinline__ uint32_t lds_address(const void* p) {     // of a wav
 __device__ __forceinline__ void dma16_to_lds(const void* src, uint32_t lds) {      // non-temporal: streamed rows
     asm volatile("s_nop 3\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off nt" ::"v"(src), "s"(lds) : "memory", "m0");
 }
+// The same from a wavefront-uniform base (scalar registers) plus a 32-bit byte offset per lane: no 64-bit
+// address arithmetic on the vector unit.
+__device__ __forceinline__ const void* uniform_pointer(const void* p) {
+    const uint64_t v = (uint64_t)(uintptr_t)p;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return (const void*)(uintptr_t)(((uint64_t)hi << 32) | lo);
+}
+__device__ __forceinline__ void dma16_to_lds(const void* uniform_base, uint32_t byte_offset, uint32_t lds) {
+    asm volatile("s_nop 3\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 nt" ::"v"(byte_offset), "s"(uniform_base), "s"(lds) : "memory", "m0");
+}
+// Byte offset of (row, col) inside a unit whose rows are `sn` elements apart (one 24-bit multiply).
+template <class E>
+__device__ __forceinline__ uint32_t row_byte_offset(int row, int64_t sn, int col) {
+    uint32_t prod;
+    asm("v_mul_u32_u24 %0, %1, %2" : "=v"(prod) : "s"((uint32_t)sn), "v"((uint32_t)row));
+    return (prod + (uint32_t)col) * (uint32_t)sizeof(E);
+}
 __device__ __forceinline__ void dma4_to_lds(const void* src, uint32_t lds) {
     asm volatile("s_nop 3\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(src), "s"(lds) : "memory", "m0");
 }
 #pragma clang diagnostic pop
+
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every global store the
+// wavefront has issued (it fences global memory at workgroup scope); in a loop that ends with output stores
+// that puts a full write round trip on the critical path of every iteration, with all wavefronts parked at
+// the barrier.  The kernels that use this exchange data through LDS alone.
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
 
 // ---- cross-lane helpers (wave64) -------------------------------------------
 // Value held by the lane 32 away, combined with the own value by max / add.
@@ -139,13 +164,18 @@ __device__ __forceinline__ int lane_now() {
     return l;
 }
 
+#ifdef PROBE_NOEXP
+__device__ __forceinline__ float fast_exp2(float x) { return x * 0.001f; }
+#else
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+#endif
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
 
-// 1 / max(||x||, eps) from a sum of squares (torch.nn.functional.normalize).
+// 1 / max(||x||, eps) from a sum of squares (torch.nn.functional.normalize): one v_rsq_f32 (1 ulp) instead of
+// a square root and an IEEE division (about twenty instructions); every use is rounded to 16 bits afterwards.
 __device__ __forceinline__ float inv_norm(float sumsq) {
-    return 1.0f / fmaxf(sqrtf(sumsq), kNormEps);
+    return __builtin_amdgcn_rsqf(fmaxf(sumsq, kNormEps * kNormEps));
 }
 
 // Row r of a 32-row MFMA A operand <-> position inside a 32-key tile such that

@@ -43,8 +43,10 @@ namespace fwa2 {
 // MASKED: this launch handles the units whose window mask is live; the other units (or all, when
 // there is no mask) go through the MASKED = false instantiation.
 // MAPPED: rows are addressed through the window map (cyclic shift + window partition done here).
-template <int DT, bool HAS_BIAS, int MASK_DT, int NT, bool VEC, bool MASKED, bool MAPPED>
-__global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p) {
+// SUB: 16-row query tiles per wavefront.  Two tiles share every K / V operand read from LDS and leave the
+// wavefront 256 registers, half as many wavefronts per workgroup.
+template <int DT, bool HAS_BIAS, int MASK_DT, int NT, bool VEC, bool MASKED, bool MAPPED, int SUB = 1>
+__global__ void __launch_bounds__(64 * NT / SUB) fwd_resident_kernel(const FwdParams p) {
     typedef typename Elem<DT>::E E;
     typedef typename Elem<DT>::V8 V8;
     typedef typename Elem<DT>::V4 V4;
@@ -53,19 +55,21 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
     typedef typename Elem<kScoreDT>::V8 SV8;
     constexpr int ROWS = 16 * NT;
     constexpr int S = kLdsStride;
+    constexpr int WR = 16 * SUB;          // rows per wavefront (queries owned, K / V rows staged)
+    constexpr int IDS = WR + 16;          // bytes of the region landing area per wavefront: ids, then the value
 
     __shared__ __attribute__((aligned(16))) SE lds_K[2][ROWS * S];
     __shared__ __attribute__((aligned(16))) E lds_V[2][ROWS * S];
     __shared__ __attribute__((aligned(16))) E lds_rawK[ROWS * 32];   // landing area: unpadded 64-byte rows
     __shared__ __attribute__((aligned(16))) E lds_rawV[ROWS * 32];
-    __shared__ __attribute__((aligned(16))) E lds_rawQ[ROWS * 32];   // the wavefront's own 16 query rows
+    __shared__ __attribute__((aligned(16))) E lds_rawQ[ROWS * 32];   // the wavefront's own query rows
     // REGIONS: the plain launch also takes the windows whose mask has region form (RegionRecord): their mask term
     // comes out of one more MFMA per score tile, query-side operand in registers, key-side operand in lds_kop
     constexpr bool REGIONS = MASK_DT >= 0 && !MASKED;
     static_assert(kLdsStride >= 40 && kScoreDT == FWA2_F16,
                   "the key-side entries of the region product live in the 8 spare fp16 columns of the staged K rows");
-    // landing area of the region record: per wavefront the ids of its 16 rows, then the record's value
-    __shared__ __attribute__((aligned(16))) uint8_t lds_rawid[REGIONS ? ROWS * 2 : 32];
+    // landing area of the region record: per wavefront the ids of its rows, then the record's value
+    __shared__ __attribute__((aligned(16))) uint8_t lds_rawid[REGIONS ? (NT / SUB) * IDS : 32];
     __shared__ uint8_t lds_live[kLiveCache];       // copy of the per-window mask flags
     __shared__ uint16_t lds_list[kLiveCache];      // windows of this launch's class, ascending
     __shared__ int lds_count;
@@ -129,60 +133,63 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
         st8<V8>(lds_rawQ + i * 8, zero8<V8>());
     }
 
-    const int qi = wave * 16 + l16;
-    const bool qv = qi < N;
-    const int qc = min(qi, N - 1);
+    bool qv[SUB];
+#pragma unroll
+    for (int u = 0; u < SUB; u++) qv[u] = wave * WR + 16 * u + l16 < N;
 
     // ---- resident tile, log2 domain.  Keys are taken 32 at a time; of such a group this lane holds
     // keys 8g .. 8g+7: acc0[2kp][i] <-> key 32kp + 8g + i, acc0[2kp+1][i] <-> key 32kp + 8g + 4 + i
     // (so bias and mask rows are read 8 consecutive entries at a time).  The tile holds
     // (bias + mask) * log2e - m_fixed, m_fixed = s log2e + max_j (bias2 + mask2)[j] being an upper bound
     // of every logit of the row; the key that attains the maximum scores at least m_fixed - 2 s log2e. ----
-    f32x4 acc0[NT];
-    float m_fixed = 0.f;
-    float bias_range = 0.f;      // largest minus smallest bias (log2 domain) of this lane's row
+    f32x4 acc0[SUB][NT];
+    float m_fixed[SUB];
+    float bias_range = 0.f;      // largest minus smallest bias (log2 domain) over this lane's rows
     auto build_tile = [&](int w) __attribute__((always_inline)) {
         // lane-derived offsets are re-materialised per call: hoisted out of the unit loop, the row
         // addresses of every key group would stay alive (and spilled) across all units
         int ln = lane;
         if (MASKED) asm volatile("" : "+v"(ln));
         const int g = ln >> 4;
-        const int qrow = min(wave * 16 + (ln & 15), N - 1);
-        const E* brow = nullptr;
-        const ME* mrow = nullptr;
-        if (HAS_BIAS) brow = reinterpret_cast<const E*>(p.bias) + h * p.bias_sh + (int64_t)qrow * p.bias_sn;
-        if (MASKED) mrow = reinterpret_cast<const ME*>(p.mask) + w * p.mask_sw + (int64_t)qrow * p.mask_sn;
-        float mb = -INFINITY, mn = INFINITY;
 #pragma unroll
-        for (int kp = 0; kp < NT / 2; kp++) {
-            float v[8];
+        for (int u = 0; u < SUB; u++) {
+            const int qrow = min(wave * WR + 16 * u + (ln & 15), N - 1);
+            const E* brow = nullptr;
+            const ME* mrow = nullptr;
+            if (HAS_BIAS) brow = reinterpret_cast<const E*>(p.bias) + h * p.bias_sh + (int64_t)qrow * p.bias_sn;
+            if (MASKED) mrow = reinterpret_cast<const ME*>(p.mask) + w * p.mask_sw + (int64_t)qrow * p.mask_sn;
+            float mb = -INFINITY, mn = INFINITY;
 #pragma unroll
-            for (int j = 0; j < 8; j++) v[j] = (32 * kp + 8 * g + j < N) ? 0.f : -INFINITY;
-            if (HAS_BIAS) {
-                const auto raw = load_raw8<VEC, E>(brow, 32 * kp + 8 * g, N, 0.f);
+            for (int kp = 0; kp < NT / 2; kp++) {
+                float v[8];
 #pragma unroll
-                for (int j = 0; j < 8; j++) v[j] += (float)raw[j] * kLog2e;
+                for (int j = 0; j < 8; j++) v[j] = (32 * kp + 8 * g + j < N) ? 0.f : -INFINITY;
+                if (HAS_BIAS) {
+                    const auto raw = load_raw8<VEC, E>(brow, 32 * kp + 8 * g, N, 0.f);
+#pragma unroll
+                    for (int j = 0; j < 8; j++) v[j] += (float)raw[j] * kLog2e;
+                }
+                if (MASKED) {
+                    const auto raw = load_raw8<VEC, ME>(mrow, 32 * kp + 8 * g, N, 0.f);
+#pragma unroll
+                    for (int j = 0; j < 8; j++) v[j] = fmaf((float)raw[j], kLog2e, v[j]);
+                }
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    acc0[u][2 * kp + (j >> 2)][j & 3] = v[j];
+                    mb = fmaxf(mb, v[j]);
+                    if (REGIONS && v[j] > -INFINITY) mn = fminf(mn, v[j]);
+                }
             }
-            if (MASKED) {
-                const auto raw = load_raw8<VEC, ME>(mrow, 32 * kp + 8 * g, N, 0.f);
+            mb = col_max(mb);
+            if (REGIONS) bias_range = fmaxf(bias_range, mb - (-col_max(-mn)));
+            if (!(mb > -INFINITY)) mb = 0.f;        // every key of the row removed: nothing to bound
+            m_fixed[u] = mb + scale2;
 #pragma unroll
-                for (int j = 0; j < 8; j++) v[j] = fmaf((float)raw[j], kLog2e, v[j]);
-            }
+            for (int kt = 0; kt < NT; kt++)
 #pragma unroll
-            for (int j = 0; j < 8; j++) {
-                acc0[2 * kp + (j >> 2)][j & 3] = v[j];
-                mb = fmaxf(mb, v[j]);
-                if (REGIONS && v[j] > -INFINITY) mn = fminf(mn, v[j]);
-            }
+                for (int i = 0; i < 4; i++) acc0[u][kt][i] -= m_fixed[u];
         }
-        mb = col_max(mb);
-        if (REGIONS) bias_range = mb - (-col_max(-mn));
-        if (!(mb > -INFINITY)) mb = 0.f;        // every key of the row removed: nothing to bound
-        m_fixed = mb + scale2;
-#pragma unroll
-        for (int kt = 0; kt < NT; kt++)
-#pragma unroll
-            for (int i = 0; i < 4; i++) acc0[kt][i] -= m_fixed;
     };
     // the maximum-free softmax is used when the row bound cannot be further than this from the
     // largest logit (the same for every row of the head)
@@ -207,6 +214,9 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
             wi_step = p.groups;
         }
     }
+    // the plain walk t -> t + groups without a division per unit: (img, wi) += (groups / cnt, groups % cnt)
+    const int step_img = cnt > 0 ? p.groups / cnt : 0;
+    const int step_wi = cnt > 0 ? p.groups - step_img * cnt : 0;
     struct Cursor { int wi, img; };
     auto valid = [&](const Cursor& c) -> bool { return MASKED ? c.wi < cnt : c.img < n_img; };
     auto first = [&]() -> Cursor {
@@ -220,9 +230,9 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
             c.img += img_step;
             if (c.img >= n_img) { c.img = img0; c.wi += wi_step; }
         } else {
-            const int t = c.img * cnt + c.wi + p.groups;
-            c.img = t / cnt;
-            c.wi = t - c.img * cnt;
+            c.img += step_img;
+            c.wi += step_wi;
+            if (c.wi >= cnt) { c.wi -= cnt; c.img += 1; }
         }
         return c;
     };
@@ -235,54 +245,71 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
         return reinterpret_cast<const RegionRecord*>(p.regions) + w;
     };
 
-    // ---- per-unit fetch: every wavefront brings in the 16 K and V rows it will stage (lane i lands
-    // at 16 i bytes from the wavefront's base) and its own 16 query rows ----
-    const int frow = wave * 16 + (lane >> 2);      // K / V row of this lane
-    const int fc8 = (lane & 3) * 8;
+    // ---- per-unit fetch: every wavefront brings in the WR rows of K, V (which it will stage) and of Q (its own
+    // queries) with that index, 16 rows per instruction (lane i lands at 16 i bytes from the base) ----
     auto fetch = [&](int b, const RegionRecord* rec) __attribute__((always_inline)) {
         // lane-derived offsets are re-materialised here: hoisted out of the unit loop they would be
         // spilled, and the reload would sit in front of every fetch
         int ln = lane;
         asm volatile("" : "+v"(ln));
-        const int frow = wave * 16 + (ln >> 2);
         const int fc8 = (ln & 3) * 8;
-        if (frow < N) {
-            dma16_to_lds(row_ptr<MAPPED, E>(p.k, p.map, b, h, frow, fc8), lds_address(lds_rawK + wave * 16 * 32));
-            dma16_to_lds(row_ptr<MAPPED, E>(p.v, p.map, b, h, frow, fc8), lds_address(lds_rawV + wave * 16 * 32));
-            dma16_to_lds(row_ptr<MAPPED, E>(p.q, p.map, b, h, frow, fc8), lds_address(lds_rawQ + wave * 16 * 32));
+        // unit starts in scalar registers, rows as 32-bit byte offsets from them
+        const void* kunit = uniform_pointer(unit_ptr<MAPPED, E>(p.k, p.map, b, h));
+        const void* vunit = uniform_pointer(unit_ptr<MAPPED, E>(p.v, p.map, b, h));
+        const void* qunit = uniform_pointer(unit_ptr<MAPPED, E>(p.q, p.map, b, h));
+#pragma unroll
+        for (int u = 0; u < SUB; u++) {
+            const int row0 = wave * WR + 16 * u;
+            const int frow = row0 + (ln >> 2);
+            if (frow < N) {
+                const int pos = unit_row<MAPPED>(p.map, b, frow);
+                dma16_to_lds(kunit, row_byte_offset<E>(pos, p.k.sn, fc8), lds_address(lds_rawK + row0 * 32));
+                dma16_to_lds(vunit, row_byte_offset<E>(pos, p.v.sn, fc8), lds_address(lds_rawV + row0 * 32));
+                dma16_to_lds(qunit, row_byte_offset<E>(pos, p.q.sn, fc8), lds_address(lds_rawQ + row0 * 32));
+            }
         }
-        if (REGIONS && rec != nullptr && ln < 5) {    // the ids of this wavefront's 16 rows (lanes 0 .. 3), the value (lane 4)
-            const void* src = ln < 4 ? (const void*)(rec->id + wave * 16 + 4 * ln) : (const void*)&rec->value;
-            dma4_to_lds(src, lds_address(lds_rawid + wave * 32));
+        if (REGIONS && rec != nullptr && ln < 4 * SUB + 1) {    // the ids of this wavefront's rows, then the value
+            const void* src = ln < 4 * SUB ? (const void*)(rec->id + wave * WR + 4 * ln) : (const void*)&rec->value;
+            dma4_to_lds(src, lds_address(lds_rawid + wave * IDS));
         }
     };
     // landing area -> tiles: K normalised and rounded to fp16, V as is (rows >= n stay zero)
-    f16x4 qop = {0, 0, 0, 0};   // query-side operand of the region product for the unit staged last
+    f16x4 qop[SUB];             // query-side operands of the region product for the unit staged last
+#pragma unroll
+    for (int u = 0; u < SUB; u++) qop[u] = f16x4{0, 0, 0, 0};
     auto stage = [&](int buf, const RegionRecord* rec) __attribute__((always_inline)) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");    // this wavefront's rows have landed
+        int ln = lane;
+        asm volatile("" : "+v"(ln));
+        const int fc8 = (ln & 3) * 8;
         if (REGIONS && rec != nullptr) {
-            int ln = lane;
-            asm volatile("" : "+v"(ln));
-            const float value = *reinterpret_cast<const float*>(lds_rawid + wave * 32 + 16);
-            qop = region_query_operand(value * kLog2e, lds_rawid[wave * 32 + (ln & 15)], ln >> 4);
-            if ((ln & 3) == 0)
-                st8<f16x8>(reinterpret_cast<_Float16*>(&lds_K[buf][(wave * 16 + (ln >> 2)) * S + 32]),
-                           region_key_entry(lds_rawid[wave * 32 + (ln >> 2)]));
+            const float value = *reinterpret_cast<const float*>(lds_rawid + wave * IDS + WR);
+#pragma unroll
+            for (int u = 0; u < SUB; u++) {
+                qop[u] = region_query_operand(value * kLog2e, lds_rawid[wave * IDS + 16 * u + (ln & 15)], ln >> 4);
+                if ((ln & 3) == 0)
+                    st8<f16x8>(reinterpret_cast<_Float16*>(&lds_K[buf][(wave * WR + 16 * u + (ln >> 2)) * S + 32]),
+                               region_key_entry(lds_rawid[wave * IDS + 16 * u + (ln >> 2)]));
+            }
         }
-        const V8 kk = ld8<V8>(lds_rawK + frow * 32 + fc8);
-        const V8 vv = ld8<V8>(lds_rawV + frow * 32 + fc8);
-        float x[8];
-        unpack8(kk, x);
-        float ss = 0.f;
 #pragma unroll
-        for (int j = 0; j < 8; j++) ss += x[j] * x[j];
-        ss = quad_add(ss);
-        const float inv = inv_norm(ss);
-        SV8 kn;
+        for (int u = 0; u < SUB; u++) {
+            const int frow = wave * WR + 16 * u + (ln >> 2);
+            const V8 kk = ld8<V8>(lds_rawK + frow * 32 + fc8);
+            const V8 vv = ld8<V8>(lds_rawV + frow * 32 + fc8);
+            float x[8];
+            unpack8(kk, x);
+            float ss = 0.f;
 #pragma unroll
-        for (int j = 0; j < 8; j++) kn[j] = (SE)(x[j] * inv);
-        st8<SV8>(&lds_K[buf][frow * S + fc8], kn);
-        st8<V8>(&lds_V[buf][frow * S + fc8], vv);
+            for (int j = 0; j < 8; j++) ss += x[j] * x[j];
+            ss = quad_add(ss);
+            const float inv = inv_norm(ss);
+            SV8 kn;
+#pragma unroll
+            for (int j = 0; j < 8; j++) kn[j] = (SE)(x[j] * inv);
+            st8<SV8>(&lds_K[buf][frow * S + fc8], kn);
+            st8<V8>(&lds_V[buf][frow * S + fc8], vv);
+        }
     };
 
     __syncthreads();                       // zero fill done
@@ -308,11 +335,12 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
             build_tile(window_at(c.wi));
             tile_wi = c.wi;
         }
-        // ---- Q operand: normalise, fold s log2e, round to fp16 ----
-        SV8 bq;
-        {
+        // ---- Q operands: normalise, fold s log2e, round to fp16 ----
+        SV8 bq[SUB];
+#pragma unroll
+        for (int u = 0; u < SUB; u++) {
             // the rows landed before the previous unit's barrier (the first unit's before the one above)
-            const V8 qq = ld8<V8>(lds_rawQ + (wave * 16 + l16) * 32 + 8 * g);
+            const V8 qq = ld8<V8>(lds_rawQ + (wave * WR + 16 * u + l16) * 32 + 8 * g);
             float x[8];
             unpack8(qq, x);
             float ss = 0.f;
@@ -321,7 +349,7 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
             ss = col_add(ss);
             const float sc = scale2 * inv_norm(ss);
 #pragma unroll
-            for (int j = 0; j < 8; j++) bq[j] = (SE)(x[j] * sc);
+            for (int j = 0; j < 8; j++) bq[u][j] = (SE)(x[j] * sc);
         }
         const RegionRecord* rec = record_of(c);
         const RegionRecord* rec_next = more ? record_of(cn) : nullptr;
@@ -330,21 +358,28 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
 
         const SE* Kb = &lds_K[cur][0];
         const E* Vb = &lds_V[cur][0];
-        f32x4 oacc[2];
+        f32x4 oacc[SUB][2];
+        f32x4 lacc[SUB];
+        float m_run[SUB];      // exact-maximum path: row maximum relative to m_fixed
 #pragma unroll
-        for (int dt = 0; dt < 2; dt++)
+        for (int u = 0; u < SUB; u++) {
+            m_run[u] = 0.f;
 #pragma unroll
-            for (int i = 0; i < 4; i++) oacc[dt][i] = 0.f;
-        float m_run = 0.f;     // exact-maximum path: row maximum relative to m_fixed
+            for (int i = 0; i < 4; i++) { oacc[u][0][i] = 0.f; oacc[u][1][i] = 0.f; lacc[u][i] = 0.f; }
+        }
 
         // scores of keys 32 kp .. 32 kp + 31: MFMA tile A holds keys 8r/4 + r%4 in its rows r, tile B
-        // the keys 4 further on, so that this lane's 8 values are keys 8g .. 8g+7 of the group
-        auto scores = [&](int kp, f32x4& s0, f32x4& s1, bool with_regions) __attribute__((always_inline)) {
+        // the keys 4 further on, so that this lane's 8 values are keys 8g .. 8g+7 of the group; the two K
+        // operands serve every query tile of the wavefront
+        auto scores = [&](int kp, f32x4 (&s0)[SUB], f32x4 (&s1)[SUB], bool with_regions) __attribute__((always_inline)) {
             const int krow = 32 * kp + 8 * (l16 >> 2) + (l16 & 3);
             const SV8 a0 = ld8<SV8>(Kb + krow * S + 8 * g);
             const SV8 a1 = ld8<SV8>(Kb + (krow + 4) * S + 8 * g);
-            s0 = Elem<kScoreDT>::mfma16(a0, bq, acc0[2 * kp]);
-            s1 = Elem<kScoreDT>::mfma16(a1, bq, acc0[2 * kp + 1]);
+#pragma unroll
+            for (int u = 0; u < SUB; u++) {
+                s0[u] = Elem<kScoreDT>::mfma16(a0, bq[u], acc0[u][2 * kp]);
+                s1[u] = Elem<kScoreDT>::mfma16(a1, bq[u], acc0[u][2 * kp + 1]);
+            }
             if (REGIONS && with_regions) {
                 // the lane's offset is derived again here: hoisted out of the unit loop, the eight addresses
                 // (one per key group) would be spilled
@@ -358,30 +393,34 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
                 asm volatile("ds_read_b64 %0, %2\n\tds_read_b64 %1, %2 offset:%3\n\ts_waitcnt lgkmcnt(0)"
                              : "=&v"(k0), "=&v"(k1)
                              : "v"((uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)ko), "n"(4 * S * 2));
-                s0 = region_mfma(k0, qop, s0);
-                s1 = region_mfma(k1, qop, s1);
+#pragma unroll
+                for (int u = 0; u < SUB; u++) {
+                    s0[u] = region_mfma(k0, qop[u], s0[u]);
+                    s1[u] = region_mfma(k1, qop[u], s1[u]);
+                }
             }
         };
-        // FAST: the row sum comes out of a third MFMA against a tile of ones, i.e. it sums the
-        // ROUNDED P~ values that also enter the product with V: o is then an exact convex
-        // combination of V rows, and the sum costs no VALU work.
-        f32x4 lacc;
-#pragma unroll
-        for (int i = 0; i < 4; i++) lacc[i] = 0.f;
+        // The row sum comes out of a third MFMA against a tile of ones, i.e. it sums the ROUNDED P~ values
+        // that also enter the product with V: o is then an exact convex combination of V rows, and the sum
+        // costs no VALU work.  The transposed V operands serve every query tile of the wavefront.
         V8 ones;
 #pragma unroll
         for (int j = 0; j < 8; j++) ones[j] = (E)1.0f;
-        auto pv = [&](int kp, const f32x4& s0, const f32x4& s1, bool sum_by_mfma) __attribute__((always_inline)) {
-            V8 bp;
+        auto pv = [&](int kp, const f32x4 (&s0)[SUB], const f32x4 (&s1)[SUB]) __attribute__((always_inline)) {
+            V8 bp[SUB];
 #pragma unroll
-            for (int i = 0; i < 4; i++) { bp[i] = (E)s0[i]; bp[4 + i] = (E)s1[i]; }
-            if (sum_by_mfma) lacc = Elem<DT>::mfma16(ones, bp, lacc);
+            for (int u = 0; u < SUB; u++) {
+#pragma unroll
+                for (int i = 0; i < 4; i++) { bp[u][i] = (E)s0[u][i]; bp[u][4 + i] = (E)s1[u][i]; }
+                lacc[u] = Elem<DT>::mfma16(ones, bp[u], lacc[u]);
+            }
 #pragma unroll
             for (int dt = 0; dt < 2; dt++) {
                 // A row m <-> d = 8 (m / 4) + 4 dt + m % 4: this lane's accumulators hold d = 8g + 4dt + i
                 const E* vlo = Vb + (32 * kp + 8 * g + (l16 >> 2)) * S + 8 * (l16 & 3) + 4 * dt;
                 const V8 av = lds_tr8<DT>(vlo, vlo + 4 * S);
-                oacc[dt] = Elem<DT>::mfma16(av, bp, oacc[dt]);
+#pragma unroll
+                for (int u = 0; u < SUB; u++) oacc[u][dt] = Elem<DT>::mfma16(av, bp[u], oacc[u][dt]);
             }
         };
 
@@ -392,43 +431,56 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
 #pragma unroll
                 for (int kp = 0; kp < NT / 2; kp++) {
                     if (32 * kp < N) {
-                        f32x4 s0, s1;
+                        f32x4 s0[SUB], s1[SUB];
                         scores(kp, s0, s1, with_regions);
 #pragma unroll
-                        for (int i = 0; i < 4; i++) {
-                            s0[i] = fast_exp2(s0[i]);
-                            s1[i] = fast_exp2(s1[i]);
-                        }
-                        pv(kp, s0, s1, true);
+                        for (int u = 0; u < SUB; u++)
+#pragma unroll
+                            for (int i = 0; i < 4; i++) {
+                                s0[u][i] = fast_exp2(s0[u][i]);
+                                s1[u][i] = fast_exp2(s1[u][i]);
+                            }
+                        pv(kp, s0, s1);
                     }
                 }
             } else {
                 // fp16 (P would underflow against a mere bound) or a very large scale: the exact row maximum
                 // first, from a pass of score products alone; the matrix pipe has the room, and the second pass
                 // then needs no running maximum, no rescaling of o and no VALU row sum
-                float bm = -INFINITY;
+                float bm[SUB];
+#pragma unroll
+                for (int u = 0; u < SUB; u++) bm[u] = -INFINITY;
 #pragma unroll
                 for (int kp = 0; kp < NT / 2; kp++) {
                     if (32 * kp < N) {
-                        f32x4 s0, s1;
+                        f32x4 s0[SUB], s1[SUB];
                         scores(kp, s0, s1, with_regions);
-                        bm = fmaxf(bm, fmaxf(fmaxf(s0[0], s0[1]), fmaxf(s0[2], s0[3])));
-                        bm = fmaxf(bm, fmaxf(fmaxf(s1[0], s1[1]), fmaxf(s1[2], s1[3])));
+#pragma unroll
+                        for (int u = 0; u < SUB; u++) {
+                            bm[u] = fmaxf(bm[u], fmaxf(fmaxf(s0[u][0], s0[u][1]), fmaxf(s0[u][2], s0[u][3])));
+                            bm[u] = fmaxf(bm[u], fmaxf(fmaxf(s1[u][0], s1[u][1]), fmaxf(s1[u][2], s1[u][3])));
+                        }
                     }
                 }
-                m_run = col_max(bm);
-                const float m_use = (m_run == -INFINITY) ? 0.f : m_run;
+                float m_use[SUB];
+#pragma unroll
+                for (int u = 0; u < SUB; u++) {
+                    m_run[u] = col_max(bm[u]);
+                    m_use[u] = (m_run[u] == -INFINITY) ? 0.f : m_run[u];
+                }
 #pragma unroll
                 for (int kp = 0; kp < NT / 2; kp++) {
                     if (32 * kp < N) {
-                        f32x4 s0, s1;
+                        f32x4 s0[SUB], s1[SUB];
                         scores(kp, s0, s1, with_regions);
 #pragma unroll
-                        for (int i = 0; i < 4; i++) {
-                            s0[i] = fast_exp2(s0[i] - m_use);
-                            s1[i] = fast_exp2(s1[i] - m_use);
-                        }
-                        pv(kp, s0, s1, true);
+                        for (int u = 0; u < SUB; u++)
+#pragma unroll
+                            for (int i = 0; i < 4; i++) {
+                                s0[u][i] = fast_exp2(s0[u][i] - m_use[u]);
+                                s1[u][i] = fast_exp2(s1[u][i] - m_use[u]);
+                            }
+                        pv(kp, s0, s1);
                     }
                 }
             }
@@ -438,24 +490,27 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
 
         if (more) stage(cur ^ 1, rec_next);     // before the stores below, so the wait covers only the fetch
         // ---- normalise, write o (input dtype) and lse (natural log, fp32) ----
-        const float l_tot = lacc[0];
-        const float inv_l = l_tot > 0.f ? 1.0f / l_tot : 0.f;
         int ln2 = lane;
         asm volatile("" : "+v"(ln2));
-        const int oq = wave * 16 + (ln2 & 15);
-        if (qv) {
-            E* orow = const_cast<E*>(row_ptr<MAPPED, E>(p.o, p.map, b, h, oq));
-            V8 ov;
 #pragma unroll
-            for (int j = 0; j < 8; j++) ov[j] = (E)(oacc[j >> 2][j & 3] * inv_l);
-            st8_stream<V8>(orow + 8 * g, ov);
-            if (g == 0) {
-                const float lse = l_tot > 0.f ? (m_fixed + m_run + fast_log2(l_tot)) * kLn2 : -INFINITY;
-                p.lse[b * p.lse_sb + h * p.lse_sh + oq] = lse;
+        for (int u = 0; u < SUB; u++) {
+            const float l_tot = lacc[u][0];
+            const float inv_l = l_tot > 0.f ? fast_rcp(l_tot) : 0.f;
+            const int oq = wave * WR + 16 * u + (ln2 & 15);
+            if (qv[u]) {
+                E* orow = const_cast<E*>(row_ptr<MAPPED, E>(p.o, p.map, b, h, oq));
+                V8 ov;
+#pragma unroll
+                for (int j = 0; j < 8; j++) ov[j] = (E)(oacc[u][j >> 2][j & 3] * inv_l);
+                st8_stream<V8>(orow + 8 * (ln2 >> 4), ov);
+                if ((ln2 >> 4) == 0) {
+                    const float lse = l_tot > 0.f ? (m_fixed[u] + m_run[u] + fast_log2(l_tot)) * kLn2 : -INFINITY;
+                    p.lse[b * p.lse_sb + h * p.lse_sh + oq] = lse;
+                }
             }
         }
 
-        __syncthreads();       // next unit staged; everybody is done with the current buffers
+        lds_barrier();         // next unit staged; everybody is done with the current buffers (the stores stay in flight)
         cur ^= 1;
         c = cn;
     }
@@ -466,6 +521,10 @@ __global__ void __launch_bounds__(64 * NT) fwd_resident_kernel(const FwdParams p
 int forward_resident_supported(int n) { return n >= 1 && n <= 256; }
 #endif
 
+#ifndef FWA2_FWD_SUB
+#define FWA2_FWD_SUB 1
+#endif
+constexpr int kFwdSub = FWA2_FWD_SUB;    // 16-row query tiles per wavefront of the 256-token forward (unmasked launch)
 constexpr int kRegionMaxImages = 32;     // images per window up to which region records are used (see launch_map)
 
 template <class K>
@@ -475,13 +534,17 @@ static int resident_fit(K kern, int threads) {
     return n;
 }
 
-template <int DT, bool HAS_BIAS, int MASK_DT, int NT, bool VEC, bool MAPPED>
+// SUBP: 16-row query tiles per wavefront in the launch over the unmasked units (the masked launch keeps one:
+// its tile rebuilds want the registers).
+template <int DT, bool HAS_BIAS, int MASK_DT, int NT, bool VEC, bool MAPPED, int SUBP>
 static hipError_t launch_map(FwdParams p, hipStream_t st) {
-    const int waves = (p.n + 15) / 16;
-    // the runtime's figure is for full 64 NT-thread groups; smaller groups only fit better
-    static const int fit_plain = resident_fit(fwd_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, false, MAPPED>, 64 * NT);
+    const int waves_plain = (p.n + 16 * SUBP - 1) / (16 * SUBP);
+    const int waves_masked = (p.n + 15) / 16;
+    // the runtime's figure is for full groups; smaller groups only fit better
+    static const int fit_plain =
+        resident_fit(fwd_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, false, MAPPED, SUBP>, 64 * NT / SUBP);
     static const int fit_masked =
-        MASK_DT >= 0 ? resident_fit(fwd_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, true, MAPPED>, 64 * NT) : 1;
+        MASK_DT >= 0 ? resident_fit(fwd_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, true, MAPPED, 1>, 64 * NT) : 1;
     auto groups_for = [&](int fit) {
         int groups = (p.cus * fit) / p.heads;
         if (groups < 1) groups = 1;
@@ -496,22 +559,23 @@ static hipError_t launch_map(FwdParams p, hipStream_t st) {
     // units with an all-zero mask (or every unit when there is no mask) ...
     if (MASK_DT < 0 || p.mask_live != nullptr) {
         p.groups = groups_for(fit_plain);
-        hipLaunchKernelGGL((fwd_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, false, MAPPED>), dim3(p.heads * p.groups),
-                           dim3(64 * waves), 0, st, p);
+        hipLaunchKernelGGL((fwd_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, false, MAPPED, SUBP>), dim3(p.heads * p.groups),
+                           dim3(64 * waves_plain), 0, st, p);
     }
     // ... and the units whose mask is live
     if (MASK_DT >= 0) {
         p.groups = groups_for(fit_masked);
-        hipLaunchKernelGGL((fwd_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, true, MAPPED>), dim3(p.heads * p.groups),
-                           dim3(64 * waves), 0, st, p);
+        hipLaunchKernelGGL((fwd_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, true, MAPPED, 1>), dim3(p.heads * p.groups),
+                           dim3(64 * waves_masked), 0, st, p);
     }
     return hipGetLastError();
 }
 
 template <int DT, bool HAS_BIAS, int MASK_DT, int NT, bool VEC>
 static hipError_t launch_nt(const FwdParams& p, hipStream_t st) {
-    if (p.map.nw > 0) return launch_map<DT, HAS_BIAS, MASK_DT, NT, VEC, true>(p, st);
-    return launch_map<DT, HAS_BIAS, MASK_DT, NT, VEC, false>(p, st);
+    constexpr int SUBP = NT == 16 ? kFwdSub : 1;       // the 256-token form; smaller tiles keep 16 rows per wavefront
+    if (p.map.nw > 0) return launch_map<DT, HAS_BIAS, MASK_DT, NT, VEC, true, SUBP>(p, st);
+    return launch_map<DT, HAS_BIAS, MASK_DT, NT, VEC, false, SUBP>(p, st);
 }
 
 template <int DT, bool HAS_BIAS, int MASK_DT>
