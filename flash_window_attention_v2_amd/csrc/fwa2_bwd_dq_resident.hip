@@ -194,6 +194,9 @@ __global__ void __launch_bounds__(64 * NT / SUB) bwd_dq_resident_kernel(const Bw
             wi_step = groups;
         }
     }
+    // the plain walk t -> t + groups without a division per unit: (img, wi) += (groups / cnt, groups % cnt)
+    const int step_img = cnt > 0 ? groups / cnt : 0;
+    const int step_wi = cnt > 0 ? groups - step_img * cnt : 0;
     struct Cursor { int wi, img; };
     auto valid = [&](const Cursor& c) -> bool { return MASKED ? c.wi < cnt : c.img < n_img; };
     auto first = [&]() -> Cursor {
@@ -207,9 +210,9 @@ __global__ void __launch_bounds__(64 * NT / SUB) bwd_dq_resident_kernel(const Bw
             c.img += img_step;
             if (c.img >= n_img) { c.img = img0; c.wi += wi_step; }
         } else {
-            const int t = c.img * cnt + c.wi + groups;
-            c.img = t / cnt;
-            c.wi = t - c.img * cnt;
+            c.img += step_img;
+            c.wi += step_wi;
+            if (c.wi >= cnt) { c.wi -= cnt; c.img += 1; }
         }
         return c;
     };
@@ -219,8 +222,8 @@ __global__ void __launch_bounds__(64 * NT / SUB) bwd_dq_resident_kernel(const Bw
     // queries) by DMA, 16 rows per instruction; lse and delta of its queries in registers ----
     // issued by hand (see dma16_to_lds): the compiler would otherwise wait for the whole fetch in front of the
     // first transposing LDS read of every unit, which it cannot tell from the landing areas
-    auto dma16 = [&](const E* src, E* lds_wave_base) __attribute__((always_inline)) {
-        dma16_to_lds(src, lds_address(lds_wave_base));
+    auto dma16 = [&](const void* unit, uint32_t byte_offset, uint32_t lds_wave_base) __attribute__((always_inline)) {
+        dma16_to_lds(unit, byte_offset, lds_wave_base);
     };
     auto fetch = [&](int b) __attribute__((always_inline)) {
         // lane-derived offsets are re-materialised here: hoisted out of the unit loop they would occupy
@@ -228,16 +231,24 @@ __global__ void __launch_bounds__(64 * NT / SUB) bwd_dq_resident_kernel(const Bw
         int ln = lane;
         asm volatile("" : "+v"(ln));
         const int fc8 = (ln & 3) * 8;
+        // unit starts in scalar registers, rows as 32-bit byte offsets from them
+        const void* kunit = uniform_pointer(unit_ptr<MAPPED, E>(p.k, p.map, b, h));
+        const void* vunit = uniform_pointer(unit_ptr<MAPPED, E>(p.v, p.map, b, h));
+        const void* qunit = uniform_pointer(unit_ptr<MAPPED, E>(p.q, p.map, b, h));
+        const void* dounit = uniform_pointer(unit_ptr<MAPPED, E>(p.d_o, p.map, b, h));
 #pragma unroll
         for (int u = 0; u < SUB; u++) {
             const int row0 = wave * WR + 16 * u;
             const int frow = row0 + (ln >> 2);
             if (frow < N) {
-                dma16(row_ptr<MAPPED, E>(p.k, p.map, b, h, frow, fc8), lds_rawK + row0 * 32);
-                dma16(row_ptr<MAPPED, E>(p.v, p.map, b, h, frow, fc8), lds_rawV + row0 * 32);
-                dma16(row_ptr<MAPPED, E>(p.q, p.map, b, h, frow, fc8), lds_rawQ + row0 * 32);
-                dma16(row_ptr<MAPPED, E>(p.d_o, p.map, b, h, frow, fc8),
-                      lds_rawDO + row0 * 32);
+                const int pos = unit_row<MAPPED>(p.map, b, frow);
+                // landing addresses as integers from the arrays' starts (the address of a __shared__ array is a
+                // compile-time constant; no pointer leaves the LDS address space on the way)
+                const uint32_t land = (uint32_t)(row0 * 32 * sizeof(E));
+                dma16(kunit, row_byte_offset<E>(pos, p.k.sn, fc8), lds_address(lds_rawK) + land);
+                dma16(vunit, row_byte_offset<E>(pos, p.v.sn, fc8), lds_address(lds_rawV) + land);
+                dma16(qunit, row_byte_offset<E>(pos, p.q.sn, fc8), lds_address(lds_rawQ) + land);
+                dma16(dounit, row_byte_offset<E>(pos, p.d_o.sn, fc8), lds_address(lds_rawDO) + land);
             }
         }
         // lse and delta of the wavefront's rows, one row per lane
@@ -309,7 +320,7 @@ __global__ void __launch_bounds__(64 * NT / SUB) bwd_dq_resident_kernel(const Bw
 #pragma unroll
             for (int j = 0; j < 8; j++) ss += x[j] * x[j];
             ss = col_add(ss);
-            inv[u] = 1.0f / fmaxf(sqrtf(ss), kNormEps);
+            inv[u] = inv_norm(ss);
             const float sc = scale2 * inv[u];
 #pragma unroll
             for (int j = 0; j < 8; j++) bq[u][j] = (SE)(x[j] * sc);
@@ -372,7 +383,7 @@ __global__ void __launch_bounds__(64 * NT / SUB) bwd_dq_resident_kernel(const Bw
 
         // ---- back through q / max(|q|, eps); q_hat . dq_hat is this row's share of dlogit_scale ----
         // q_hat is taken back from the fp16 score operand (q_hat s log2e), which is live anyway
-        const float unscale = 1.0f / scale2;
+        const float unscale = fast_rcp(scale2);
         int ln2 = lane;
         asm volatile("" : "+v"(ln2));
 #pragma unroll
@@ -398,7 +409,7 @@ __global__ void __launch_bounds__(64 * NT / SUB) bwd_dq_resident_kernel(const Bw
             }
         }
 
-        __syncthreads();
+        lds_barrier();         // next unit staged; everybody is done with the current buffers (the stores stay in flight)
         cur ^= 1;
         c = cn;
     }
