@@ -222,41 +222,43 @@ __global__ void __launch_bounds__(64 * NT / SUB) bwd_dq_resident_kernel(const Bw
     // queries) by DMA, 16 rows per instruction; lse and delta of its queries in registers ----
     // issued by hand (see dma16_to_lds): the compiler would otherwise wait for the whole fetch in front of the
     // first transposing LDS read of every unit, which it cannot tell from the landing areas
-    auto dma16 = [&](const void* unit, uint32_t byte_offset, uint32_t lds_wave_base) __attribute__((always_inline)) {
-        dma16_to_lds(unit, byte_offset, lds_wave_base);
-    };
-    auto fetch = [&](int b) __attribute__((always_inline)) {
+    // The fetch of a unit comes in four parts (k rows with lse and delta, v, q, dO rows), each issued behind one of
+    // the first four key groups of the unit before: requested in one burst right behind the barrier, the eighty
+    // instructions of a workgroup queue up in the address unit for as long as two key groups take, with every
+    // wavefront waiting in that queue and nothing to compute.
+    auto fetch_part = [&](int b, int part) __attribute__((always_inline)) {
         // lane-derived offsets are re-materialised here: hoisted out of the unit loop they would occupy
         // a dozen registers for the whole kernel
         int ln = lane;
         asm volatile("" : "+v"(ln));
         const int fc8 = (ln & 3) * 8;
-        // unit starts in scalar registers, rows as 32-bit byte offsets from them
-        const void* kunit = uniform_pointer(unit_ptr<MAPPED, E>(p.k, p.map, b, h));
-        const void* vunit = uniform_pointer(unit_ptr<MAPPED, E>(p.v, p.map, b, h));
-        const void* qunit = uniform_pointer(unit_ptr<MAPPED, E>(p.q, p.map, b, h));
-        const void* dounit = uniform_pointer(unit_ptr<MAPPED, E>(p.d_o, p.map, b, h));
+        const T4& t = part == 0 ? p.k : (part == 1 ? p.v : (part == 2 ? p.q : p.d_o));
+        // unit start in scalar registers, rows as 32-bit byte offsets from it; landing addresses as integers from
+        // the arrays' starts (the address of a __shared__ array is a compile-time constant; no pointer leaves the
+        // LDS address space on the way)
+        const void* unit = uniform_pointer(unit_ptr<MAPPED, E>(t, p.map, b, h));
+        const uint32_t base = part == 0 ? lds_address(lds_rawK)
+                                        : (part == 1 ? lds_address(lds_rawV) : (part == 2 ? lds_address(lds_rawQ) : lds_address(lds_rawDO)));
 #pragma unroll
         for (int u = 0; u < SUB; u++) {
             const int row0 = wave * WR + 16 * u;
             const int frow = row0 + (ln >> 2);
-            if (frow < N) {
-                const int pos = unit_row<MAPPED>(p.map, b, frow);
-                // landing addresses as integers from the arrays' starts (the address of a __shared__ array is a
-                // compile-time constant; no pointer leaves the LDS address space on the way)
-                const uint32_t land = (uint32_t)(row0 * 32 * sizeof(E));
-                dma16(kunit, row_byte_offset<E>(pos, p.k.sn, fc8), lds_address(lds_rawK) + land);
-                dma16(vunit, row_byte_offset<E>(pos, p.v.sn, fc8), lds_address(lds_rawV) + land);
-                dma16(qunit, row_byte_offset<E>(pos, p.q.sn, fc8), lds_address(lds_rawQ) + land);
-                dma16(dounit, row_byte_offset<E>(pos, p.d_o.sn, fc8), lds_address(lds_rawDO) + land);
+            if (frow < N)
+                dma16_to_lds(unit, row_byte_offset<E>(unit_row<MAPPED>(p.map, b, frow), t.sn, fc8),
+                             base + (uint32_t)(row0 * 32 * sizeof(E)));
+        }
+        if (part == 0) {
+            // lse and delta of the wavefront's rows, one row per lane
+            const int q = wave * WR + ln;
+            if (ln < WR && q < N) {
+                dma4_to_lds(p.lse + b * p.lse_sb + h * p.lse_sh + q, lds_address(lds_rawLse + wave * WR));
+                dma4_to_lds(p.delta + ((int64_t)b * p.heads + h) * p.delta_stride + q, lds_address(lds_rawDelta + wave * WR));
             }
         }
-        // lse and delta of the wavefront's rows, one row per lane
-        const int q = wave * WR + ln;
-        if (ln < WR && q < N) {
-            dma4_to_lds(p.lse + b * p.lse_sb + h * p.lse_sh + q, lds_address(lds_rawLse + wave * WR));
-            dma4_to_lds(p.delta + ((int64_t)b * p.heads + h) * p.delta_stride + q, lds_address(lds_rawDelta + wave * WR));
-        }
+    };
+    auto fetch = [&](int b) __attribute__((always_inline)) {
+#pragma unroll
+        for (int part = 0; part < 4; part++) fetch_part(b, part);
     };
     auto stage = [&](int buf) __attribute__((always_inline)) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -340,7 +342,7 @@ __global__ void __launch_bounds__(64 * NT / SUB) bwd_dq_resident_kernel(const Bw
 #pragma unroll
             for (int i = 0; i < 4; i++) { dqacc[u][0][i] = 0.f; dqacc[u][1][i] = 0.f; ndv[u][i] = nd; }
         }
-        if (more) fetch(unit_of(cn));      // in flight while this unit is computed
+        const int b_next = more ? unit_of(cn) : 0;
 
         const SE* Kb = &lds_K[cur][0];
         const E* Vb = &lds_V[cur][0];
@@ -374,8 +376,14 @@ __global__ void __launch_bounds__(64 * NT / SUB) bwd_dq_resident_kernel(const Bw
         };
         auto body = [&](bool folded) __attribute__((always_inline)) {
 #pragma unroll
-            for (int kp = 0; kp < NT / 2; kp++)
+            for (int kp = 0; kp < NT / 2; kp++) {
                 if (32 * kp < N) group(kp, folded);
+                if (kp < 4 && more) fetch_part(b_next, kp);      // in flight while the rest of this unit is computed
+            }
+            if (more) {
+#pragma unroll
+                for (int part = NT / 2; part < 4; part++) fetch_part(b_next, part);     // tiles of fewer than four groups
+            }
         };
         if (fold) body(true); else body(false);
 
