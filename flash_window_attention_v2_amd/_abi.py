@@ -14,7 +14,7 @@ ABI_VERSION = 3
 OK, ERR_INVALID_ARGUMENT, ERR_UNSUPPORTED, ERR_HIP, ERR_NO_DEVICE = range(5)
 F16, BF16, F32 = 0, 1, 2
 SCALE_DEFAULT, SCALE_TENSOR = 0, 1
-STATIC_SCRATCH_BYTES = 64 << 20     # FWA2_STATIC_SCRATCH_BYTES of include/fwa2.h
+STATIC_SCRATCH_BYTES = 128 << 20    # FWA2_STATIC_SCRATCH_BYTES of include/fwa2.h
 MASK_REGION_BYTES = 272             # FWA2_MASK_REGION_BYTES of include/fwa2.h
 
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libfwa2.so")

@@ -230,15 +230,20 @@ int fwa2_backward(const fwa2_problem* p);
  * Has no counterpart in the reference (whose launcher allocates dq_accum, db_accum, dscale_accum and delta with
  * torch on every call, attn_kernel_backward.py:582-626).
  *   - a problem whose fwa2_backward_workspace_bytes() exceeds FWA2_STATIC_SCRATCH_BYTES is refused with
- *     FWA2_ERR_UNSUPPORTED (windows of 256 tokens with bias and mask fit up to about 10 workgroups per head
- *     and launch; the 4 096-window benchmark shape does not: use fwa2_backward there);
+ *     FWA2_ERR_UNSUPPORTED.  The need grows with the batch (one fp32 delta value per query row), with the
+ *     device's compute-unit count (one N x N fp32 dbias tile per persistent workgroup) and, for windows of 161
+ *     to 256 tokens with a mask, with the number of windows per image (one N x N fp32 table slot per window and
+ *     head): 3 heads of 256-token windows with a 64-window mask need 124.5 MiB at 4 096 windows per call (the
+ *     reference's benchmark shape; fits), 80 MiB with a 16-window mask at 1 024 windows per call, 36 MiB for
+ *     64-token windows at 4 096 per call; windows of 576 tokens and more need their fp32 dk / dv partials here
+ *     too (0.7 GiB at 256 windows of 6 heads) and do not fit: use fwa2_backward there;
  *   - the device that is current at the call must be the one the tensors and the stream belong to; the address
  *     of that device's copy of the array is looked up on the first call per device;
  *   - every call on a GPU shares that GPU's array: calls that may overlap on one GPU (different streams, or
  *     different threads without ordering) race on it.  Calls on one stream are ordered and safe.  Nothing in
  *     the array needs clearing between calls: every kernel writes what a later kernel of the same call reads.
  */
-#define FWA2_STATIC_SCRATCH_BYTES ((size_t)64 << 20)
+#define FWA2_STATIC_SCRATCH_BYTES ((size_t)128 << 20)
 int fwa2_backward_static(const fwa2_problem* p);
 
 /*

@@ -181,17 +181,17 @@ def test_header_compiles_as_c_and_cxx(tmp_path):
 
 
 def test_static_scratch_backward_refuses_oversize_without_a_device(lib):
-    """The allocation-free backward sizes the problem before it looks for a device: the benchmark shape needs
-    more scratch than the library's static buffer and is refused with the limit in the message."""
-    p = _good_problem(n=256, bw=4096, heads=3, backward=True)
-    p.bias.ptr, p.bias.stride_a, p.bias.stride_n = 0x10000, 256 * 256, 256
+    """The allocation-free backward sizes the problem before it looks for a device: windows of 576 tokens need
+    more scratch than the library's static buffer and are refused with the limit in the message."""
+    p = _good_problem(n=576, bw=256, heads=6, backward=True)
+    p.bias.ptr, p.bias.stride_a, p.bias.stride_n = 0x10000, 576 * 576, 576
     p.dbias = 0x10000
     assert lib.fwa2_backward_workspace_bytes(p) > _abi.STATIC_SCRATCH_BYTES
     assert lib.fwa2_backward_static(p) == _abi.ERR_UNSUPPORTED
     msg = lib.fwa2_last_error().decode()
     assert "static buffer holds" in msg and str(_abi.STATIC_SCRATCH_BYTES) in msg
     header = open(os.path.join(ROOT, "include", "fwa2.h")).read()
-    assert re.search(r"#define FWA2_STATIC_SCRATCH_BYTES \(\(size_t\)64 << 20\)", header) and _abi.STATIC_SCRATCH_BYTES == 64 << 20
+    assert re.search(r"#define FWA2_STATIC_SCRATCH_BYTES \(\(size_t\)128 << 20\)", header) and _abi.STATIC_SCRATCH_BYTES == 128 << 20
 
 
 def test_problem_filled_the_way_a_binding_fills_it(lib):

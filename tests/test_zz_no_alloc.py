@@ -63,8 +63,9 @@ def _case(lib, batch, n_windows, heads, n, resolution, window, shift, dtype, see
 
 def test_static_scratch_backward_matches_workspace_backward_twice():
     lib = _abi.load()
-    # first a window of 256 tokens (key-side + query-side kernels, about 25 MiB of scratch) ...
-    _case(lib, batch=4, n_windows=4, heads=3, n=256, resolution=32, window=16, shift=8, dtype=torch.bfloat16, seed=11)
+    # first windows of 256 tokens with a 16-window mask (key-side + query-side kernels, score tables; about
+    # 80 MiB of scratch on a 256-CU part) ...
+    _case(lib, batch=4, n_windows=16, heads=3, n=256, resolution=64, window=16, shift=8, dtype=torch.bfloat16, seed=11)
     # ... then a smaller problem on the fused kernel, which finds the first call's leftovers in the scratch
     _case(lib, batch=2, n_windows=4, heads=2, n=64, resolution=16, window=8, shift=4, dtype=torch.float16, seed=12)
     # ... and once more the larger shape class at 144 tokens (padded tiles, other offsets into the scratch)
@@ -79,13 +80,13 @@ def test_static_scratch_backward_refuses_what_does_not_fit():
     o, lse, _ = kernels._flash_attn_forward(dev["q"], dev["k"], dev["v"], dev["logit_scale"], dev["bias"], dev["mask"],
                                             scale_type="tensor")
     p = kernels._describe(dev["q"], dev["k"], dev["v"], o, lse, dev["logit_scale"], dev["bias"], dev["mask"], None, "tensor")
-    # the same pointers described as the benchmark shape: refused on its size before anything is launched
-    p.bw, p.heads, p.n, p.n_windows = 4096, 3, 256, 64
+    # the same pointers described as 256 windows of 576 tokens: refused on its size before anything is launched
+    p.bw, p.heads, p.n, p.n_windows = 256, 6, 576, 4
     for t in (p.q, p.k, p.v, p.o):
-        t.stride_bw, t.stride_h, t.stride_n = 3 * 256 * 32, 256 * 32, 32
-    p.bias.stride_a = p.mask.stride_a = 256 * 256
-    p.bias.stride_n = p.mask.stride_n = 256
-    p.lse_stride_bw, p.lse_stride_h = 3 * 256, 256
+        t.stride_bw, t.stride_h, t.stride_n = 6 * 576 * 32, 576 * 32, 32
+    p.bias.stride_a = p.mask.stride_a = 576 * 576
+    p.bias.stride_n = p.mask.stride_n = 576
+    p.lse_stride_bw, p.lse_stride_h = 6 * 576, 576
     assert lib.fwa2_backward_workspace_bytes(ctypes.byref(p)) > _abi.STATIC_SCRATCH_BYTES
     with pytest.raises(NotImplementedError, match="static buffer holds"):
         _abi.check(lib.fwa2_backward_static(ctypes.byref(p)), "fwa2_backward_static")
