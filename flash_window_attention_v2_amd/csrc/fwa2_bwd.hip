@@ -794,32 +794,23 @@ size_t backward_workspace_bytes(int heads, int n, int bw, bool has_bias, bool ha
 }
 #endif
 
-// Persistent workgroups should all be resident at once (one that waits for a slot starts its share late; nothing
-// depends on it for correctness): ask the runtime how many fit on a CU.
-template <class K>
-static int resident_per_cu(K kern, int threads) {
-    int n = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kern, threads, 0) != hipSuccess || n < 1) n = 1;
-    return n;
-}
-
 template <int DT, bool HAS_BIAS, int MASK_DT, int NQB, int KT, bool BIG, bool MAPPED = false>
 static hipError_t launch_main(BwdParams p, const BwdPlan& pl, hipStream_t st, int* groups_out) {
     // Up to 64 tokens one launch walks masked and unmasked units alike; above that the two copies of
     // the block sequence cost occupancy (128 tokens) or spill (256), and each kind gets a launch.
     constexpr bool kOneLaunch = MASK_DT >= 0 && NQB <= 2 && !BIG;
-    // asked once per block size (the wavefront count follows the window length); a benign race at worst repeats the query
-    static std::atomic<int> fit_by_waves[17];
-    int fit = pl.waves <= 16 ? fit_by_waves[pl.waves].load(std::memory_order_relaxed) : 0;
-    if (fit == 0) {
-        if constexpr (kOneLaunch) {
-            fit = resident_per_cu(bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, 2, BIG, MAPPED>, 64 * pl.waves);
-        } else {
-            const int a = resident_per_cu(bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, 0, BIG, MAPPED>, 64 * pl.waves);
-            const int b = MASK_DT >= 0 ? resident_per_cu(bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, 1, BIG, MAPPED>, 64 * pl.waves) : a;
-            fit = a < b ? a : b;
-        }
-        if (pl.waves <= 16) fit_by_waves[pl.waves].store(fit, std::memory_order_relaxed);
+    // asked once per device and block size (the wavefront count follows the window length)
+    static std::atomic<int> fit_by_waves[17][3][kFitDevices];
+    const int wslot = pl.waves <= 16 ? pl.waves : 0;
+    int fit;
+    if constexpr (kOneLaunch) {
+        fit = resident_per_cu_cached(bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, 2, BIG, MAPPED>, 64 * pl.waves, fit_by_waves[wslot][2]);
+    } else {
+        const int a = resident_per_cu_cached(bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, 0, BIG, MAPPED>, 64 * pl.waves, fit_by_waves[wslot][0]);
+        const int b = MASK_DT >= 0 ? resident_per_cu_cached(bwd_kernel<DT, HAS_BIAS, MASK_DT, NQB, KT, 1, BIG, MAPPED>, 64 * pl.waves,
+                                                            fit_by_waves[wslot][1])
+                                   : a;
+        fit = a < b ? a : b;
     }
     const int tiles = pl.n_chunks * pl.n_chunks;
     // never more workgroups per head (and super-tile) than the plan sized the workspace for

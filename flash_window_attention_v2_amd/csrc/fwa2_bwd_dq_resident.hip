@@ -440,23 +440,19 @@ __global__ void __launch_bounds__(64 * NT / SUB) bwd_dq_resident_kernel(const Bw
 int backward_dq_resident_supported(int n) { return n >= 1 && n <= 256; }
 #endif
 
-template <class K>
-static int resident_fit(K kern, int threads) {
-    int n = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kern, threads, 0) != hipSuccess || n < 1) n = 1;
-    return n;
-}
-
 // Launches the kernel(s) and reports how many dscale partials per head they wrote.
 // SUBP: 16-row query tiles per wavefront in the launch over the unmasked units; the masked launch always
 // uses kDqSub (its tile rebuilds leave no room in 128 registers).
 template <int DT, bool HAS_BIAS, int MASK_DT, int NT, bool VEC, int SUBP = kDqSub, bool MAPPED = false>
 static hipError_t launch_nt(BwdParams p, hipStream_t st, int max_groups, int* ds_parts_out) {
     constexpr int SUBM = kDqSub;
-    static const int fit_plain =
-        resident_fit(bwd_dq_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, false, SUBP, MAPPED>, 64 * NT / SUBP);
-    static const int fit_masked =
-        MASK_DT >= 0 ? resident_fit(bwd_dq_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, true, SUBM, MAPPED>, 64 * NT / SUBM) : 1;
+    static std::atomic<int> fit_plain_by_device[kFitDevices], fit_masked_by_device[kFitDevices];
+    const int fit_plain = resident_per_cu_cached(bwd_dq_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, false, SUBP, MAPPED>,
+                                                 64 * NT / SUBP, fit_plain_by_device);
+    const int fit_masked =
+        MASK_DT >= 0 ? resident_per_cu_cached(bwd_dq_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, true, SUBM, MAPPED>,
+                                              64 * NT / SUBM, fit_masked_by_device)
+                     : 1;
     auto groups_for = [&](int fit) {
         int groups = (p.cus * fit) / p.heads;
         if (groups < 1) groups = 1;

@@ -456,22 +456,18 @@ __global__ void __launch_bounds__(64 * NT, 3) bwd_fused_kernel(const BwdParams p
 // ---- host side -----------------------------------------------------------------
 int backward_fused_supported(int n) { return n >= 1 && n <= 64; }
 
-template <class K>
-static int resident_fit(K kern, int threads) {
-    int n = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kern, threads, 0) != hipSuccess || n < 1) n = 1;
-    return n;
-}
-
 // Launches the kernel(s); reports how many partial tiles / dscale partials per head they wrote.
 template <int DT, bool HAS_BIAS, int MASK_DT, bool VEC, bool MAPPED>
 static hipError_t launch_map(BwdParams p, hipStream_t st, int max_groups, int* parts_out) {
     constexpr int NT = 4;
     // wavefront pairs share a 32-key group in phase B, so there is always an even number of them
     const int waves = 2 * ((p.n + 31) / 32);
-    static const int fit_plain = resident_fit(bwd_fused_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, false, MAPPED>, 64 * NT);
-    static const int fit_masked =
-        MASK_DT >= 0 ? resident_fit(bwd_fused_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, true, MAPPED>, 64 * NT) : 1;
+    static std::atomic<int> fit_plain_by_device[kFitDevices], fit_masked_by_device[kFitDevices];
+    const int fit_plain =
+        resident_per_cu_cached(bwd_fused_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, false, MAPPED>, 64 * NT, fit_plain_by_device);
+    const int fit_masked =
+        MASK_DT >= 0 ? resident_per_cu_cached(bwd_fused_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, true, MAPPED>, 64 * NT, fit_masked_by_device)
+                     : 1;
     auto groups_for = [&](int fit) {
         int groups = (p.cus * fit) / p.heads;
         if (groups < 1) groups = 1;

@@ -569,21 +569,10 @@ __global__ void __launch_bounds__(256) build_table_kernel(const E* bias, int64_t
 }
 
 // ---- host side -----------------------------------------------------------------
-template <class K>
-static int resident_per_cu(K kern, int threads) {
-    int n = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kern, threads, 0) != hipSuccess || n < 1) n = 1;
-    return n;
-}
-
 template <int DT, bool HAS_BIAS, bool HAS_TAB, bool MASKED, bool MAPPED>
 static hipError_t launch_key(BwdParams p, hipStream_t st, int max_groups, int* groups_out) {
-    static std::atomic<int> fit_cached{0};
-    int fit = fit_cached.load(std::memory_order_relaxed);
-    if (fit == 0) {
-        fit = resident_per_cu(bwd_key_kernel<DT, HAS_BIAS, HAS_TAB, MASKED, MAPPED>, key256::NT);
-        fit_cached.store(fit, std::memory_order_relaxed);
-    }
+    static std::atomic<int> fit_by_device[kFitDevices];
+    const int fit = resident_per_cu_cached(bwd_key_kernel<DT, HAS_BIAS, HAS_TAB, MASKED, MAPPED>, key256::NT, fit_by_device);
     int groups = (p.cus * fit) / p.heads;
     if (groups < 1) groups = 1;
     if (groups > max_groups) groups = max_groups;

@@ -6,9 +6,28 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/fwa2.h"
 
 namespace fwa2 {
+
+// Workgroups of `kern` that fit on one compute unit of the CURRENT device: asked from the runtime once per device
+// and call site (`slots` is the call site's static array, kFitDevices entries; a benign race at worst repeats
+// the query).  Persistent workgroups should all be resident at once: one that waits for a slot starts its share
+// late (nothing depends on it for correctness).
+constexpr int kFitDevices = 64;
+template <class K>
+static inline int resident_per_cu_cached(K kern, int threads, std::atomic<int>* slots) {
+    int dev = 0;
+    const bool tracked = hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < kFitDevices;
+    int n = tracked ? slots[dev].load(std::memory_order_relaxed) : 0;
+    if (n == 0) {
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kern, threads, 0) != hipSuccess || n < 1) n = 1;
+        if (tracked) slots[dev].store(n, std::memory_order_relaxed);
+    }
+    return n;
+}
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));

@@ -527,13 +527,6 @@ int forward_resident_supported(int n) { return n >= 1 && n <= 256; }
 constexpr int kFwdSub = FWA2_FWD_SUB;    // 16-row query tiles per wavefront of the 256-token forward (unmasked launch)
 constexpr int kRegionMaxImages = 32;     // images per window up to which region records are used (see launch_map)
 
-template <class K>
-static int resident_fit(K kern, int threads) {
-    int n = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kern, threads, 0) != hipSuccess || n < 1) n = 1;
-    return n;
-}
-
 // SUBP: 16-row query tiles per wavefront in the launch over the unmasked units (the masked launch keeps one:
 // its tile rebuilds want the registers).
 template <int DT, bool HAS_BIAS, int MASK_DT, int NT, bool VEC, bool MAPPED, int SUBP>
@@ -541,10 +534,12 @@ static hipError_t launch_map(FwdParams p, hipStream_t st) {
     const int waves_plain = (p.n + 16 * SUBP - 1) / (16 * SUBP);
     const int waves_masked = (p.n + 15) / 16;
     // the runtime's figure is for full groups; smaller groups only fit better
-    static const int fit_plain =
-        resident_fit(fwd_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, false, MAPPED, SUBP>, 64 * NT / SUBP);
-    static const int fit_masked =
-        MASK_DT >= 0 ? resident_fit(fwd_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, true, MAPPED, 1>, 64 * NT) : 1;
+    static std::atomic<int> fit_plain_by_device[kFitDevices], fit_masked_by_device[kFitDevices];
+    const int fit_plain = resident_per_cu_cached(fwd_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, false, MAPPED, SUBP>,
+                                                 64 * NT / SUBP, fit_plain_by_device);
+    const int fit_masked = MASK_DT >= 0 ? resident_per_cu_cached(fwd_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, true, MAPPED, 1>,
+                                                                 64 * NT, fit_masked_by_device)
+                                        : 1;
     auto groups_for = [&](int fit) {
         int groups = (p.cus * fit) / p.heads;
         if (groups < 1) groups = 1;
