@@ -56,12 +56,12 @@ __global__ void __launch_bounds__(512) bwd_dq_kernel(const BwdParams p) {
     const int b = idx / p.heads;
 
     // rows are addressed through the window map when there is one (cyclic shift + window partition done here)
-    const E* qbase = reinterpret_cast<const E*>(p.q.ptr);
-    const E* kbase = reinterpret_cast<const E*>(p.k.ptr);
-    const E* vbase = reinterpret_cast<const E*>(p.v.ptr);
-    const E* obase = reinterpret_cast<const E*>(p.o.ptr);
-    const E* dobase = reinterpret_cast<const E*>(p.d_o.ptr);
-    E* dqbase = reinterpret_cast<E*>(const_cast<void*>(p.dq.ptr));
+    const E* qptr = reinterpret_cast<const E*>(p.q.ptr) + unit_off_any(p.q, p.map, b, h);
+    const E* kptr = reinterpret_cast<const E*>(p.k.ptr) + unit_off_any(p.k, p.map, b, h);
+    const E* vptr = reinterpret_cast<const E*>(p.v.ptr) + unit_off_any(p.v, p.map, b, h);
+    const E* optr = reinterpret_cast<const E*>(p.o.ptr) + unit_off_any(p.o, p.map, b, h);
+    const E* doptr = reinterpret_cast<const E*>(p.d_o.ptr) + unit_off_any(p.d_o, p.map, b, h);
+    E* dqptr = reinterpret_cast<E*>(const_cast<void*>(p.dq.ptr)) + unit_off_any(p.dq, p.map, b, h);
 
     float s_true;
     if (p.scale_kind == FWA2_SCALE_TENSOR) {
@@ -84,9 +84,10 @@ __global__ void __launch_bounds__(512) bwd_dq_kernel(const BwdParams p) {
     if (wave_live) {
         V8 a = zero8<V8>(), c = zero8<V8>(), o0 = zero8<V8>(), o1 = zero8<V8>();
         if (qv) {
-            const E* qrow = qbase + row_off_any(p.q, p.map, b, h, qi);
-            const E* dorow = dobase + row_off_any(p.d_o, p.map, b, h, qi);
-            const E* orow = obase + row_off_any(p.o, p.map, b, h, qi);
+            const int qpos = unit_row_any(p.map, b, qi);
+            const E* qrow = qptr + (int64_t)qpos * p.q.sn;
+            const E* dorow = doptr + (int64_t)qpos * p.d_o.sn;
+            const E* orow = optr + (int64_t)qpos * p.o.sn;
             a = ld8<V8>(qrow + 8 * hf);
             c = ld8<V8>(qrow + 16 + 8 * hf);
             bd0 = ld8<V8>(dorow + 8 * hf);
@@ -135,8 +136,9 @@ __global__ void __launch_bounds__(512) bwd_dq_kernel(const BwdParams p) {
             const int dch = (tid & 3) * 8;
             V8 kk = zero8<V8>(), vv = zero8<V8>();
             if (r < rows) {
-                kk = ld8<V8>(kbase + row_off_any(p.k, p.map, b, h, c0 + r) + dch);
-                vv = ld8<V8>(vbase + row_off_any(p.v, p.map, b, h, c0 + r) + dch);
+                const int pos = unit_row_any(p.map, b, c0 + r);
+                kk = ld8<V8>(kptr + (int64_t)pos * p.k.sn + dch);
+                vv = ld8<V8>(vptr + (int64_t)pos * p.v.sn + dch);
             }
             float x[8];
             unpack8(kk, x);
@@ -219,7 +221,7 @@ __global__ void __launch_bounds__(512) bwd_dq_kernel(const BwdParams p) {
             V4 q4;
 #pragma unroll
             for (int j = 0; j < 4; j++) q4[j] = 0;
-            if (qv) q4 = *reinterpret_cast<const V4*>(qbase + row_off_any(p.q, p.map, b, h, qi) + 8 * c + 4 * hf);
+            if (qv) q4 = *reinterpret_cast<const V4*>(qptr + (int64_t)unit_row_any(p.map, b, qi) * p.q.sn + 8 * c + 4 * hf);
 #pragma unroll
             for (int j = 0; j < 4; j++) { x[4 * c + j] = (float)q4[j]; ss += x[4 * c + j] * x[4 * c + j]; }
         }
@@ -237,7 +239,7 @@ __global__ void __launch_bounds__(512) bwd_dq_kernel(const BwdParams p) {
                 V4 o4;
 #pragma unroll
                 for (int j = 0; j < 4; j++) o4[j] = (E)(f * (dqacc[4 * c + j] - x[4 * c + j] * proj));
-                *reinterpret_cast<V4*>(dqbase + row_off_any(p.dq, p.map, b, h, qi) + 8 * c + 4 * hf) = o4;
+                *reinterpret_cast<V4*>(dqptr + (int64_t)unit_row_any(p.map, b, qi) * p.dq.sn + 8 * c + 4 * hf) = o4;
             }
         }
         if (!qv || hf != 0) dot = 0.f;

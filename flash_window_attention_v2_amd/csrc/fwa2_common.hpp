@@ -389,6 +389,15 @@ __device__ __forceinline__ const E* row_ptr(const T4& t, const WinMap& m, int b,
     return row_at(unit_ptr<MAPPED, E>(t, m, b, h), unit_row<MAPPED>(m, b, row), t.sn, col);
 }
 
+// The two halves of that for a loop over rows: the unit's start (uniform, taken once) and the row's position
+// inside it.
+__device__ __forceinline__ int64_t unit_off_any(const T4& t, const WinMap& m, int b, int h) {
+    return (m.nw > 0 ? (int64_t)(b / m.nw) * t.sb : (int64_t)b * t.sb) + h * t.sh;
+}
+__device__ __forceinline__ int unit_row_any(const WinMap& m, int b, int row) {
+    return m.nw > 0 ? unit_row<true>(m, b, row) : row;
+}
+
 struct FwdParams {
     T4 q, k, v, o;
     WinMap map;

@@ -61,10 +61,10 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdParams p) {
     const int b = idx / p.heads;
 
     // rows are addressed through the window map when there is one (cyclic shift + window partition done here)
-    const E* qbase = reinterpret_cast<const E*>(p.q.ptr);
-    const E* kbase = reinterpret_cast<const E*>(p.k.ptr);
-    const E* vbase = reinterpret_cast<const E*>(p.v.ptr);
-    E* obase = reinterpret_cast<E*>(const_cast<void*>(p.o.ptr));
+    const E* qptr = reinterpret_cast<const E*>(p.q.ptr) + unit_off_any(p.q, p.map, b, h);
+    const E* kptr = reinterpret_cast<const E*>(p.k.ptr) + unit_off_any(p.k, p.map, b, h);
+    const E* vptr = reinterpret_cast<const E*>(p.v.ptr) + unit_off_any(p.v, p.map, b, h);
+    E* optr = reinterpret_cast<E*>(const_cast<void*>(p.o.ptr)) + unit_off_any(p.o, p.map, b, h);
 
     float scale2;
     if (p.scale_kind == FWA2_SCALE_TENSOR) {
@@ -84,7 +84,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdParams p) {
     if (wave_live) {
         V8 a = zero8<V8>(), c = zero8<V8>();
         if (qv) {
-            const E* qrow = qbase + row_off_any(p.q, p.map, b, h, qi);
+            const E* qrow = qptr + (int64_t)unit_row_any(p.map, b, qi) * p.q.sn;
             a = ld8<V8>(qrow + 8 * hf);
             c = ld8<V8>(qrow + 16 + 8 * hf);
         }
@@ -125,8 +125,9 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdParams p) {
             const int dch = (tid & 3) * 8;
             V8 kk = zero8<V8>(), vv = zero8<V8>();
             if (r < rows) {
-                kk = ld8<V8>(kbase + row_off_any(p.k, p.map, b, h, c0 + r) + dch);
-                vv = ld8<V8>(vbase + row_off_any(p.v, p.map, b, h, c0 + r) + dch);
+                const int pos = unit_row_any(p.map, b, c0 + r);
+                kk = ld8<V8>(kptr + (int64_t)pos * p.k.sn + dch);
+                vv = ld8<V8>(vptr + (int64_t)pos * p.v.sn + dch);
             }
             float x[8];
             unpack8(kk, x);
@@ -239,7 +240,7 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdParams p) {
             V4 ov;
 #pragma unroll
             for (int j = 0; j < 4; j++) ov[j] = (E)(oacc[4 * c + j] * inv_l);
-            *reinterpret_cast<V4*>(obase + row_off_any(p.o, p.map, b, h, qi) + 8 * c + 4 * hf) = ov;
+            *reinterpret_cast<V4*>(optr + (int64_t)unit_row_any(p.map, b, qi) * p.o.sn + 8 * c + 4 * hf) = ov;
         }
         if (hf == 0) {
             const float lse = l_tot > 0.f ? (m_run + fast_log2(l_tot)) * kLn2 : -INFINITY;
