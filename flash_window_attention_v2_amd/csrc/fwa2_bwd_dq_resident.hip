@@ -377,6 +377,7 @@ __global__ void __launch_bounds__(64 * NT / SUB) bwd_dq_resident_kernel(const Bw
         auto body = [&](bool folded) __attribute__((always_inline)) {
 #pragma unroll
             for (int kp = 0; kp < NT / 2; kp++) {
+                progress_priority(kp, NT / 2);
                 if (32 * kp < N) group(kp, folded);
                 if (kp < 4 && more) fetch_part(b_next, kp);      // in flight while the rest of this unit is computed
             }

@@ -153,6 +153,19 @@ __device__ __forceinline__ void lds_barrier() {
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
+// Issue priority that falls as a wavefront advances through the `steps` key groups of a unit (3 in the first
+// quarter ... 0 in the last and in everything up to the next unit's first group).  The arbiter otherwise favours the
+// oldest wavefront of a SIMD, which then reaches the barrier early and leaves the end of every unit to one
+// wavefront per SIMD with nothing to hide its waits; with this, whoever is behind goes first and the wavefronts
+// of a SIMD finish together.
+__device__ __forceinline__ void progress_priority(int step, int steps) {
+    if (steps < 4) return;
+    if (step == 0) __builtin_amdgcn_s_setprio(3);
+    else if (step == steps / 4) __builtin_amdgcn_s_setprio(2);
+    else if (step == steps / 2) __builtin_amdgcn_s_setprio(1);
+    else if (step == 3 * steps / 4) __builtin_amdgcn_s_setprio(0);
+}
+
 // ---- cross-lane helpers (wave64) -------------------------------------------
 // Value held by the lane 32 away, combined with the own value by max / add.
 __device__ __forceinline__ float xor32_max(float x) {

@@ -431,6 +431,7 @@ __global__ void __launch_bounds__(64 * NT / SUB) fwd_resident_kernel(const FwdPa
 #pragma unroll
                 for (int kp = 0; kp < NT / 2; kp++) {
                     if (32 * kp < N) {
+                        progress_priority(kp, NT / 2);
                         f32x4 s0[SUB], s1[SUB];
                         scores(kp, s0, s1, with_regions);
 #pragma unroll
