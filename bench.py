@@ -8,7 +8,7 @@ synthetic batch (benchmark configuration 3: B=64 images x 64 windows of N=256 to
 logit_scale = ln 10), inputs already resident in HBM.  One JSON line goes to
 stdout; progress goes to stderr.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extras] [--sweep]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extras | --basic-extras] [--sweep]
 
 `extras` carries the forward-only and N = 64 figures, peak memory, the window-size sweep of the reference's
 operator benchmark as HIP graph replays and one end-to-end model step; `--sweep` prints the sweep alone, with
@@ -270,6 +270,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip forward-only, N=64 and memory figures")
+    ap.add_argument("--basic-extras", action="store_true",
+                    help="extras without the window-size sweep and the model step (forward-only, N=64 and memory figures only)")
     ap.add_argument("--sweep", action="store_true",
                     help="instead of the benchmark line, print the window-size sweep (TFLOP/s versus N) as one JSON line")
     ap.add_argument("--copy-bytes", type=int, default=0,
@@ -385,10 +387,11 @@ def main():
         extras["c2_tflops"] = round(flops_matmul(bw2, c2["heads"], c2["n"], c2["d"]) / ms2 * 1e-9, 2)
         del dev2
         torch.cuda.empty_cache()
-        log("[bench] window-size sweep as graph replays")
-        extras["window_sweep"] = window_sweep(torch, 10, 2, eager=False)
-        log("[bench] end-to-end model step")
-        extras["model"] = model_step(torch, 8, 2)
+        if not args.basic_extras:
+            log("[bench] window-size sweep as graph replays")
+            extras["window_sweep"] = window_sweep(torch, 10, 2, eager=False)
+            log("[bench] end-to-end model step")
+            extras["model"] = model_step(torch, 8, 2)
         result["extras"] = extras
 
     if args.copy_bytes:
