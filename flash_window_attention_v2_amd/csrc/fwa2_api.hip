@@ -200,6 +200,11 @@ fwa2::WinMap to_map(const fwa2_problem* p) {
 bool row_vec_ok(const void* ptr, int64_t sa, int64_t sn, int n) {
     return aligned16(ptr) && (sa % 8) == 0 && (sn % 8) == 0 && (n % 8) == 0;
 }
+// Rows that start on 16-byte boundaries and are long enough for whole groups of 8 entries, whatever n is (the
+// caller padded them): the entries beyond n are never used.
+bool row_groups_ok(const void* ptr, int64_t sa, int64_t sn, int n) {
+    return aligned16(ptr) && (sa % 8) == 0 && (sn % 8) == 0 && sn >= ((n + 7) & ~7);
+}
 
 }  // namespace
 
@@ -305,6 +310,8 @@ int fwa2_forward(const fwa2_problem* p) {
     k.default_scale = 1.0f / sqrtf((float)(p->scale_head_dim > 0 ? p->scale_head_dim : p->head_dim));
     k.side_vec = (!p->bias.ptr || row_vec_ok(p->bias.ptr, p->bias.stride_a, p->bias.stride_n, p->n)) &&
                  (!p->mask.ptr || row_vec_ok(p->mask.ptr, p->mask.stride_a, p->mask.stride_n, p->n));
+    k.side_vec_rows = (!p->bias.ptr || row_groups_ok(p->bias.ptr, p->bias.stride_a, p->bias.stride_n, p->n)) &&
+                      (!p->mask.ptr || row_groups_ok(p->mask.ptr, p->mask.stride_a, p->mask.stride_n, p->n));
     k.cus = cu_count();
     hipError_t e = fwa2::launch_forward(k, p->dtype, p->bias.ptr != nullptr, p->mask.ptr ? p->mask_dtype : -1,
                                         (hipStream_t)p->stream);
@@ -338,6 +345,8 @@ static int run_backward(const fwa2_problem* p) {
     k.dbias = p->dbias; k.dscale = p->dscale;
     k.side_vec = (!p->bias.ptr || row_vec_ok(p->bias.ptr, p->bias.stride_a, p->bias.stride_n, p->n)) &&
                  (!p->mask.ptr || row_vec_ok(p->mask.ptr, p->mask.stride_a, p->mask.stride_n, p->n));
+    k.side_vec_rows = (!p->bias.ptr || row_groups_ok(p->bias.ptr, p->bias.stride_a, p->bias.stride_n, p->n)) &&
+                      (!p->mask.ptr || row_groups_ok(p->mask.ptr, p->mask.stride_a, p->mask.stride_n, p->n));
     k.workspace = p->workspace;
     k.cus = cu_count();
     k.ev_start = (hipEvent_t)g_ev_start.load();

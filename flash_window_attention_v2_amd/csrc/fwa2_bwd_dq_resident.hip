@@ -487,7 +487,7 @@ static hipError_t launch_mask(const BwdParams& p, hipStream_t st, int mg, int* o
     if (p.map.nw > 0) {
         // windows of up to 64 tokens with a map go to the fused kernel, never here
         if (nt == 4) return hipErrorInvalidValue;
-        if (p.side_vec) {
+        if (p.side_vec || p.side_vec_rows) {
             if (nt == 8) return launch_nt<DT, HAS_BIAS, MASK_DT, 8, true, kDqSub, true>(p, st, mg, out);
             if (p.n <= 160) return launch_nt<DT, HAS_BIAS, MASK_DT, 10, true, 1, true>(p, st, mg, out);
             return launch_nt<DT, HAS_BIAS, MASK_DT, 16, true, kDqSub, true>(p, st, mg, out);
@@ -496,7 +496,7 @@ static hipError_t launch_mask(const BwdParams& p, hipStream_t st, int mg, int* o
         if (p.n <= 160) return launch_nt<DT, HAS_BIAS, MASK_DT, 10, false, 1, true>(p, st, mg, out);
         return launch_nt<DT, HAS_BIAS, MASK_DT, 16, false, kDqSub, true>(p, st, mg, out);
     }
-    if (p.side_vec) {
+    if (p.side_vec || p.side_vec_rows) {
         if (nt == 4) return launch_nt<DT, HAS_BIAS, MASK_DT, 4, true>(p, st, mg, out);
         if (nt == 8) return launch_nt<DT, HAS_BIAS, MASK_DT, 8, true>(p, st, mg, out);
         // 129 .. 160 tokens: tiles of 160 keys (40 registers of resident bias per 16 rows instead of 64), and 16 rows

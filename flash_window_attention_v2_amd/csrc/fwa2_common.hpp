@@ -196,11 +196,7 @@ __device__ __forceinline__ int lane_now() {
     return l;
 }
 
-#ifdef PROBE_NOEXP
-__device__ __forceinline__ float fast_exp2(float x) { return x * 0.001f; }
-#else
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
-#endif
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
 
@@ -309,9 +305,13 @@ template <bool VEC, class T>
 __device__ __forceinline__ auto load_raw8(const T* row, int c0, int n, float pad) {
     typedef T TV8 __attribute__((ext_vector_type(8)));
     TV8 v;
-    if (VEC) {   // n % 8 == 0 and rows 16-byte aligned: a group of 8 is all real or all padding
+    if (VEC) {   // rows 16-byte aligned and at least n rounded up to 8 entries long: a whole group can be read
         if (c0 < n) {
             v = *reinterpret_cast<const TV8*>(row + c0);
+            if (c0 + 8 > n) {   // the last group of a row whose length is not a multiple of 8: the tail is padding
+#pragma unroll
+                for (int i = 0; i < 8; i++) v[i] = (c0 + i < n) ? v[i] : (T)pad;
+            }
         } else {
 #pragma unroll
             for (int i = 0; i < 8; i++) v[i] = (T)pad;
@@ -430,6 +430,7 @@ struct FwdParams {
     int scale_kind;
     float default_scale;  // 1/sqrt(head_dim), used when no logit scale is given
     bool side_vec;    // rows of bias and mask may be read with 16-byte loads and n % 8 == 0
+    bool side_vec_rows;   // ... or n % 8 != 0 but every row is at least n rounded up to 8 entries long (resident kernels)
     int waves;        // wavefronts per workgroup
     int q_chunks;     // workgroups per (bw, head)
     int cus;          // compute units of the device
@@ -476,6 +477,7 @@ struct BwdParams {
     int dq_waves;        // wavefronts per workgroup of the dq kernel
     int dq_chunks;       // dq workgroups per (bw, head)
     bool side_vec;       // rows of bias and mask (query-major) may be read with 16-byte loads, n % 8 == 0
+    bool side_vec_rows;  // ... or n % 8 != 0 but every row is at least n rounded up to 8 entries long (resident kernels)
     const void* bias_t;  // [H, NP, NQ] input dtype: bias transposed to key-major, zero padded
     const void* mask_t;  // [nW, NP, NQ] mask dtype: mask transposed to key-major, zero padded
     const float* tab;    // table mode of the key-side kernel: (bias + mask) * log2e in accumulator order, slot h for

@@ -577,7 +577,7 @@ static hipError_t launch_nt(const FwdParams& p, hipStream_t st) {
 template <int DT, bool HAS_BIAS, int MASK_DT>
 static hipError_t launch_mask(const FwdParams& p, hipStream_t st) {
     const int nt = p.n <= 64 ? 4 : (p.n <= 128 ? 8 : 16);
-    if (p.side_vec) {
+    if (p.side_vec || p.side_vec_rows) {
         if (nt == 4) return launch_nt<DT, HAS_BIAS, MASK_DT, 4, true>(p, st);
         if (nt == 8) return launch_nt<DT, HAS_BIAS, MASK_DT, 8, true>(p, st);
         return launch_nt<DT, HAS_BIAS, MASK_DT, 16, true>(p, st);

@@ -105,6 +105,27 @@ def mask_window_flags(mask):
     return live
 
 
+def _rows_of_8(t, cache):
+    """`t` ([A, N, N], N not a multiple of 8) with rows padded to the next multiple of 8 entries.  With `cache`
+    the copy is kept on the tensor object under the same rules as the mask flags (a mask is the same tensor call
+    after call; a bias is rebuilt every step)."""
+    if t is None or t.shape[-1] % 8 == 0:
+        return t
+    version = tensor_version(t) if cache else None
+    key = (version, t.data_ptr(), t.device)
+    if version is not None:
+        cached = getattr(t, "_fwa2_rows8", None)
+        if cached is not None and cached[0] == key:
+            return cached[1]
+    padded = torch.nn.functional.pad(t, (0, -t.shape[-1] % 8))
+    if version is not None and not torch.cuda.is_current_stream_capturing():
+        try:
+            t._fwa2_rows8 = (key, padded)
+        except Exception:
+            pass
+    return padded
+
+
 def _describe(q, k, v, o, lse, logit_scale, bias, mask, mask_live, scale_type, window_map=None, scale_dim=0):
     bw, heads, n, d = q.shape
     p = _abi.new_problem()
@@ -123,6 +144,13 @@ def _describe(q, k, v, o, lse, logit_scale, bias, mask, mask_live, scale_type, w
     _set_t4(p.q, q); _set_t4(p.k, k); _set_t4(p.v, v); _set_t4(p.o, o)
     if scale_type == "tensor":
         p.logit_scale = logit_scale.data_ptr()
+    if 64 < n <= 256 and n % 8 and p.n_keys == 0:
+        # Windows such as 14 x 14 tokens: rows of bias and mask start off 16-byte boundaries, which would put the
+        # resident-tile kernels on element-wise loads.  Copies with rows padded to a multiple of 8 entries keep
+        # them on 16-byte loads; the kernels never use the entries beyond n.  The copies live as long as the
+        # problem description (the launch that follows is ordered behind them on the same stream).
+        bias, mask = _rows_of_8(bias, cache=False), _rows_of_8(mask, cache=True)
+        p._keep = (bias, mask)
     if bias is not None:
         p.bias.ptr, p.bias.stride_a, p.bias.stride_n = bias.data_ptr(), bias.stride(0), bias.stride(1)
     if mask is not None:

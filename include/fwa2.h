@@ -69,7 +69,11 @@ typedef struct fwa2_tensor4 {
     int64_t stride_n;
 } fwa2_tensor4;
 
-/* A [A, N, N] tensor (bias: A = H, mask: A = nW) with unit innermost stride. */
+/* A [A, N, N] tensor (bias: A = H, mask: A = nW) with unit innermost stride.  stride_n >= N; the elements of a
+ * row past its N-th are never used.  The kernels read bias and mask with 16-byte loads when ptr is 16-byte
+ * aligned, both strides are multiples of 8 elements and stride_n >= N rounded up to a multiple of 8; a caller
+ * whose N is not a multiple of 8 gets that path by padding the rows (with anything), and the element-wise path
+ * otherwise. */
 typedef struct fwa2_tensor3 {
     void*   ptr;       /* NULL = absent */
     int64_t stride_a;

@@ -136,10 +136,10 @@ def test_more_windows_than_the_flag_cache_and_no_flags(monkeypatch):
     assert len(described) == 6 and all(ptr is None for ptr in described), described
 
 
-@pytest.mark.parametrize("n", [1, 7, 17, 31, 33, 47, 63, 65, 100, 129, 200, 255])
+@pytest.mark.parametrize("n", [1, 7, 17, 31, 33, 47, 63, 65, 100, 129, 196, 200, 225, 255])
 def test_ragged_window_sizes(n):
-    """Window sizes that are no multiple of 8, 16 or 32 (element-wise side loads, padded query rows and key
-    columns, odd numbers of wavefronts), with a random 0 / -100 mask on some windows, forward and backward."""
+    """Window sizes that are no multiple of 8, 16 or 32 (bias and mask rows padded to 8 entries above 64 tokens
+    and element-wise side loads below, padded query rows and key columns, odd numbers of wavefronts), with a random 0 / -100 mask on some windows, forward and backward."""
     dtype = torch.bfloat16 if n % 2 else torch.float16
     n_w = 3
     inp = make_inputs(batch=2, n_windows=n_w, heads=2, n=n, dtype=dtype, seed=100 + n, with_mask=False)
