@@ -56,8 +56,13 @@ class _on_device:
 def _rows_16b_aligned(t):
     """What the kernels address directly: unit inner stride, rows on 16-byte boundaries, and a row stride small
     enough for the 32-bit offsets they use inside one unit (below 2^24 elements, rows x stride below 2^30)."""
-    return (t.stride(-1) == 1 and t.data_ptr() % 16 == 0 and all(s % 8 == 0 for s in t.stride()[:-1])
-            and t.stride(-2) < (1 << 24) and t.shape[-2] * t.stride(-2) < (1 << 30))
+    st = t.stride()
+    if len(st) == 4:            # q, k, v, o and their gradients: no generator in the way
+        s0, s1, s2, s3 = st
+        return (s3 == 1 and (s0 | s1 | s2) % 8 == 0 and t.data_ptr() % 16 == 0 and s2 < (1 << 24)
+                and t.shape[2] * s2 < (1 << 30))
+    return (st[-1] == 1 and t.data_ptr() % 16 == 0 and all(s % 8 == 0 for s in st[:-1])
+            and st[-2] < (1 << 24) and t.shape[-2] * st[-2] < (1 << 30))
 
 
 def _kernel_ready(t):
