@@ -32,7 +32,7 @@ HBM_PEAK_GBS = 8000.0              # MI355X HBM3E
 # HBM bytes per launch of the key-side backward kernel at the benchmark shape, from
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a copy kernel of known size
 # (profiles/kernels_C3_fwd_bwd.txt: FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0).
-BWD_KERNEL_TRAFFIC_BYTES = 1.631e9
+BWD_KERNEL_TRAFFIC_BYTES = 1.630e9
 
 
 def log(*a):
