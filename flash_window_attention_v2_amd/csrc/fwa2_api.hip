@@ -221,6 +221,15 @@ int fwa2_validate(const fwa2_problem* p, int backward) {
 
 size_t fwa2_backward_workspace_bytes(const fwa2_problem* p) {
     if (p == nullptr) return 0;
+    // sizes fwa2_validate refuses: nothing to reserve
+    if (p->bw <= 0 || p->heads <= 0 || p->n <= 0 || p->head_dim <= 0 || p->n_keys < 0) return 0;
+    if (p->mask.ptr != nullptr && (p->n_windows <= 0 || p->n_windows > p->bw)) return 0;
+    {
+        // sizes no device can hold (the partial tiles of dbias, the partial sums of dk / dv): answered without
+        // forming the products, which would wrap
+        const double n = p->n, nk = p->n_keys > 0 ? p->n_keys : p->n, units = (double)p->bw * p->heads;
+        if (p->heads * n * (n > nk ? n : nk) > 0x1p44 || units * n * (n > nk ? n : nk) > 0x1p52) return SIZE_MAX;
+    }
     if (fwa2::generic_problem(p->head_dim, p->n, p->n_keys > 0 ? p->n_keys : p->n))
         return fwa2::generic_workspace_bytes(p->heads, p->n, p->n_keys > 0 ? p->n_keys : p->n, p->bw, p->bias.ptr != nullptr);
     return fwa2::backward_workspace_bytes(p->heads, p->n, p->bw, p->bias.ptr != nullptr, p->mask.ptr != nullptr,

@@ -206,7 +206,12 @@ int fwa2_mask_scan_regions(const void* mask, int mask_dtype, int n_windows, int 
 /*
  * Bytes of device scratch fwa2_backward needs for this problem on the CURRENT
  * device (fp32 accumulators for dbias and dscale; the reference allocates these
- * as db_accum / dscale_accum, attn_kernel_backward.py:609-626).  0 if none.
+ * as db_accum / dscale_accum, attn_kernel_backward.py:609-626).  0 if none, or
+ * if bw, heads, n, head_dim or the mask's n_windows is out of range
+ * (fwa2_validate names the field);
+ * SIZE_MAX for sizes no device can hold (heads * n^2 beyond 2^44 or
+ * bw * heads * n^2 beyond 2^52), which fwa2_validate then reports as a
+ * workspace that is too small.
  * The figure grows with the device's compute-unit count (one partial dbias
  * tile per persistent workgroup); see fwa2_validate.
  */

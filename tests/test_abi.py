@@ -118,6 +118,50 @@ def test_validate_accepts_and_rejects(lib):
     assert lib.fwa2_validate(p, 1) == _abi.ERR_INVALID_ARGUMENT
 
 
+def test_validate_survives_arbitrary_descriptions(lib):
+    """Seeded random problem descriptions (sizes from zero to absurd, negative strides, odd pointers, window maps
+    that do not divide the grid): fwa2_validate and the workspace query only ever answer with a status or a size,
+    on a machine without a GPU too, and a rejected description always leaves a message."""
+    import random
+    rng = random.Random(20240607)
+    sizes = [-3, 0, 1, 2, 7, 8, 31, 32, 63, 64, 100, 144, 196, 256, 257, 576, 1024, 1025, 4096, 1 << 20, (1 << 31) - 1]
+    strides = [-64, 0, 1, 8, 31, 32, 40, 64, 2048, 4096, 1 << 20, 1 << 24, 1 << 40, (1 << 62)]
+    ptrs = [0, 0x10000, 0x10002, 0x10008, 0x7fff00000010]
+    seen = set()
+    for _ in range(4000):
+        backward = rng.random() < 0.5
+        p = _good_problem(n=rng.choice([64, 144, 256, 576]), bw=rng.choice([1, 8, 64]), heads=rng.choice([1, 3]),
+                          backward=backward)
+        for _ in range(rng.randint(1, 4)):
+            what = rng.randrange(12)
+            if what == 0: p.n = rng.choice(sizes)
+            elif what == 1: p.bw = rng.choice(sizes)
+            elif what == 2: p.heads = rng.choice(sizes)
+            elif what == 3: p.head_dim = rng.choice(sizes)
+            elif what == 4: p.n_keys = rng.choice(sizes)
+            elif what == 5: p.n_windows = rng.choice(sizes)
+            elif what == 6:
+                t = rng.choice([p.q, p.k, p.v, p.o, p.d_o, p.dq, p.dk, p.dv])
+                t.ptr, t.stride_bw, t.stride_h, t.stride_n = (rng.choice(ptrs), rng.choice(strides), rng.choice(strides),
+                                                               rng.choice(strides))
+            elif what == 7:
+                t = rng.choice([p.bias, p.mask])
+                t.ptr, t.stride_a, t.stride_n = rng.choice(ptrs), rng.choice(strides), rng.choice(strides)
+            elif what == 8:
+                p.grid_h, p.grid_w, p.win_h, p.win_w, p.shift_h, p.shift_w = (rng.choice(sizes[:12]) for _ in range(6))
+            elif what == 9: p.dtype, p.mask_dtype = rng.randrange(-1, 5), rng.randrange(-1, 5)
+            elif what == 10: p.scale_kind, p.scale_head_dim = rng.randrange(-1, 4), rng.choice(sizes[:10])
+            else: p.lse_stride_bw, p.lse_stride_h, p.workspace_bytes = rng.choice(strides), rng.choice(strides), rng.choice(sizes)
+        st = lib.fwa2_validate(p, int(backward))
+        assert st in (_abi.OK, _abi.ERR_INVALID_ARGUMENT, _abi.ERR_UNSUPPORTED), st
+        if st != _abi.OK:
+            assert len(lib.fwa2_last_error()) > 0
+        need = lib.fwa2_backward_workspace_bytes(p)
+        assert 0 <= need < (1 << 62) or need == (1 << 64) - 1        # a size, or "no device can hold this"
+        seen.add(st)
+    assert seen == {_abi.OK, _abi.ERR_INVALID_ARGUMENT, _abi.ERR_UNSUPPORTED}
+
+
 def test_workspace_size_is_reported(lib):
     p = _good_problem(n=256, bw=4096, heads=3, backward=True)
     p.bias = _abi.Tensor3(0x10000, 65536, 256)
