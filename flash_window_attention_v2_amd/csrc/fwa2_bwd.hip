@@ -214,7 +214,7 @@ __device__ __forceinline__ void unit_blocks(BwdLds<DT, NQB>& L, WaveRegs<DT, NQB
 // BIG: windows of more than 256 tokens.  The N x N score matrix is cut into 256 x 256 (or 192 x 192) super-tiles;
 // a workgroup then belongs to one (head, query chunk, key chunk), reads only those rows, keeps that
 // tile of dbias in registers and writes its share of dk / dv (already taken back through the
-// normalisation, which is linear) as fp32 partials that dkv_reduce_kernel sums over the query chunks.
+// normalisation, which is linear) as fp32 partials that are summed over the query chunks by workgroups of the dq launch (dkv_reduce_rows).
 // MAPPED: rows are addressed through the window map (cyclic shift + window partition done here).  BIG decides that
 // at run time (p.map.nw > 0): its row fetches are a small part of a super-tile's work.
 template <int DT, bool HAS_BIAS, int MASK_DT, int NQB, int KT, int MODE, bool BIG, bool MAPPED = false>
@@ -650,39 +650,6 @@ __global__ void __launch_bounds__(256) reduce_kernel(const BwdParams p, int npk,
     }
 }
 
-// dk, dv = sum over the query chunks of the fp32 partials, cast to the input dtype.
-template <int DT>
-__global__ void __launch_bounds__(256) dkv_reduce_kernel(const BwdParams p) {
-    typedef typename Elem<DT>::E E;
-    typedef typename Elem<DT>::V8 V8;
-    const int64_t rows = (int64_t)p.bw * p.heads * p.n;
-    const int64_t i = (int64_t)blockIdx.x * 64 + (threadIdx.x >> 2);     // (b, h, key) row, 4 threads of 8 columns each
-    if (i >= rows) return;
-    const int key = (int)(i % p.n);
-    const int64_t bh = i / p.n;
-    const int h = (int)(bh % p.heads);
-    const int64_t b = bh / p.heads;
-    const int c8 = (threadIdx.x & 3) * 8;
-    float sk[8], sv[8];
-#pragma unroll
-    for (int j = 0; j < 8; j++) { sk[j] = 0.f; sv[j] = 0.f; }
-    for (int qs = 0; qs < p.n_chunks; qs++) {
-        const int64_t row = (((int64_t)qs * p.bw + b) * p.heads + h) * p.npk_tot + key;
-#pragma unroll
-        for (int v = 0; v < 2; v++) {
-            const f32x4 a = *reinterpret_cast<const f32x4*>(p.part_dk + row * 32 + c8 + 4 * v);
-            const f32x4 c = *reinterpret_cast<const f32x4*>(p.part_dv + row * 32 + c8 + 4 * v);
-#pragma unroll
-            for (int j = 0; j < 4; j++) { sk[4 * v + j] += a[j]; sv[4 * v + j] += c[j]; }
-        }
-    }
-    V8 ok, ov;
-#pragma unroll
-    for (int j = 0; j < 8; j++) { ok[j] = (E)sk[j]; ov[j] = (E)sv[j]; }
-    st8<V8>(reinterpret_cast<E*>(const_cast<void*>(p.dk.ptr)) + row_off_any(p.dk, p.map, (int)b, h, key) + c8, ok);
-    st8<V8>(reinterpret_cast<E*>(const_cast<void*>(p.dv.ptr)) + row_off_any(p.dv, p.map, (int)b, h, key) + c8, ov);
-}
-
 // ---- host side -----------------------------------------------------------------
 static size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
@@ -932,12 +899,7 @@ static hipError_t launch_bwd_dt(BwdParams p, bool has_bias, int mask_dt, hipStre
     if (e != hipSuccess) return e;
     p.groups = gr_out[0];
     p.db_parts = gr_out[1];
-    if (pl.n_chunks > 1) {
-        const int64_t rows = (int64_t)p.bw * p.heads * p.n;
-        hipLaunchKernelGGL(dkv_reduce_kernel<DT>, dim3((unsigned)((rows + 63) / 64)), dim3(256), 0, st, p);
-        e = hipGetLastError();
-        if (e != hipSuccess) return e;
-    }
+    // (windows of more than 256 tokens: the fp32 dk / dv partials are summed inside the dq launch that follows)
     if (backward_dq_resident_supported(p.n)) {
         int parts = 0;
         e = launch_backward_dq_resident(p, DT, has_bias, mask_dt, st, pl.dq_max_groups, &parts);

@@ -50,6 +50,18 @@ __global__ void __launch_bounds__(512) bwd_dq_kernel(const BwdParams p) {
     const int blk1 = (lane >> 4) & 1;
 
     int idx = blockIdx.x;
+    if (p.dkv_blocks > 0) {
+        // Some workgroups of this launch sum the fp32 dk / dv partials of the key-side kernel instead (bound by HBM,
+        // while the dq work is bound by compute).  They are spread evenly among the others: with D dq workgroups out
+        // of T, workgroup i does dq work iff floor((i + 1) D / T) > floor(i D / T), as dq workgroup floor(i D / T).
+        const int64_t total = gridDim.x, dq_blocks = total - p.dkv_blocks;
+        const int64_t before = (int64_t)idx * dq_blocks / total, upto = ((int64_t)idx + 1) * dq_blocks / total;
+        if (upto == before) {
+            dkv_reduce_rows<DT>(p, idx - before, (int)blockDim.x, (int)threadIdx.x);
+            return;
+        }
+        idx = (int)before;
+    }
     const int qc = idx % p.dq_chunks;
     idx /= p.dq_chunks;
     const int h = idx % p.heads;
@@ -286,10 +298,17 @@ void dq_geometry(int n, int* waves, int* chunks) {
     *chunks = (q_tiles + *waves - 1) / *waves;
 }
 
-hipError_t launch_backward_dq(const BwdParams& p, int dtype, bool has_bias, int mask_dt, hipStream_t st) {
+hipError_t launch_backward_dq(const BwdParams& p_in, int dtype, bool has_bias, int mask_dt, hipStream_t st) {
+    BwdParams p = p_in;
     const int chunk_rows = ((p.n < kKeyChunk ? p.n : kKeyChunk) + 63) & ~63;
     const size_t smem = (size_t)2 * chunk_rows * kLdsStride * 2 + 8 * sizeof(float);
-    dim3 grid((unsigned)((int64_t)p.bw * p.heads * p.dq_chunks)), block(64 * p.dq_waves);
+    const dim3 block(64 * p.dq_waves);
+    const int64_t dq_blocks = (int64_t)p.bw * p.heads * p.dq_chunks;
+    // the fp32 dk / dv partials of the super-tiled key-side kernel are summed by extra workgroups of this launch
+    const int64_t rows_per_block = block.x / 4, rows = (int64_t)p.bw * p.heads * p.n;
+    p.dkv_blocks = p.n_chunks > 1 ? (int)((rows + rows_per_block - 1) / rows_per_block) : 0;
+    if (dq_blocks + p.dkv_blocks > 0x7fffffffLL) return hipErrorInvalidValue;
+    dim3 grid((unsigned)(dq_blocks + p.dkv_blocks));
     if (dtype == FWA2_BF16) return launch_dt<FWA2_BF16>(p, has_bias, mask_dt, grid, block, smem, st);
     return launch_dt<FWA2_F16>(p, has_bias, mask_dt, grid, block, smem, st);
 }

@@ -476,6 +476,7 @@ struct BwdParams {
     float* part_dv;
     int dq_waves;        // wavefronts per workgroup of the dq kernel
     int dq_chunks;       // dq workgroups per (bw, head)
+    int dkv_blocks;      // windows of more than 256 tokens: workgroups of the dq launch that sum the dk / dv partials instead
     bool side_vec;       // rows of bias and mask (query-major) may be read with 16-byte loads, n % 8 == 0
     bool side_vec_rows;  // ... or n % 8 != 0 but every row is at least n rounded up to 8 entries long (resident kernels)
     const void* bias_t;  // [H, NP, NQ] input dtype: bias transposed to key-major, zero padded
@@ -483,5 +484,39 @@ struct BwdParams {
     const float* tab;    // table mode of the key-side kernel: (bias + mask) * log2e in accumulator order, slot h for
                          // head h alone and slot heads + w * heads + h for window w with a live mask
 };
+
+// dk, dv = sum over the query chunks of the fp32 partials (windows of more than 256 tokens), cast to the input
+// dtype.  Four threads per (b, h, key) row, 8 columns each; `block` counts workgroups of `threads` threads.
+template <int DT>
+__device__ __forceinline__ void dkv_reduce_rows(const BwdParams& p, int64_t block, int threads, int tid) {
+    typedef typename Elem<DT>::E E;
+    typedef typename Elem<DT>::V8 V8;
+    const int64_t rows = (int64_t)p.bw * p.heads * p.n;
+    const int64_t i = block * (threads >> 2) + (tid >> 2);
+    if (i >= rows) return;
+    const int key = (int)(i % p.n);
+    const int64_t bh = i / p.n;
+    const int h = (int)(bh % p.heads);
+    const int64_t b = bh / p.heads;
+    const int c8 = (tid & 3) * 8;
+    float sk[8], sv[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) { sk[j] = 0.f; sv[j] = 0.f; }
+    for (int qs = 0; qs < p.n_chunks; qs++) {
+        const int64_t row = (((int64_t)qs * p.bw + b) * p.heads + h) * p.npk_tot + key;
+#pragma unroll
+        for (int v = 0; v < 2; v++) {
+            const f32x4 a = *reinterpret_cast<const f32x4*>(p.part_dk + row * 32 + c8 + 4 * v);
+            const f32x4 c = *reinterpret_cast<const f32x4*>(p.part_dv + row * 32 + c8 + 4 * v);
+#pragma unroll
+            for (int j = 0; j < 4; j++) { sk[4 * v + j] += a[j]; sv[4 * v + j] += c[j]; }
+        }
+    }
+    V8 ok, ov;
+#pragma unroll
+    for (int j = 0; j < 8; j++) { ok[j] = (E)sk[j]; ov[j] = (E)sv[j]; }
+    st8<V8>(reinterpret_cast<E*>(const_cast<void*>(p.dk.ptr)) + row_off_any(p.dk, p.map, (int)b, h, key) + c8, ok);
+    st8<V8>(reinterpret_cast<E*>(const_cast<void*>(p.dv.ptr)) + row_off_any(p.dv, p.map, (int)b, h, key) + c8, ov);
+}
 
 }  // namespace fwa2
