@@ -595,12 +595,15 @@ static hipError_t launch_key_dt(const BwdParams& p, bool has_bias, int mask_dt, 
         const dim3 gr(key256::R * key256::R / 4 / 256, slots);
         float* tab = const_cast<float*>(p.tab);
         const E* bias = reinterpret_cast<const E*>(p.bias);
+        // The kernel lists the flags of up to kLive windows; with more it treats every window as live and reads
+        // every window's table, so every table has to be built then, whatever the flags say.
+        const uint8_t* live = p.n_windows <= key256::kLive ? p.mask_live : nullptr;
         if (mask_dt == FWA2_F32)
             hipLaunchKernelGGL((build_table_kernel<E, float>), gr, dim3(256), 0, st, bias, p.bias_sh, p.bias_sn,
-                               reinterpret_cast<const float*>(p.mask), p.mask_sw, p.mask_sn, p.mask_live, p.n, p.heads, tab);
+                               reinterpret_cast<const float*>(p.mask), p.mask_sw, p.mask_sn, live, p.n, p.heads, tab);
         else
             hipLaunchKernelGGL((build_table_kernel<E, E>), gr, dim3(256), 0, st, bias, p.bias_sh, p.bias_sn,
-                               reinterpret_cast<const E*>(p.mask), p.mask_sw, p.mask_sn, p.mask_live, p.n, p.heads, tab);
+                               reinterpret_cast<const E*>(p.mask), p.mask_sw, p.mask_sn, live, p.n, p.heads, tab);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }

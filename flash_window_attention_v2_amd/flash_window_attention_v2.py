@@ -24,15 +24,23 @@ def _scale_argument(logit_scale, device):
     return torch.empty((), device=device), "scalar"
 
 
-def _packed_forward(q, k, v, units, logit_scale, bias, mask, scale_type, window_map=None):
+def _packed_forward(q, k, v, units, logit_scale, bias, mask, scale_type, window_map=None, mask_flags=None):
     """Forward of the two packed Functions: q, k, v are [B, H, L, d] views of one qkv buffer, `units` the
     (number of windows, tokens per window) the library sees.  Returns out [B, L, H, d], lse and the mask's
-    per-window flags (kept for backward)."""
+    per-window flags (kept for backward).  `mask_flags`: flags the caller already holds for this mask (the
+    result of `mask_window_flags`), for masks that cannot carry their own cache."""
     b, heads, length, d = q.shape
     bw, n = units
     lse = torch.empty((bw, heads, (n + 63) // 64 * 64), device=q.device, dtype=torch.float32)
     out = torch.empty((b, length, heads, d), device=q.device, dtype=q.dtype)
-    mask_live = mask_window_flags(mask) if mask is not None else None
+    if mask is None:
+        mask_live = None
+    elif mask_flags is not None:
+        assert (mask_flags.dtype == torch.uint8 and mask_flags.device == mask.device
+                and mask_flags.shape == (mask.shape[0],)), "mask_flags must be what mask_window_flags(mask) returns"
+        mask_live = mask_flags
+    else:
+        mask_live = mask_window_flags(mask)
     p = _describe(q, k, v, out.transpose(1, 2), lse, logit_scale, bias, mask, mask_live, scale_type, window_map)
     with _on_device(q.device) as stream:
         p.stream = stream
@@ -100,7 +108,7 @@ class FlashWindowAttentionV2QKVPacked(torch.autograd.Function):
     take the same strided views but return separate tensors."""
 
     @staticmethod
-    def forward(ctx, qkv, logit_scale=None, bias=None, mask=None):
+    def forward(ctx, qkv, logit_scale=None, bias=None, mask=None, mask_flags=None):
         assert qkv.dim() == 5 and qkv.shape[2] == 3, "qkv must be [BW, N, 3, H, d]"
         if not (_rows_16b_aligned(qkv) and qkv.is_contiguous()):
             qkv = qkv.contiguous()
@@ -113,7 +121,7 @@ class FlashWindowAttentionV2QKVPacked(torch.autograd.Function):
             mask = mask.contiguous()
 
         bw, heads, n, d = q.shape
-        out, lse, mask_live = _packed_forward(q, k, v, (bw, n), logit_scale, bias, mask, scale_type)
+        out, lse, mask_live = _packed_forward(q, k, v, (bw, n), logit_scale, bias, mask, scale_type, mask_flags=mask_flags)
 
         ctx.save_for_backward(qkv, out, lse, logit_scale, bias, mask)
         ctx.scale_type = scale_type
@@ -129,7 +137,7 @@ class FlashWindowAttentionV2QKVPacked(torch.autograd.Function):
         if not _rows_16b_aligned(do):
             do = do.contiguous()
         dqkv, dscale, db = _packed_backward(qkv, q, k, v, out, lse, logit_scale, bias, mask, ctx.mask_live, scale_type, do)
-        return dqkv, dscale, db, None
+        return dqkv, dscale, db, None, None
 
 
 MAPPED_MAX_N = 1024     # largest window the library addresses through a window map
@@ -146,7 +154,7 @@ class FlashWindowAttentionV2Grid(torch.autograd.Function):
     Has no counterpart in the reference."""
 
     @staticmethod
-    def forward(ctx, qkv, grid, window, shift, logit_scale=None, bias=None, mask=None):
+    def forward(ctx, qkv, grid, window, shift, logit_scale=None, bias=None, mask=None, mask_flags=None):
         (gh, gw), (wh, ww), (sh, sw) = grid, window, shift
         assert qkv.dim() == 5 and qkv.shape[2] == 3 and qkv.shape[1] == gh * gw, "qkv must be [B, gh * gw, 3, H, d]"
         assert gh % wh == 0 and gw % ww == 0, "the grid must be a whole number of windows"
@@ -172,7 +180,8 @@ class FlashWindowAttentionV2Grid(torch.autograd.Function):
                 mask = mask.contiguous()
 
         window_map = ((gh, gw), (wh, ww), (sh % gh, sw % gw))
-        out, lse, mask_live = _packed_forward(q, k, v, (b * nw, n), logit_scale, bias, mask, scale_type, window_map)
+        out, lse, mask_live = _packed_forward(q, k, v, (b * nw, n), logit_scale, bias, mask, scale_type, window_map,
+                                              mask_flags=mask_flags)
 
         ctx.save_for_backward(qkv, out, lse, logit_scale, bias, mask)
         ctx.scale_type = scale_type
@@ -190,7 +199,7 @@ class FlashWindowAttentionV2Grid(torch.autograd.Function):
             do = do.contiguous()
         dqkv, dscale, db = _packed_backward(qkv, q, k, v, out, lse, logit_scale, bias, mask, ctx.mask_live, scale_type, do,
                                             ctx.window_map)
-        return dqkv, None, None, None, dscale, db, None
+        return dqkv, None, None, None, dscale, db, None, None
 
 
 class CpbBias(torch.autograd.Function):

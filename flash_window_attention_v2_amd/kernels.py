@@ -88,7 +88,9 @@ def mask_window_flags(mask):
     never cached and scan on every call: a mask created under torch.inference_mode, which tracks no
     modifications, and a first scan made while a graph is being captured, whose flags live in the graph's
     own memory pool and must not be handed to eager calls (scan once eagerly before capturing to avoid the
-    extra node)."""
+    extra node).  A caller that owns such a mask and never edits it (the Swin block and its `attn_mask` buffer)
+    scans it once itself and hands the flags to the packed operators (`mask_flags=`).
+    The region records only serve windows of up to 256 tokens; longer windows get the plain scan."""
     version = tensor_version(mask)
     key = (version, mask.data_ptr(), mask.device)
     cached = getattr(mask, "_fwa2_live", None)
@@ -96,12 +98,18 @@ def mask_window_flags(mask):
         return cached[1]
     lib = _abi.load()
     live = torch.empty(mask.shape[0], dtype=torch.uint8, device=mask.device)
-    regions = torch.empty(mask.shape[0] * _abi.MASK_REGION_BYTES, dtype=torch.uint8, device=mask.device)
-    with _on_device(mask.device) as stream:
-        st = lib.fwa2_mask_scan_regions(mask.data_ptr(), _DTYPES[mask.dtype], mask.shape[0], mask.shape[1],
-                                        mask.stride(0), mask.stride(1), live.data_ptr(), regions.data_ptr(), stream)
-    _abi.check(st, "fwa2_mask_scan_regions")
-    live._fwa2_regions = regions
+    if mask.shape[1] <= 256:
+        regions = torch.empty(mask.shape[0] * _abi.MASK_REGION_BYTES, dtype=torch.uint8, device=mask.device)
+        with _on_device(mask.device) as stream:
+            st = lib.fwa2_mask_scan_regions(mask.data_ptr(), _DTYPES[mask.dtype], mask.shape[0], mask.shape[1],
+                                            mask.stride(0), mask.stride(1), live.data_ptr(), regions.data_ptr(), stream)
+        _abi.check(st, "fwa2_mask_scan_regions")
+        live._fwa2_regions = regions
+    else:
+        with _on_device(mask.device) as stream:
+            st = lib.fwa2_mask_scan(mask.data_ptr(), _DTYPES[mask.dtype], mask.shape[0], mask.shape[1],
+                                    mask.stride(0), mask.stride(1), live.data_ptr(), stream)
+        _abi.check(st, "fwa2_mask_scan")
     if version is not None and not torch.cuda.is_current_stream_capturing():
         try:
             mask._fwa2_live = (key, live)
@@ -135,6 +143,9 @@ def _describe(q, k, v, o, lse, logit_scale, bias, mask, mask_live, scale_type, w
     bw, heads, n, d = q.shape
     p = _abi.new_problem()
     p.scale_head_dim = scale_dim
+    # whatever the description points at stays alive with it: the flags and region records may be temporaries
+    # (an uncached scan), and a later allocation must not land on their memory before the launch has been queued
+    p._keep = (mask_live, getattr(mask_live, "_fwa2_regions", None))
     if window_map is not None:
         # q, k, v, o are token grids [B, H, gh * gw, d]; the library partitions them into windows
         (gh, gw), (wh, ww), (sh, sw) = window_map
@@ -155,7 +166,7 @@ def _describe(q, k, v, o, lse, logit_scale, bias, mask, mask_live, scale_type, w
         # them on 16-byte loads; the kernels never use the entries beyond n.  The copies live as long as the
         # problem description (the launch that follows is ordered behind them on the same stream).
         bias, mask = _rows_of_8(bias, cache=False), _rows_of_8(mask, cache=True)
-        p._keep = (bias, mask)
+        p._keep = p._keep + (bias, mask)
     if bias is not None:
         p.bias.ptr, p.bias.stride_a, p.bias.stride_n = bias.data_ptr(), bias.stride(0), bias.stride(1)
     if mask is not None:

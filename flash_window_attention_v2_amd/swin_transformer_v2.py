@@ -20,6 +20,7 @@ from torch.utils.checkpoint import checkpoint
 from .win_attention_func import (flash_win_attn_v2_func, flash_win_attn_v2_grid_func, flash_win_attn_v2_qkvpacked_func,
                                  win_attention_torch)
 from .flash_window_attention_v2 import CpbBias, MAPPED_MAX_N, tensor_version
+from .kernels import mask_window_flags
 
 
 def _pair(x):
@@ -198,8 +199,9 @@ class WindowAttention(nn.Module):
         bias = per_offset[self.relative_position_index.view(-1)].view(n, n, self.num_heads)
         return 16 * torch.sigmoid(bias.permute(2, 0, 1).contiguous())
 
-    def forward(self, x, mask=None):
-        """x: [B * nW, N, C]; mask: [nW, N, N] of 0 / -100 or None."""
+    def forward(self, x, mask=None, mask_flags=None):
+        """x: [B * nW, N, C]; mask: [nW, N, N] of 0 / -100 or None.  `mask_flags`: the per-window flags of `mask`
+        when the caller holds them already (`kernels.mask_window_flags`); used by the packed path only."""
         b_, n, c = x.shape
         bias = None
         if self.q_bias is not None:
@@ -212,7 +214,7 @@ class WindowAttention(nn.Module):
         if self.is_flash and self.packed_qkv:
             # the kernels read q, k, v out of the GEMM output and write [B_, N, H, d]: no copies either
             # side, and one packed gradient instead of three that autograd would have to re-pack
-            out = flash_win_attn_v2_qkvpacked_func(qkv, scale, rel_bias, mask).reshape(b_, n, c)
+            out = flash_win_attn_v2_qkvpacked_func(qkv, scale, rel_bias, mask, mask_flags).reshape(b_, n, c)
         else:
             q, k, v = qkv.permute(2, 0, 3, 1, 4).unbind(0)      # strided views, unit inner stride
             if self.is_flash:
@@ -249,7 +251,7 @@ class WindowAttention(nn.Module):
             return False
         return self.window_size[0] * self.window_size[1] <= MAPPED_MAX_N and self.window_size[1] <= 64
 
-    def forward_grid(self, x, grid, shift, mask=None):
+    def forward_grid(self, x, grid, shift, mask=None, mask_flags=None):
         """The attention of every (shifted) window of the token grid x [B, gh * gw, C], result in the same
         layout: what the reference's block computes with roll + window_partition around `forward` and
         window_reverse + roll after it (swin_transformer_v2.py:419-441), with the permutation done by the
@@ -261,7 +263,7 @@ class WindowAttention(nn.Module):
         qkv = F.linear(x, self.qkv.weight, bias).reshape(b, length, 3, self.num_heads, -1)
         rel_bias = self.relative_position_bias()
         scale, rel_bias = self._operator_dtype(qkv, self.logit_scale, rel_bias)
-        out = flash_win_attn_v2_grid_func(qkv, grid, self.window_size, shift, scale, rel_bias, mask)
+        out = flash_win_attn_v2_grid_func(qkv, grid, self.window_size, shift, scale, rel_bias, mask, mask_flags)
         return self.proj_drop(self.proj(out.reshape(b, length, c)))
 
     def extra_repr(self):
@@ -300,6 +302,29 @@ class SwinTransformerBlock(nn.Module):
         if self.shift_size > 0:
             mask = shifted_window_attn_mask(input_resolution, self.window_size, self.shift_size)
         self.register_buffer("attn_mask", mask)
+        self._attn_mask_flags = None
+
+    def _apply(self, fn, *args, **kwargs):
+        # .to() / .cuda() / .half() replace the buffer: its flags are scanned again on the next call
+        self._attn_mask_flags = None
+        return super()._apply(fn, *args, **kwargs)
+
+    def mask_flags(self):
+        """Per-window flags of `attn_mask` for the fused operator, scanned once per buffer and kept on the block.
+        The block owns the buffer and never edits it, so the flags stay valid whatever mode the buffer was
+        created in: a model built under torch.inference_mode (benchmark/bench_model.py:14-19 of the reference)
+        has a mask without a modification counter, which `mask_window_flags` alone would rescan on every call."""
+        mask = self.attn_mask
+        if mask is None or not (self.is_flash and mask.is_cuda):
+            return None
+        key = (mask.data_ptr(), mask.device, mask.dtype, tuple(mask.shape), tensor_version(mask))
+        held = self._attn_mask_flags
+        if held is not None and held[0] == key:
+            return held[1]
+        flags = mask_window_flags(mask)
+        if not torch.cuda.is_current_stream_capturing():
+            self._attn_mask_flags = (key, flags)
+        return flags
 
     def forward(self, x):
         h, w = self.input_resolution
@@ -308,14 +333,15 @@ class SwinTransformerBlock(nn.Module):
         shortcut = x
         if self.attn.grid_ready(x):
             # roll, window_partition, window_reverse and the roll back happen inside the kernels
-            x = self.attn.forward_grid(x, (h, w), (self.shift_size, self.shift_size), mask=self.attn_mask)
+            x = self.attn.forward_grid(x, (h, w), (self.shift_size, self.shift_size), mask=self.attn_mask,
+                                       mask_flags=self.mask_flags())
             x = shortcut + self.drop_path(self.norm1(x))
             return x + self.drop_path(self.norm2(self.mlp(x)))
         x = x.view(b, h, w, c)
         if self.shift_size > 0:
             x = torch.roll(x, shifts=(-self.shift_size, -self.shift_size), dims=(1, 2))
         windows = window_partition(x, self.window_size).view(-1, self.window_size * self.window_size, c)
-        windows = self.attn(windows, mask=self.attn_mask)
+        windows = self.attn(windows, mask=self.attn_mask, mask_flags=self.mask_flags())
         x = window_reverse(windows.view(-1, self.window_size, self.window_size, c), self.window_size, h, w)
         if self.shift_size > 0:
             x = torch.roll(x, shifts=(self.shift_size, self.shift_size), dims=(1, 2))

@@ -73,7 +73,10 @@ typedef struct fwa2_tensor4 {
  * row past its N-th are never used.  The kernels read bias and mask with 16-byte loads when ptr is 16-byte
  * aligned, both strides are multiples of 8 elements and stride_n >= N rounded up to a multiple of 8; a caller
  * whose N is not a multiple of 8 gets that path by padding the rows (with anything), and the element-wise path
- * otherwise. */
+ * otherwise.  On the 16-byte path EVERY row, the last row of the last head or window included, is read up to
+ * N rounded up to a multiple of 8: the allocation behind ptr must cover (A - 1) * stride_a + (N - 1) * stride_n
+ * + roundup8(N) elements.  A view that ends exactly at its N-th element of the last row must either be padded
+ * or be described with a stride_n that is not a multiple of 8 (which selects the element-wise path). */
 typedef struct fwa2_tensor3 {
     void*   ptr;       /* NULL = absent */
     int64_t stride_a;
@@ -247,7 +250,11 @@ int fwa2_backward(const fwa2_problem* p);
  *     64-token windows at 4 096 per call; windows of 576 tokens and more need their fp32 dk / dv partials here
  *     too (0.7 GiB at 256 windows of 6 heads) and do not fit: use fwa2_backward there;
  *   - the device that is current at the call must be the one the tensors and the stream belong to; the address
- *     of that device's copy of the array is looked up on the first call per device;
+ *     of that device's copy of the array is looked up on the first call per device (hipGetSymbolAddress, which
+ *     may load the code object): make that first call OUTSIDE any stream capture, e.g. one warm-up call before
+ *     the capture starts; later calls on the same device only launch kernels;
+ *   - the array costs FWA2_STATIC_SCRATCH_BYTES of device memory on every GPU of every process that loads the
+ *     library, whether or not this entry point is ever called;
  *   - every call on a GPU shares that GPU's array: calls that may overlap on one GPU (different streams, or
  *     different threads without ordering) race on it.  Calls on one stream are ordered and safe.  Nothing in
  *     the array needs clearing between calls: every kernel writes what a later kernel of the same call reads.

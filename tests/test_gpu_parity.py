@@ -136,6 +136,20 @@ def test_more_windows_than_the_flag_cache_and_no_flags(monkeypatch):
     assert len(described) == 6 and all(ptr is None for ptr in described), described
 
 
+def test_more_windows_than_the_key_side_kernel_lists():
+    """Windows of 161 .. 256 tokens with more windows than the key-side backward lists in LDS (256) and one
+    head, so that the score tables still fit the table budget: every window then counts as live in that kernel
+    and the table of a window whose mask is all zero must have been built too (dk, dv, dbias read it)."""
+    n_w, n = 260, 192
+    inp = make_inputs(batch=1, n_windows=n_w, heads=1, n=n, dtype=torch.bfloat16, seed=31, with_mask=False)
+    g = torch.Generator().manual_seed(32)
+    mask = torch.where(torch.rand(n_w, n, n, generator=g) < 0.3, -100.0, 0.0)
+    mask[torch.arange(n_w) % 4 != 0] = 0.0          # three quarters of the windows: all-zero masks
+    mask[:, torch.arange(n), torch.arange(n)] = 0.0
+    inp["mask"] = mask.to(torch.bfloat16)
+    _run_and_check(inp, torch.bfloat16, tag="260 windows of 192 tokens")
+
+
 @pytest.mark.parametrize("n", [1, 7, 17, 31, 33, 47, 63, 65, 100, 129, 196, 200, 225, 255])
 def test_ragged_window_sizes(n):
     """Window sizes that are no multiple of 8, 16 or 32 (bias and mask rows padded to 8 entries above 64 tokens

@@ -259,6 +259,46 @@ def test_fused_position_bias_gpu(window, dtype):
 
 
 @pytest.mark.gpu
+def test_block_built_under_inference_mode_scans_its_mask_once_gpu(monkeypatch):
+    """A model built under torch.inference_mode (the reference's forward benchmark, benchmark/bench_model.py:14-19)
+    has an attn_mask without a modification counter, which the operator alone rescans on every call; the block
+    scans its own buffer once and hands the flags down.  The output is the one of a block built normally."""
+    from flash_window_attention_v2_amd import _abi
+    dev = torch.device("cuda")
+    torch.manual_seed(5)
+    plain = swin.SwinTransformerBlock(96, (32, 32), 3, window_size=8, shift_size=4, is_flash=True).to(dev).bfloat16()
+    x = torch.randn(2, 32 * 32, 96, device=dev).bfloat16()
+    with torch.no_grad():
+        want = plain(x)
+    lib = _abi.load()
+    calls = {"scan": 0}
+    for name in ("fwa2_mask_scan", "fwa2_mask_scan_regions"):
+        real = getattr(lib, name)
+
+        def counted(*args, _real=real):
+            calls["scan"] += 1
+            return _real(*args)
+
+        monkeypatch.setattr(lib, name, counted)
+    with torch.inference_mode():
+        blk = swin.SwinTransformerBlock(96, (32, 32), 3, window_size=8, shift_size=4, is_flash=True)
+        blk.load_state_dict(plain.state_dict())
+        blk = blk.to(dev).bfloat16()
+        assert blk.attn_mask.is_inference()
+        xi = x.clone()
+        outs = [blk(xi) for _ in range(3)]
+    assert calls["scan"] == 1, calls
+    for o in outs:
+        assert torch.equal(o, want)
+    # a cast replaces the buffer: one more scan, not one per call
+    with torch.inference_mode():
+        blk = blk.half().bfloat16()
+        outs = [blk(xi) for _ in range(2)]
+    assert calls["scan"] == 2, calls
+    assert torch.equal(outs[1], want)
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("window,shift,res", [(8, 0, 32), (8, 4, 32), (16, 8, 32), (24, 12, 48)])
 def test_block_window_map_matches_partition_gpu(window, shift, res):
     """SwinTransformerBlock with the roll / partition / reverse done by the kernels' addressing against the
@@ -341,7 +381,7 @@ def test_model_flash_matches_classic_gpu():
 
 @pytest.mark.gpu
 def test_model_of_the_end_to_end_benchmark_gpu():
-    """The model the reference times end to end (benchmark/bench_swin.py:110-131: 256 x 256 images,
+    """The model the reference times end to end (benchmark/config.py:40-47 + bench_model.py:23-38: 256 x 256 images,
     patch 4, depths 2/2/6/2, heads 3/6/12/24, windows of 16 x 16 tokens, which the last stage's 8 x 8 grid
     cuts down to 8 x 8) at a reduced batch: every stage's kernels, both window sizes, shifted and
     unshifted blocks, patch merging and the head in one step."""
