@@ -292,7 +292,7 @@ def test_block_built_under_inference_mode_scans_its_mask_once_gpu(monkeypatch):
         assert torch.equal(o, want)
     # a cast replaces the buffer: one more scan, not one per call
     with torch.inference_mode():
-        blk = blk.half().bfloat16()
+        blk = blk.float().bfloat16()        # exact for the bf16 weights; the mask buffer is a new tensor
         outs = [blk(xi) for _ in range(2)]
     assert calls["scan"] == 2, calls
     assert torch.equal(outs[1], want)
@@ -392,6 +392,8 @@ def test_model_of_the_end_to_end_benchmark_gpu():
     shifts = [blk.shift_size for layer in model.layers for blk in layer.blocks]
     assert windows[:10] == [(16, 16)] * 10 and windows[10:] == [(8, 8)] * 2
     assert shifts == [0, 8, 0, 8] + [0] * 8          # the 16 x 16 and 8 x 8 grids are one window: no shift
+    print(f"C5 batch 4: loss ref {losses['ref']:.6f} fused {losses['fused']:.6f} eager {losses['eager']:.6f}; "
+          f"worst parameter-gradient error fused {fused:.4e} eager {eager:.4e}")
     assert abs(losses["fused"] - losses["ref"]) < 3e-2
     assert abs(losses["fused"] - losses["ref"]) <= max(2.0 * abs(losses["eager"] - losses["ref"]), 1e-2)
     assert fused < max(2.0 * eager, 5e-2), (fused, eager)
