@@ -673,6 +673,18 @@ constexpr size_t kTableBudget = (size_t)96 << 20;
 
 hipError_t launch_backward_key(const BwdParams& p, int dtype, bool has_bias, int mask_dt, hipStream_t st, int max_groups,
                                int* groups_out);
+hipError_t launch_backward_one(const BwdParams& p, int dtype, bool has_bias, int mask_dt, hipStream_t st, int max_groups,
+                               int* groups_out);
+#if FWA2_HALF != 2
+// FWA2_BWD_TWO_PASS=1 in the environment keeps windows of 161 .. 256 tokens on the key-side + query-side pair of
+// kernels instead of the one-pass kernel (read once per process; for comparing the two).
+bool backward_two_pass() {
+    static const bool two = [] { const char* e = getenv("FWA2_BWD_TWO_PASS"); return e && e[0] == '1'; }();
+    return two;
+}
+#else
+bool backward_two_pass();
+#endif
 
 struct BwdPlan {
     int waves, groups, npk, r, nqb_t, kt, dq_waves, dq_chunks, ds_parts, dq_max_groups;
@@ -885,6 +897,20 @@ static hipError_t launch_bwd_dt(BwdParams p, bool has_bias, int mask_dt, hipStre
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     int gr_out[2] = {pl.groups, pl.groups};
+    const bool one_pass = pl.key256 && !backward_two_pass();
+    if (one_pass) {
+        e = launch_backward_one(p, DT, has_bias, mask_dt, st, pl.groups, gr_out);
+        if (e != hipSuccess) return e;
+        p.groups = gr_out[0];
+        p.db_parts = gr_out[1];
+        p.ds_parts = gr_out[0];
+        if (has_bias || p.scale_kind == FWA2_SCALE_TENSOR) {
+            dim3 gr(has_bias ? pl.r / 32 : 1, has_bias ? pl.npk : 1, p.heads);
+            hipLaunchKernelGGL(reduce_kernel<DT>, gr, dim3(256), 0, st, p, pl.npk, pl.r, has_bias);
+            e = hipGetLastError();
+        }
+        return e;
+    }
     if (pl.key256) {
         e = launch_backward_key(p, DT, has_bias, mask_dt, st, pl.groups, gr_out);
     } else if (has_bias) {

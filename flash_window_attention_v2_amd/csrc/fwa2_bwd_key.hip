@@ -584,31 +584,37 @@ static hipError_t launch_key(BwdParams p, hipStream_t st, int max_groups, int* g
     return hipGetLastError();
 }
 
+// The score tables of a call: slot h for every head, slot heads + w * heads + h for every window whose mask is live.
 template <int DT>
-static hipError_t launch_key_dt(const BwdParams& p, bool has_bias, int mask_dt, hipStream_t st, int max_groups, int* groups_out) {
+static hipError_t build_tables(const BwdParams& p, bool has_bias, int mask_dt, hipStream_t st) {
     typedef typename Elem<DT>::E E;
     const bool masked = mask_dt >= 0;
     const bool has_tab = has_bias || masked || p.n < key256::R;
+    if (!has_tab) return hipSuccess;
+    const int slots = p.heads * (1 + (masked ? p.n_windows : 0));
+    const dim3 gr(key256::R * key256::R / 4 / 256, slots);
+    float* tab = const_cast<float*>(p.tab);
+    const E* bias = reinterpret_cast<const E*>(p.bias);
+    // The kernels list the flags of up to kLive windows; with more they treat every window as live and read
+    // every window's table, so every table has to be built then, whatever the flags say.
+    const uint8_t* live = p.n_windows <= key256::kLive ? p.mask_live : nullptr;
+    if (mask_dt == FWA2_F32)
+        hipLaunchKernelGGL((build_table_kernel<E, float>), gr, dim3(256), 0, st, bias, p.bias_sh, p.bias_sn,
+                           reinterpret_cast<const float*>(p.mask), p.mask_sw, p.mask_sn, live, p.n, p.heads, tab);
+    else
+        hipLaunchKernelGGL((build_table_kernel<E, E>), gr, dim3(256), 0, st, bias, p.bias_sh, p.bias_sn,
+                           reinterpret_cast<const E*>(p.mask), p.mask_sw, p.mask_sn, live, p.n, p.heads, tab);
+    return hipGetLastError();
+}
+
+template <int DT>
+static hipError_t launch_key_dt(const BwdParams& p, bool has_bias, int mask_dt, hipStream_t st, int max_groups, int* groups_out) {
+    const bool masked = mask_dt >= 0;
+    const bool has_tab = has_bias || masked || p.n < key256::R;
     const bool mapped = p.map.nw > 0;
-    if (has_tab) {
-        const int slots = p.heads * (1 + (masked ? p.n_windows : 0));
-        const dim3 gr(key256::R * key256::R / 4 / 256, slots);
-        float* tab = const_cast<float*>(p.tab);
-        const E* bias = reinterpret_cast<const E*>(p.bias);
-        // The kernel lists the flags of up to kLive windows; with more it treats every window as live and reads
-        // every window's table, so every table has to be built then, whatever the flags say.
-        const uint8_t* live = p.n_windows <= key256::kLive ? p.mask_live : nullptr;
-        if (mask_dt == FWA2_F32)
-            hipLaunchKernelGGL((build_table_kernel<E, float>), gr, dim3(256), 0, st, bias, p.bias_sh, p.bias_sn,
-                               reinterpret_cast<const float*>(p.mask), p.mask_sw, p.mask_sn, live, p.n, p.heads, tab);
-        else
-            hipLaunchKernelGGL((build_table_kernel<E, E>), gr, dim3(256), 0, st, bias, p.bias_sh, p.bias_sn,
-                               reinterpret_cast<const E*>(p.mask), p.mask_sw, p.mask_sn, live, p.n, p.heads, tab);
-        hipError_t e = hipGetLastError();
-        if (e != hipSuccess) return e;
-    }
+    hipError_t e = build_tables<DT>(p, has_bias, mask_dt, st);
+    if (e != hipSuccess) return e;
     if (p.ev_start) (void)hipEventRecord(p.ev_start, st);
-    hipError_t e;
 #define FWA2_KEY_CASE(B, T, M)                                                                                       \
     (mapped ? launch_key<DT, B, T, M, true>(p, st, max_groups, groups_out) : launch_key<DT, B, T, M, false>(p, st, max_groups, groups_out))
     if (has_bias) e = masked ? FWA2_KEY_CASE(true, true, true) : FWA2_KEY_CASE(true, true, false);
@@ -628,6 +634,11 @@ hipError_t launch_backward_key_f16(const BwdParams& p, bool has_bias, int mask_d
 #if FWA2_HALF == 1
 hipError_t launch_backward_key_f16(const BwdParams& p, bool has_bias, int mask_dt, hipStream_t st, int max_groups, int* groups_out);
 #endif
+// The tables alone, for the one-pass kernel (fwa2_bwd_one.hip), which reads them in the same order.
+hipError_t launch_key_tables(const BwdParams& p, int dtype, bool has_bias, int mask_dt, hipStream_t st) {
+    return dtype == FWA2_BF16 ? build_tables<FWA2_BF16>(p, has_bias, mask_dt, st) : build_tables<FWA2_F16>(p, has_bias, mask_dt, st);
+}
+
 // dk, dv, delta and the dbias partial tiles of a call with 161 .. 256 tokens per window; p.tab points at room for
 // heads * (1 + windows) tables of 256 x 256 floats.  groups_out: workgroups per head, partial tiles per head.
 hipError_t launch_backward_key(const BwdParams& p, int dtype, bool has_bias, int mask_dt, hipStream_t st, int max_groups,
