@@ -48,6 +48,7 @@ constexpr int NT = 64 * WAVES;
 constexpr int kLdsQb = 2;     // query blocks whose dbias accumulators live in LDS (see bwd_key_kernel)
 __host__ __device__ constexpr bool db_in_lds(int qb) { return qb >= NQB - kLdsQb; }
 constexpr int kLive = 256;    // windows whose mask flags are listed in LDS (more: every window counts as live)
+constexpr int kLandE = 3 * 32 * 32 + 512;   // elements of a landing slot: three tensors' rows and 1 KB for lse
 constexpr int kPartRow = 36;  // floats per query row of a dq partial tile (32 + 4: rows 144 bytes apart)
 
 // sum of squares / dot product of 4 elements, two at a time on the dot unit
@@ -140,6 +141,24 @@ __device__ __forceinline__ void vm_store8_if_below(E* dst, V4 v, int idx, int li
                  : "memory", "vcc");
 }
 
+// 16 bytes per lane from base + voff (base: wavefront-uniform).  The result registers are only valid after a wait
+// that the caller places (tables_arrived below): the compiler neither sees the load nor waits for it.
+__device__ __forceinline__ f32x4 vm_load16(const float* base, uint32_t voff) {
+    f32x4 r;
+    asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(r) : "v"(voff), "s"(base) : "memory");
+    return r;
+}
+// At most `n` loads outstanding from here on; a and b (loaded earlier) may be used behind this point.
+template <int N_OUT>
+__device__ __forceinline__ void tables_arrived(f32x4& a, f32x4& b) {
+    asm volatile("s_waitcnt vmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N_OUT) : "memory");
+}
+// 8 bytes per lane at base + voff (base: wavefront-uniform)
+template <class V4>
+__device__ __forceinline__ void vm_store8(void* base, uint32_t voff, V4 v) {
+    asm volatile("global_store_dwordx2 %0, %1, %2 nt" ::"v"(voff), "v"(v), "s"(base) : "memory");
+}
+
 // 1 / max(|x|, eps) from the sum of squares
 __device__ __forceinline__ float inv_norm_fast(float sumsq) {
     return __builtin_amdgcn_rsqf(fmaxf(sumsq, kNormEps * kNormEps));
@@ -148,10 +167,14 @@ __device__ __forceinline__ float inv_norm_fast(float sumsq) {
 }  // namespace one256
 
 // HAS_BIAS: dbias is wanted.  HAS_TAB: a table of (bias + mask) * log2e exists (always when there is a bias, a mask
-// or padded keys).  MASKED: some units take the table of their (window, head) instead of the head's.
-template <int DT, bool HAS_BIAS, bool HAS_TAB, bool MASKED, bool MAPPED>
+// or padded keys).  MASKED: some units take the table of their (window, head) instead of the head's.  ROWS: how
+// rows are addressed -- 0 any window length without a window map, 1 through the window map, 2 windows of exactly
+// 256 tokens without a map (every block is whole: no clamping, no predicated stores, no branches in the copies).
+template <int DT, bool HAS_BIAS, bool HAS_TAB, bool MASKED, int ROWS>
 __global__ void __launch_bounds__(one256::NT) bwd_one_kernel(const BwdParams p) {
     using namespace one256;
+    constexpr bool MAPPED = ROWS == 1;
+    constexpr bool PLAIN = ROWS == 2;
     constexpr int SDT = kScoreDT;
     typedef typename Elem<DT>::E E;
     typedef typename Elem<DT>::V8 V8;
@@ -165,19 +188,18 @@ __global__ void __launch_bounds__(one256::NT) bwd_one_kernel(const BwdParams p) 
     const int N = p.n;
 
     // landing slots (block X & 1): 32 rows of q, dO, o as they are in memory, and their lse
-    __shared__ __attribute__((aligned(16))) E lds_raw[2][3][32 * 32];
-    __shared__ __attribute__((aligned(16))) float lds_rawLse[2][64];
+    // (per slot: q, dO, o rows, 2 KB each, then 1 KB for the lse values: what wavefront w copies lands 2 KB x w
+    // into the slot)
+    __shared__ __attribute__((aligned(16))) E lds_raw[2][kLandE];
     // tile slots (block X & 3)
     __shared__ __attribute__((aligned(16))) SE lds_Qs[4][32 * kRow];
     __shared__ __attribute__((aligned(16))) E lds_dOs[4][32 * kRow];
-    __shared__ __attribute__((aligned(16))) float lds_nlse2[4][32];
-    __shared__ __attribute__((aligned(16))) float lds_ndelta[4][32];
-    __shared__ __attribute__((aligned(16))) float lds_qinv[4][32];
+    // per tile slot: -delta, -lse * log2e, 1 / |q| of its 32 rows, and a row nobody reads
+    __shared__ __attribute__((aligned(16))) float lds_meta[4][4][32];
     // per wavefront: dZ of the running block, [key of the wavefront][query of the block] (also K_hat once per unit)
     __shared__ __attribute__((aligned(16))) SE lds_zst[WAVES][64 * kRow];
     // dQ_hat partials (block X & 1) of the four wavefronts, [query][d] fp32
     __shared__ __attribute__((aligned(16))) float lds_part[2][WAVES][32 * kPartRow];
-    __shared__ float lds_dummy[NT];
     __shared__ float lds_red[WAVES];
     __shared__ __attribute__((aligned(16))) float lds_db[HAS_BIAS ? kLdsQb * KT * 2 * NT * 4 : 4];
 
@@ -270,94 +292,148 @@ __global__ void __launch_bounds__(one256::NT) bwd_one_kernel(const BwdParams p) 
         const int slot = live ? p.heads + (b % p.n_windows) * p.heads + h : h;
         return p.tab + (int64_t)slot * (R * R) + ((wave * KT * NQB * 2) << 8);     // wavefront-uniform; the lane adds 4 * lane
     };
-    const int lane4 = 4 * lane;
+    const uint32_t lane16 = 16u * (uint32_t)lane;
 
+    // Wavefront-uniform start of unit b inside a tensor whose head offset is already part of `base`.
+    auto unit_start = [&](const char* base, int64_t sb, int b) -> const char* {
+        return base + (int64_t)(MAPPED ? b / p.map.nw : b) * sb * (int64_t)sizeof(E);
+    };
     // ---- rows of block qb of unit b, global memory -> landing slot.  Wavefront 0 moves the 32 rows of q (16 per
     // instruction), 1 those of dO, 2 those of o, 3 the lse values (twice, so that every wavefront has issued the
-    // same number of copies).  Rows beyond n re-read row n - 1 (the tile builder zeroes them). ----
-    auto dma_block = [&](int b, int qb, int slot) __attribute__((always_inline)) {
-        const int ln = lane_now();
-        if (wave < 3) {
-            const T4& t4 = wave == 0 ? p.q : wave == 1 ? p.d_o : p.o;
-            const E* unit = unit_ptr<MAPPED, E>(t4, p.map, b, h);
+    // same number of copies).  Rows beyond n re-read row n - 1 (the tile builder zeroes them).  What a wavefront
+    // copies never changes, so its tensor is picked once. ----
+    const T4& mine = wave == 0 ? p.q : wave == 1 ? p.d_o : p.o;
+    const char* const mine_base = reinterpret_cast<const char*>(mine.ptr) + (int64_t)h * mine.sh * (int64_t)sizeof(E);
+    const int64_t mine_sb = mine.sb, mine_sn = mine.sn;
+    const float* const lse_base = p.lse + h * p.lse_sh;
+    const int meta_lane = min(tid & 7, 3) * 32 + (tid >> 3);
+    // Whole blocks without a window map (PLAIN): a lane's byte offset into its source is a constant of the lane
+    // plus a scalar of the block, and wavefront 3 copies its 128 bytes of lse with the same 16-byte instruction
+    // (8 lanes' worth, repeated), so the copies are the same two instructions in every wavefront.
+    const uint32_t mine_lane = wave < 3 ? (uint32_t)(((lane >> 2) * (int)mine_sn + (lane & 3) * 8) * (int)sizeof(E)) : 16u * (uint32_t)(lane & 7);
+    const uint32_t mine_blk = wave < 3 ? (uint32_t)(32 * (int)mine_sn * (int)sizeof(E)) : 128u;      // one block further on
+    const uint32_t mine_half = wave < 3 ? mine_blk / 2 : 0u;                                          // its second 16 rows
+    const uint32_t land_wave = lds_addr(&lds_raw[0][0]) + 2048u * (uint32_t)wave;
+    const uint32_t land_half = wave < 3 ? 1024u : 0u;
+    // the wavefront's source inside unit b: its tensor's rows, or the unit's lse values
+    auto source_of = [&](int b) -> const char* {
+        return wave < 3 ? unit_start(mine_base, mine_sb, b) : reinterpret_cast<const char*>(lse_base + b * p.lse_sb);
+    };
+    auto dma_block = [&](const char* src, int b, int qb, int slot) __attribute__((always_inline)) {
+        if (PLAIN) {
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                uint32_t voff = mine_lane, blk = mine_blk, half = mine_half, dst = land_wave, dhalf = land_half;
+                // taken as opaque here: one add per copy instead of a register per block and slot kept across the loop
+                asm volatile("" : "+v"(voff), "+s"(blk), "+s"(half), "+s"(dst), "+s"(dhalf));
+                vm_dma16(src, voff + (uint32_t)qb * blk + (uint32_t)i * half, dst + (uint32_t)(slot * kLandE * (int)sizeof(E)) + (uint32_t)i * dhalf);
+            }
+        } else if (wave < 3) {
+            const int ln = lane_now();
             const int dc = (ln & 3) * 8;
 #pragma unroll
             for (int i = 0; i < 2; i++) {
                 const int r = min(32 * qb + 16 * i + (ln >> 2), N - 1);
-                const uint32_t voff = (uint32_t)(reinterpret_cast<const char*>(row_at(unit, unit_row<MAPPED>(p.map, b, r), t4.sn, dc)) -
-                                                 reinterpret_cast<const char*>(unit));
-                vm_dma16(unit, voff, lds_addr(&lds_raw[slot][wave][16 * i * 32]));
+                vm_dma16(src, row_byte_offset<E>(unit_row<MAPPED>(p.map, b, r), mine_sn, dc), lds_addr(&lds_raw[slot][wave * 1024 + 16 * i * 32]));
             }
         } else {
+            const int ln = lane_now();
             const int r = min(32 * qb + (ln & 31), N - 1);
-            const float* src = p.lse + b * p.lse_sb + h * p.lse_sh;
-            vm_dma4(src, 4u * (uint32_t)r, lds_addr(&lds_rawLse[slot][0]));
-            vm_dma4(src, 4u * (uint32_t)r, lds_addr(&lds_rawLse[slot][0]));
+            vm_dma4(src, 4u * (uint32_t)r, lds_addr(&lds_raw[slot][3 * 1024]));
+            vm_dma4(src, 4u * (uint32_t)r, lds_addr(&lds_raw[slot][3 * 1024]));
         }
     };
 
     // ---- landing slot -> tile slot: q_hat * s * log2e, dO, -delta, -lse * log2e, 1 / |q|.  Thread = 4 columns of one
-    // row (8 threads per row, 32 rows).  Straight-line code: of the eight lanes of a row, lane 0 writes -delta,
-    // lane 1 -lse * log2e, lane 2 1 / |q| and the rest a dummy word, through one store whose address and value are
-    // selected per lane. ----
-    auto normalise = [&](int qb, int lslot, int tslot) __attribute__((always_inline)) {
+    // row (8 threads per row, 32 rows; wavefront w has rows 8 w .. 8 w + 7).  Straight-line code: of the eight lanes
+    // of a row, lane 0 writes -delta, lane 1 -lse * log2e, lane 2 1 / |q| and the rest a word nobody reads, through one
+    // store whose address and value are selected per lane.  In two halves, so that the reads of all the side
+    // stages of an iteration can be issued before anything waits for one of them. ----
+    struct NormIn { V4 q4, do4, o4; float lse; };
+    auto normalise_load = [&](int lslot) __attribute__((always_inline)) -> NormIn {
         const int r = tid >> 3, c4 = (tid & 7) * 4;
-        V4 q4 = *reinterpret_cast<const V4*>(&lds_raw[lslot][0][r * 32 + c4]);
-        V4 do4 = *reinterpret_cast<const V4*>(&lds_raw[lslot][1][r * 32 + c4]);
-        const V4 o4 = *reinterpret_cast<const V4*>(&lds_raw[lslot][2][r * 32 + c4]);
-        const float lse_r = lds_rawLse[lslot][r];
+        NormIn x;
+        x.q4 = *reinterpret_cast<const V4*>(&lds_raw[lslot][0 * 1024 + r * 32 + c4]);
+        x.do4 = *reinterpret_cast<const V4*>(&lds_raw[lslot][1 * 1024 + r * 32 + c4]);
+        x.o4 = *reinterpret_cast<const V4*>(&lds_raw[lslot][2 * 1024 + r * 32 + c4]);
+        x.lse = reinterpret_cast<const float*>(&lds_raw[lslot][3 * 1024])[r];
+        return x;
+    };
+    auto normalise_store = [&](NormIn x, int qb, int tslot) __attribute__((always_inline)) {
+        const int r = tid >> 3, c4 = (tid & 7) * 4;
         const int row = 32 * qb + r;
-        if (N < R && row >= N) {
+        if (!PLAIN && row >= N) {
 #pragma unroll
-            for (int j = 0; j < 4; j++) { q4[j] = 0; do4[j] = 0; }
+            for (int j = 0; j < 4; j++) { x.q4[j] = 0; x.do4[j] = 0; }
         }
-        const float sq = oct_add(dot4(q4, q4));
-        const float dl = oct_add(dot4(o4, do4));
+        const float sq = oct_add(dot4(x.q4, x.q4));
+        const float dl = oct_add(dot4(x.o4, x.do4));
         const float inv = inv_norm_fast(sq);
         const float iq = inv * scale2;
         SV4 qn;
 #pragma unroll
-        for (int j = 0; j < 4; j++) qn[j] = (SE)((float)q4[j] * iq);
+        for (int j = 0; j < 4; j++) qn[j] = (SE)((float)x.q4[j] * iq);
         *reinterpret_cast<SV4*>(&lds_Qs[tslot][r * kRow + c4]) = qn;
-        *reinterpret_cast<V4*>(&lds_dOs[tslot][r * kRow + c4]) = do4;
-        const float l2 = (row < N && lse_r != -INFINITY) ? -lse_r * kLog2e : -INFINITY;   // padded / fully masked rows: P = 0
+        *reinterpret_cast<V4*>(&lds_dOs[tslot][r * kRow + c4]) = x.do4;
+        const float l2 = ((PLAIN || row < N) && x.lse != -INFINITY) ? -x.lse * kLog2e : -INFINITY;   // padded / fully masked rows: P = 0
         const int role = tid & 7;
-        float* dst = role == 0 ? &lds_ndelta[tslot][r] : role == 1 ? &lds_nlse2[tslot][r] : role == 2 ? &lds_qinv[tslot][r] : lds_dummy + tid;
-        *dst = role == 0 ? -dl : role == 1 ? l2 : inv;
+        (&lds_meta[tslot][0][0])[meta_lane] = role == 0 ? -dl : role == 1 ? l2 : inv;
+    };
+    auto normalise = [&](int qb, int lslot, int tslot) __attribute__((always_inline)) {
+        normalise_store(normalise_load(lslot), qb, tslot);
     };
 
     // ---- dq of block qb of unit b: sum of the four wavefronts' partials, back through q / max(|q|, eps); wavefront w
-    // takes rows 8 w .. 8 w + 7, lane = 4 columns of one row.  q_hat is taken back from the score operand. ----
+    // takes rows 8 w .. 8 w + 7 (the rows it normalised: it may read them from a tile slot right before it
+    // overwrites that slot), lane = 4 columns of one row.  q_hat is taken back from the score operand. ----
     float ds_acc = 0.f;
-    auto sum_block = [&](int b, int qb, int pslot, int tslot) __attribute__((always_inline)) {
+    const char* const dq_base = reinterpret_cast<const char*>(p.dq.ptr) + (int64_t)h * p.dq.sh * (int64_t)sizeof(E);
+    struct SumIn { f32x4 part[WAVES]; SV4 qs; float inv; };
+    auto sum_load = [&](int pslot, int tslot) __attribute__((always_inline)) -> SumIn {
+        const int r = tid >> 3, c4 = (tid & 7) * 4;
+        SumIn x;
+#pragma unroll
+        for (int w = 0; w < WAVES; w++) x.part[w] = *reinterpret_cast<const f32x4*>(&lds_part[pslot][w][r * kPartRow + c4]);
+        x.qs = *reinterpret_cast<const SV4*>(&lds_Qs[tslot][r * kRow + c4]);
+        x.inv = lds_meta[tslot][2][r];
+        return x;
+    };
+    const uint32_t dq_lane = (uint32_t)(((tid >> 3) * (int)p.dq.sn + (tid & 7) * 4) * (int)sizeof(E));
+    const uint32_t dq_rows32 = (uint32_t)(32 * (int)p.dq.sn * (int)sizeof(E));
+    auto sum_store = [&](const SumIn& x, const char* dq_unit, int b, int qb) __attribute__((always_inline)) {
         const int ln = lane_now();
         const int r = 8 * wave + (ln >> 3), c4 = (ln & 7) * 4;
-        f32x4 acc = *reinterpret_cast<const f32x4*>(&lds_part[pslot][0][r * kPartRow + c4]);
+        f32x4 acc = x.part[0];
 #pragma unroll
-        for (int w = 1; w < WAVES; w++) {
-            const f32x4 x = *reinterpret_cast<const f32x4*>(&lds_part[pslot][w][r * kPartRow + c4]);
+        for (int w = 1; w < WAVES; w++)
 #pragma unroll
-            for (int j = 0; j < 4; j++) acc[j] += x[j];
-        }
-        const SV4 qs = *reinterpret_cast<const SV4*>(&lds_Qs[tslot][r * kRow + c4]);
-        const float inv = lds_qinv[tslot][r];
-        float qh[4];
-        float dot = 0.f;
+            for (int j = 0; j < 4; j++) acc[j] += x.part[w][j];
+        // with qs = q_hat s2 (s2 = s log2e):  dq = s / |q| (acc - q_hat (q_hat . acc)) = f acc - qs (f (qs . acc) / s2^2)
+        float dots = 0.f;
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            qh[j] = (float)qs[j] * unscale;
-            dot += acc[j] * qh[j];
-        }
-        dot = oct_add(dot);
-        const float proj = inv < 0.5f / kNormEps ? dot : 0.f;      // |q| <= eps: no projection
-        const float f = s_true * inv;
+        for (int j = 0; j < 4; j++) dots += acc[j] * (float)x.qs[j];
+        dots = oct_add(dots);
+        const float dot = dots * unscale;                               // q_hat . dq_hat / s: the row's dlogit_scale term
+        const float f = s_true * x.inv;
+        const float c = x.inv < 0.5f / kNormEps ? f * dot * unscale : 0.f;      // |q| <= eps: no projection
         V4 o4;
 #pragma unroll
-        for (int j = 0; j < 4; j++) o4[j] = (E)(f * (acc[j] - qh[j] * proj));
+        for (int j = 0; j < 4; j++) o4[j] = (E)(f * acc[j] - (float)x.qs[j] * c);
         const int q = 32 * qb + r;
-        const int qrow = min(q, N - 1);
-        vm_store8_if_below(const_cast<E*>(row_ptr<MAPPED, E>(p.dq, p.map, b, h, qrow)) + c4, o4, q, N);
-        ds_acc += ((ln & 7) == 0 && q < N) ? dot : 0.f;
+        if (PLAIN) {
+            uint32_t voff = dq_lane;
+            asm volatile("" : "+v"(voff));
+            vm_store8(const_cast<char*>(dq_unit), voff + (uint32_t)qb * dq_rows32, o4);
+            ds_acc += (ln & 7) == 0 ? dot : 0.f;
+        } else {
+            const int qrow = min(q, N - 1);
+            E* dst = reinterpret_cast<E*>(const_cast<char*>(dq_unit) + row_byte_offset<E>(unit_row<MAPPED>(p.map, b, qrow), p.dq.sn, c4));
+            vm_store8_if_below(dst, o4, q, N);
+            ds_acc += ((ln & 7) == 0 && q < N) ? dot : 0.f;
+        }
+    };
+    auto sum_block = [&](int b, int qb, int pslot, int tslot) __attribute__((always_inline)) {
+        sum_store(sum_load(pslot, tslot), unit_start(dq_base, p.dq.sb, b), b, qb);
     };
 
     // The rows of the wavefront's own keys (k and v, 16 bytes per lane and key tile) skip the landing area: they
@@ -395,10 +471,10 @@ __global__ void __launch_bounds__(one256::NT) bwd_one_kernel(const BwdParams p) 
 #pragma unroll
             for (int kt = 0; kt < KT; kt++)
 #pragma unroll
-                for (int tt = 0; tt < 2; tt++) tb[kt][tt] = *reinterpret_cast<const f32x4*>(cur.tab + lane4 + (((kt * NQB) * 2 + tt) << 8));
+                for (int tt = 0; tt < 2; tt++) tb[kt][tt] = vm_load16(cur.tab + (((kt * NQB) * 2 + tt) << 8), lane16);
         }
-        dma_block(cur.b, 0, 0);
-        dma_block(cur.b, 1, 1);
+        dma_block(source_of(cur.b), cur.b, 0, 0);
+        dma_block(source_of(cur.b), cur.b, 1, 1);
         fetch_keys(cur.b);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
@@ -409,17 +485,51 @@ __global__ void __launch_bounds__(one256::NT) bwd_one_kernel(const BwdParams p) 
     }
     __syncthreads();
     if (any) {
-        dma_block(cur.b, 2, 0);
+        dma_block(source_of(cur.b), cur.b, 2, 0);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
     __syncthreads();
 
     bool have_prev = false;      // a block whose dq partials wait for their sum
     int b_prev = 0;
+    const char* dq_prev = nullptr;
     // lane parts of the LDS addresses inside a tile slot; what depends on the block is a compile-time constant
     const int row_base = (8 * (l16 >> 2) + (l16 & 3)) * kRow + 8 * g;       // + 4 t * kRow
     const int tr_base = (8 * g + (l16 >> 2)) * kRow + 8 * (l16 & 3);         // + 4 dt (+ 4 kRow)
     SE* const zst = &lds_zst[0][0] + wave * (64 * kRow);
+
+    // ---- dQ_hat^T of a block over this wavefront's keys: B operand = dZ^T out of the slab, A operand = K_hat^T.
+    // Column n of query tile t is query 8 (n / 4) + 4 t + n % 4 of the block; the lane's rows are d = 8 g + 4 dt + i.
+    // The partial goes to LDS as [query][d]. ----
+    SV8 akt[2][2];
+    auto dq_load = [&](SV8 (&bz)[2][2]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int c = 0; c < 2; c++)
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+                bz[c][t] = lds_tr8<SDT>(zst + 32 * c * kRow + tr_base + 4 * t, zst + 32 * c * kRow + tr_base + 4 * t + 4 * kRow);
+    };
+    auto dq_products = [&](const SV8 (&bz)[2][2], int pslot) __attribute__((always_inline)) {
+        f32x4 dqa[2][2];
+#pragma unroll
+        for (int dt = 0; dt < 2; dt++)
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) dqa[dt][t][i] = 0.f;
+#pragma unroll
+        for (int c = 0; c < 2; c++)
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+#pragma unroll
+                for (int dt = 0; dt < 2; dt++) dqa[dt][t] = Elem<SDT>::mfma16(akt[dt][c], bz[c][t], dqa[dt][t]);
+        float* part = &lds_part[pslot][0][0] + wave * (32 * kPartRow);
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+#pragma unroll
+            for (int dt = 0; dt < 2; dt++)
+                *reinterpret_cast<f32x4*>(part + (8 * (l16 >> 2) + 4 * t + (l16 & 3)) * kPartRow + 8 * g + 4 * dt) = dqa[dt][t];
+    };
 
     while (cur.t < t_end) {
         const int b = cur.b;
@@ -429,6 +539,9 @@ __global__ void __launch_bounds__(one256::NT) bwd_one_kernel(const BwdParams p) 
         const float* tab = cur.tab;
         const float* tab_next = have_next ? nxt.tab : tab;
         Unit after = nxt;
+        const char* const src_cur = source_of(b);
+        const char* const src_next = source_of(b_next);
+        const char* const dq_cur = unit_start(dq_base, p.dq.sb, b);
 
         // ---- this wavefront's keys: k_hat (score type) and v as B operands, 1 / |k| for the epilogue ----
         SV8 bk[KT];
@@ -439,7 +552,7 @@ __global__ void __launch_bounds__(one256::NT) bwd_one_kernel(const BwdParams p) 
             const int key = 64 * wave + 16 * kt + l16;
             V8 k8 = kraw[kt];
             bv[kt] = vraw[kt];
-            if (N < R && key >= N) { k8 = zero8<V8>(); bv[kt] = zero8<V8>(); }
+            if (!PLAIN && key >= N) { k8 = zero8<V8>(); bv[kt] = zero8<V8>(); }
             const float sk = col_add(dot8(k8, k8));
             const float ik = inv_norm_fast(sk);
 #pragma unroll
@@ -448,7 +561,6 @@ __global__ void __launch_bounds__(one256::NT) bwd_one_kernel(const BwdParams p) 
         }
         // K_hat^T of the same keys as the A operand of dQ_hat^T += K_hat^T dZ^T: through the wavefront's own slab.
         // A row m <-> d = 8 (m / 4) + 4 dt + m % 4; k-slots 8 g + j <-> key 32 c + 8 g + j of the wavefront.
-        SV8 akt[2][2];
 #pragma unroll
         for (int kt = 0; kt < KT; kt++) st8<SV8>(zst + (16 * kt + l16) * kRow + 8 * g, bk[kt]);
         asm volatile("" ::: "memory");
@@ -480,18 +592,28 @@ __global__ void __launch_bounds__(one256::NT) bwd_one_kernel(const BwdParams p) 
             for (int tt = 0; tt < 2; tt++) {
                 aq[tt] = ld8<SV8>(&lds_Qs[s][row_base + 4 * tt * kRow]);
                 ado[tt] = ld8<V8>(&lds_dOs[s][row_base + 4 * tt * kRow]);
-                nd[tt] = *reinterpret_cast<const f32x4*>(&lds_ndelta[s][8 * g + 4 * tt]);
+                nd[tt] = *reinterpret_cast<const f32x4*>(&lds_meta[s][0][8 * g + 4 * tt]);
             }
         };
         load_rows(0);
 
 #pragma unroll
         for (int qb = 0; qb < NQB; qb++) {
-            // ---- the other stages of the pipeline ----
-            dma_block(qb + 3 < NQB ? b : b_next, (qb + 3) & 7, (qb + 3) & 1);
-            if (qb > 0) sum_block(b, qb - 1, (qb - 1) & 1, (qb - 1) & 3);
-            else if (have_prev) sum_block(b_prev, NQB - 1, 1, 3);
-            normalise((qb + 2) & 7, qb & 1, (qb + 2) & 3);
+            // ---- the other stages of the pipeline, all independent of each other: their LDS reads first, then the
+            // arithmetic (the dq products run on the matrix pipe meanwhile), the stores to memory last ----
+            {
+                const bool do_dq = qb > 0;                 // block 7's products follow the loop
+                const bool do_sum = qb >= 2 || have_prev;
+                SV8 bz[2][2];
+                if (do_dq) dq_load(bz);
+                SumIn si;
+                if (do_sum) si = sum_load(qb & 1, (qb + 2) & 3);
+                const NormIn ni = normalise_load(qb & 1);
+                dma_block(qb + 3 < NQB ? src_cur : src_next, qb + 3 < NQB ? b : b_next, (qb + 3) & 7, (qb + 3) & 1);
+                if (do_dq) dq_products(bz, (qb - 1) & 1);
+                if (do_sum) sum_store(si, qb >= 2 ? dq_cur : dq_prev, qb >= 2 ? b : b_prev, (qb + 6) & 7);
+                normalise_store(ni, (qb + 2) & 7, (qb + 2) & 3);
+            }
             __builtin_amdgcn_sched_barrier(0);
 
             // ---- block qb against the wavefront's 64 keys ----
@@ -500,7 +622,7 @@ __global__ void __launch_bounds__(one256::NT) bwd_one_kernel(const BwdParams p) 
             V8 tdo[2];
             SV8 tq[2];
 #pragma unroll
-            for (int tt = 0; tt < 2; tt++) nl[tt] = *reinterpret_cast<const f32x4*>(&lds_nlse2[s][8 * g + 4 * tt]);
+            for (int tt = 0; tt < 2; tt++) nl[tt] = *reinterpret_cast<const f32x4*>(&lds_meta[s][1][8 * g + 4 * tt]);
 #pragma unroll
             for (int dt = 0; dt < 2; dt++) {
                 // A row m <-> d = 8 (m / 4) + 4 dt + m % 4: the lane's dk / dv values are d = 8 g + 4 dt + i
@@ -510,6 +632,10 @@ __global__ void __launch_bounds__(one256::NT) bwd_one_kernel(const BwdParams p) 
 #pragma unroll
             for (int kt = 0; kt < KT; kt++) {
                 f32x4 sacc[2], pacc[2];
+                // The table values of this key tile were requested a block ago.  Loads return in order, and the
+                // loads issued since are the 6 of the other key tiles and the 2 row copies of this iteration (more
+                // where a unit began in between), so "at most 8 outstanding" covers them, whatever the stores do.
+                if (HAS_TAB) tables_arrived<8>(tb[kt][0], tb[kt][1]);
 #pragma unroll
                 for (int tt = 0; tt < 2; tt++) {
                     // (S + bias + mask) * log2e with the table as the C operand; dP - delta
@@ -521,7 +647,7 @@ __global__ void __launch_bounds__(one256::NT) bwd_one_kernel(const BwdParams p) 
                 if (HAS_TAB) {
                     const float* src = qb + 1 < NQB ? tab + (((kt * NQB + qb + 1) * 2) << 8) : tab_next + (((kt * NQB) * 2) << 8);
 #pragma unroll
-                    for (int tt = 0; tt < 2; tt++) tb[kt][tt] = *reinterpret_cast<const f32x4*>(src + lane4 + (tt << 8));
+                    for (int tt = 0; tt < 2; tt++) tb[kt][tt] = vm_load16(src + (tt << 8), lane16);
                 }
                 if (kt == KT - 1) load_rows((qb + 1) & 7);
                 // everything read ahead is on its way before this tile's elementwise work starts
@@ -559,40 +685,18 @@ __global__ void __launch_bounds__(one256::NT) bwd_one_kernel(const BwdParams p) 
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
-
-            // ---- dQ_hat^T of the block over this wavefront's keys: B operand = dZ^T out of the slab.  Column n of
-            // query tile t is query 8 (n / 4) + 4 t + n % 4 of the block; the lane's rows are d = 8 g + 4 dt + i. ----
-            {
-                asm volatile("" ::: "memory");
-                f32x4 dqa[2][2];
-#pragma unroll
-                for (int dt = 0; dt < 2; dt++)
-#pragma unroll
-                    for (int t = 0; t < 2; t++)
-#pragma unroll
-                        for (int i = 0; i < 4; i++) dqa[dt][t][i] = 0.f;
-#pragma unroll
-                for (int c = 0; c < 2; c++)
-#pragma unroll
-                    for (int t = 0; t < 2; t++) {
-                        const SV8 bz = lds_tr8<SDT>(zst + 32 * c * kRow + tr_base + 4 * t, zst + 32 * c * kRow + tr_base + 4 * t + 4 * kRow);
-#pragma unroll
-                        for (int dt = 0; dt < 2; dt++) dqa[dt][t] = Elem<SDT>::mfma16(akt[dt][c], bz, dqa[dt][t]);
-                    }
-                float* part = &lds_part[qb & 1][0][0] + wave * (32 * kPartRow);
-#pragma unroll
-                for (int t = 0; t < 2; t++)
-#pragma unroll
-                    for (int dt = 0; dt < 2; dt++)
-                        *reinterpret_cast<f32x4*>(part + (8 * (l16 >> 2) + 4 * t + (l16 & 3)) * kPartRow + 8 * g + 4 * dt) = dqa[dt][t];
-                asm volatile("" ::: "memory");
-            }
             // The rows requested at the top of this iteration are tiles in the next one: they have landed once at most
             // the table loads issued since (8) are outstanding.
             if (HAS_TAB) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
             else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             lds_barrier();
             __builtin_amdgcn_sched_barrier(0);
+        }
+        {
+            SV8 bz[2][2];
+            dq_load(bz);
+            dq_products(bz, 1);       // block 7; its sum follows in the second iteration from here (or behind the loop)
+            asm volatile("" ::: "memory");
         }
         fetch_keys(b_next);
         // ---- epilogue dk, dv: lane (key, g) holds d = 8 g + 4 dt + i, which is 16 bytes of a row ----
@@ -624,12 +728,17 @@ __global__ void __launch_bounds__(one256::NT) bwd_one_kernel(const BwdParams p) 
             vm_store16_if_below(const_cast<E*>(row_ptr<MAPPED, E>(p.dv, p.map, b, h, krow)) + 8 * g, v8, key, N);
         }
         b_prev = b;
+        dq_prev = dq_cur;
         have_prev = true;
         cur = nxt;
         nxt = after;
     }
-    // the last block of the last unit (its partials were complete at the loop's last barrier)
-    if (have_prev) sum_block(b_prev, NQB - 1, 1, 3);
+    // the last two blocks of the last unit
+    if (have_prev) {
+        lds_barrier();
+        sum_block(b_prev, NQB - 2, 0, 2);
+        sum_block(b_prev, NQB - 1, 1, 3);
+    }
 
     // ---- dlogit_scale: one partial per workgroup ----
     if (p.scale_kind == FWA2_SCALE_TENSOR) {
@@ -663,10 +772,10 @@ __global__ void __launch_bounds__(one256::NT) bwd_one_kernel(const BwdParams p) 
 }
 
 // ---- host side -----------------------------------------------------------------
-template <int DT, bool HAS_BIAS, bool HAS_TAB, bool MASKED, bool MAPPED>
+template <int DT, bool HAS_BIAS, bool HAS_TAB, bool MASKED, int ROWS>
 static hipError_t launch_one(BwdParams p, hipStream_t st, int max_groups, int* groups_out) {
     static std::atomic<int> fit_by_device[kFitDevices];
-    const int fit = resident_per_cu_cached(bwd_one_kernel<DT, HAS_BIAS, HAS_TAB, MASKED, MAPPED>, one256::NT, fit_by_device);
+    const int fit = resident_per_cu_cached(bwd_one_kernel<DT, HAS_BIAS, HAS_TAB, MASKED, ROWS>, one256::NT, fit_by_device);
     int groups = (p.cus * fit) / p.heads;
     if (groups < 1) groups = 1;
     if (groups > max_groups) groups = max_groups;
@@ -674,7 +783,7 @@ static hipError_t launch_one(BwdParams p, hipStream_t st, int max_groups, int* g
     p.db_parts = groups;
     p.db_slot0 = 0;
     p.ds_parts = groups;
-    hipLaunchKernelGGL((bwd_one_kernel<DT, HAS_BIAS, HAS_TAB, MASKED, MAPPED>), dim3(p.heads * groups), dim3(one256::NT), 0, st, p);
+    hipLaunchKernelGGL((bwd_one_kernel<DT, HAS_BIAS, HAS_TAB, MASKED, ROWS>), dim3(p.heads * groups), dim3(one256::NT), 0, st, p);
     if (groups_out) { groups_out[0] = groups; groups_out[1] = groups; }
     return hipGetLastError();
 }
@@ -688,11 +797,13 @@ static hipError_t launch_one_dt(const BwdParams& p, bool has_bias, int mask_dt, 
     if (e != hipSuccess) return e;
     if (p.ev_start) (void)hipEventRecord(p.ev_start, st);
 #define FWA2_ONE_CASE(B, T, M)                                                                                       \
-    (mapped ? launch_one<DT, B, T, M, true>(p, st, max_groups, groups_out) : launch_one<DT, B, T, M, false>(p, st, max_groups, groups_out))
+    (mapped ? launch_one<DT, B, T, M, 1>(p, st, max_groups, groups_out)                                              \
+            : p.n == one256::R ? launch_one<DT, B, T, M, 2>(p, st, max_groups, groups_out) : launch_one<DT, B, T, M, 0>(p, st, max_groups, groups_out))
     if (has_bias) e = masked ? FWA2_ONE_CASE(true, true, true) : FWA2_ONE_CASE(true, true, false);
     else if (masked) e = FWA2_ONE_CASE(false, true, true);
     else if (has_tab) e = FWA2_ONE_CASE(false, true, false);
-    else e = FWA2_ONE_CASE(false, false, false);
+    else e = mapped ? launch_one<DT, false, false, false, 1>(p, st, max_groups, groups_out)
+                    : launch_one<DT, false, false, false, 2>(p, st, max_groups, groups_out);      // no table: 256 tokens
 #undef FWA2_ONE_CASE
     if (p.ev_stop) (void)hipEventRecord(p.ev_stop, st);
     return e;
