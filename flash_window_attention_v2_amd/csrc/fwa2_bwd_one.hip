@@ -596,6 +596,7 @@ __global__ void __launch_bounds__(one256::NT) bwd_one_kernel(const BwdParams p) 
             }
         };
         load_rows(0);
+        SV8 bz[2][2];      // dZ^T of the block before: read behind its last key tile, used at the top of the next iteration
 
 #pragma unroll
         for (int qb = 0; qb < NQB; qb++) {
@@ -604,8 +605,6 @@ __global__ void __launch_bounds__(one256::NT) bwd_one_kernel(const BwdParams p) 
             {
                 const bool do_dq = qb > 0;                 // block 7's products follow the loop
                 const bool do_sum = qb >= 2 || have_prev;
-                SV8 bz[2][2];
-                if (do_dq) dq_load(bz);
                 SumIn si;
                 if (do_sum) si = sum_load(qb & 1, (qb + 2) & 3);
                 const NormIn ni = normalise_load(qb & 1);
@@ -650,6 +649,13 @@ __global__ void __launch_bounds__(one256::NT) bwd_one_kernel(const BwdParams p) 
                     for (int tt = 0; tt < 2; tt++) tb[kt][tt] = vm_load16(src + (tt << 8), lane16);
                 }
                 if (kt == KT - 1) load_rows((qb + 1) & 7);
+                // the dbias accumulators of the last blocks come out of LDS: requested here, used behind the exponentials
+                f32x4 dbs[2];
+                if (HAS_BIAS && db_in_lds(qb)) {
+#pragma unroll
+                    for (int hf = 0; hf < 2; hf++)
+                        dbs[hf] = *reinterpret_cast<const f32x4*>(lds_db + ((((qb - (NQB - kLdsQb)) * KT + kt) * 2 + hf) * NT + tid) * 4);
+                }
                 // everything read ahead is on its way before this tile's elementwise work starts
                 asm volatile("" : "+v"(sacc[0]), "+v"(sacc[1]) :: "memory");
                 if (kt == 2 && qb == 3 && have_next) after = unit_at(nxt.t + p.groups);      // scalar work, off the critical path
@@ -672,7 +678,7 @@ __global__ void __launch_bounds__(one256::NT) bwd_one_kernel(const BwdParams p) 
                     for (int hf = 0; hf < 2; hf++) {
                         if (db_in_lds(qb)) {
                             f32x4* slot = reinterpret_cast<f32x4*>(lds_db + ((((qb - (NQB - kLdsQb)) * KT + kt) * 2 + hf) * NT + tid) * 4);
-                            *slot = Elem<SDT>::mfma16(sel[hf], z8, *slot);
+                            *slot = Elem<SDT>::mfma16(sel[hf], z8, dbs[hf]);
                         } else {
                             dbq[qb][kt][hf] = Elem<SDT>::mfma16(sel[hf], z8, dbq[qb][kt][hf]);
                         }
@@ -685,19 +691,20 @@ __global__ void __launch_bounds__(one256::NT) bwd_one_kernel(const BwdParams p) 
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
+            // dZ^T of this block for the dq products of the next iteration: the wavefront's own data, so the reads
+            // need not wait for the barrier, and the barrier need not wait for them: it waits until the 8 youngest
+            // LDS operations (these reads) are all that is outstanding, i.e. for every write before them.
+            asm volatile("" ::: "memory");
+            dq_load(bz);
             // The rows requested at the top of this iteration are tiles in the next one: they have landed once at most
             // the table loads issued since (8) are outstanding.
             if (HAS_TAB) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
             else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            lds_barrier();
+            asm volatile("s_waitcnt lgkmcnt(8)\n\ts_barrier" ::: "memory");
             __builtin_amdgcn_sched_barrier(0);
         }
-        {
-            SV8 bz[2][2];
-            dq_load(bz);
-            dq_products(bz, 1);       // block 7; its sum follows in the second iteration from here (or behind the loop)
-            asm volatile("" ::: "memory");
-        }
+        dq_products(bz, 1);       // block 7; its sum follows in the second iteration from here (or behind the loop)
+        asm volatile("" ::: "memory");
         fetch_keys(b_next);
         // ---- epilogue dk, dv: lane (key, g) holds d = 8 g + 4 dt + i, which is 16 bytes of a row ----
         const int ln_e = lane_now();
