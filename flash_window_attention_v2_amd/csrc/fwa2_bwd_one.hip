@@ -153,6 +153,11 @@ template <int N_OUT>
 __device__ __forceinline__ void tables_arrived(f32x4& a, f32x4& b) {
     asm volatile("s_waitcnt vmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N_OUT) : "memory");
 }
+// 16 bytes per lane at base + voff (base: wavefront-uniform); two wait states before the data registers may change
+template <class V8>
+__device__ __forceinline__ void vm_store16(void* base, uint32_t voff, V8 v) {
+    asm volatile("global_store_dwordx4 %0, %1, %2 nt\n\ts_nop 1" ::"v"(voff), "v"(v), "s"(base) : "memory");
+}
 // 8 bytes per lane at base + voff (base: wavefront-uniform)
 template <class V4>
 __device__ __forceinline__ void vm_store8(void* base, uint32_t voff, V4 v) {
@@ -439,7 +444,24 @@ __global__ void __launch_bounds__(one256::NT) bwd_one_kernel(const BwdParams p) 
     // The rows of the wavefront's own keys (k and v, 16 bytes per lane and key tile) skip the landing area: they
     // are requested after the last block of a unit and used once the dk / dv of that unit have been stored.
     V8 kraw[KT], vraw[KT];
+    // byte offset of this lane's 16 bytes of key row 64 wave + l16 in a tensor with rows `sn` elements apart (whole
+    // windows without a map: the other key tiles are 16 rows further on each)
+    auto key_lane_offset = [&](int64_t sn) -> uint32_t {
+        const int ln = lane_now();
+        return (uint32_t)(((64 * wave + (ln & 15)) * (int)sn + 8 * (ln >> 4)) * (int)sizeof(E));
+    };
     auto fetch_keys = [&](int b) __attribute__((always_inline)) {
+        if (PLAIN) {
+            const char* ku = unit_start(reinterpret_cast<const char*>(p.k.ptr) + (int64_t)h * p.k.sh * (int64_t)sizeof(E), p.k.sb, b);
+            const char* vu = unit_start(reinterpret_cast<const char*>(p.v.ptr) + (int64_t)h * p.v.sh * (int64_t)sizeof(E), p.v.sb, b);
+            const uint32_t ko = key_lane_offset(p.k.sn), vo = key_lane_offset(p.v.sn);
+#pragma unroll
+            for (int kt = 0; kt < KT; kt++) {
+                kraw[kt] = ld8<V8>(reinterpret_cast<const E*>(ku + (ko + (uint32_t)(16 * kt * (int)sizeof(E)) * (uint32_t)p.k.sn)));
+                vraw[kt] = ld8<V8>(reinterpret_cast<const E*>(vu + (vo + (uint32_t)(16 * kt * (int)sizeof(E)) * (uint32_t)p.v.sn)));
+            }
+            return;
+        }
         const int ln = lane_now();
         const int l16 = ln & 15, g = ln >> 4;
 #pragma unroll
@@ -708,31 +730,45 @@ __global__ void __launch_bounds__(one256::NT) bwd_one_kernel(const BwdParams p) 
         fetch_keys(b_next);
         // ---- epilogue dk, dv: lane (key, g) holds d = 8 g + 4 dt + i, which is 16 bytes of a row ----
         const int ln_e = lane_now();
+        const char* dk_unit = nullptr;
+        const char* dv_unit = nullptr;
+        uint32_t dk_off = 0, dv_off = 0;
+        if (PLAIN) {
+            dk_unit = unit_start(reinterpret_cast<const char*>(p.dk.ptr) + (int64_t)h * p.dk.sh * (int64_t)sizeof(E), p.dk.sb, b);
+            dv_unit = unit_start(reinterpret_cast<const char*>(p.dv.ptr) + (int64_t)h * p.dv.sh * (int64_t)sizeof(E), p.dv.sb, b);
+            dk_off = key_lane_offset(p.dk.sn);
+            dv_off = key_lane_offset(p.dv.sn);
+        }
 #pragma unroll
         for (int kt = 0; kt < KT; kt++) {
             const int l16 = ln_e & 15, g = ln_e >> 4;
             const int key = 64 * wave + 16 * kt + l16;
-            float x[8], a[8];
+            // dk = (dk_hat - k_hat (k_hat . dk_hat)) / |k| with dk_hat = ln2 * accumulator (undoing the log2e folded into Q_hat)
+            float x[8];
             float dot = 0.f;
 #pragma unroll
             for (int j = 0; j < 8; j++) {
                 x[j] = (float)bk[kt][j];
-                a[j] = dkacc[kt][j >> 2][j & 3] * kLn2;      // undo the log2e folded into Q_hat
-                dot += a[j] * x[j];
+                dot += dkacc[kt][j >> 2][j & 3] * x[j];
             }
             dot = col_add(dot);
-            const float inv = fabsf(kinv[kt]);
+            const float c = fabsf(kinv[kt]) * kLn2;
             const float proj = kinv[kt] > 0.f ? dot : 0.f;
             V8 o8, v8;
 #pragma unroll
             for (int j = 0; j < 8; j++) {
-                o8[j] = (E)(inv * (a[j] - x[j] * proj));
+                o8[j] = (E)(c * (dkacc[kt][j >> 2][j & 3] - x[j] * proj));
                 v8[j] = (E)dvacc[kt][j >> 2][j & 3];
             }
-            // keys beyond n (only with n < 256) address row n - 1 and are masked out of the store
-            const int krow = min(key, N - 1);
-            vm_store16_if_below(const_cast<E*>(row_ptr<MAPPED, E>(p.dk, p.map, b, h, krow)) + 8 * g, o8, key, N);
-            vm_store16_if_below(const_cast<E*>(row_ptr<MAPPED, E>(p.dv, p.map, b, h, krow)) + 8 * g, v8, key, N);
+            if (PLAIN) {
+                vm_store16(const_cast<char*>(dk_unit), dk_off + (uint32_t)(16 * kt * (int)sizeof(E)) * (uint32_t)p.dk.sn, o8);
+                vm_store16(const_cast<char*>(dv_unit), dv_off + (uint32_t)(16 * kt * (int)sizeof(E)) * (uint32_t)p.dv.sn, v8);
+            } else {
+                // keys beyond n (only with n < 256) address row n - 1 and are masked out of the store
+                const int krow = min(key, N - 1);
+                vm_store16_if_below(const_cast<E*>(row_ptr<MAPPED, E>(p.dk, p.map, b, h, krow)) + 8 * g, o8, key, N);
+                vm_store16_if_below(const_cast<E*>(row_ptr<MAPPED, E>(p.dv, p.map, b, h, krow)) + 8 * g, v8, key, N);
+            }
         }
         b_prev = b;
         dq_prev = dq_cur;

@@ -361,11 +361,22 @@ def _model_step_against_classic(kw, batch, classes):
         grads[name] = {k: p.grad.float() for k, p in model.named_parameters()}
         assert all(torch.isfinite(g).all() for g in grads[name].values()), name
 
-    def worst(name):
-        return max(float((grads[name][k] - grads["ref"][k]).abs().max() / (grads["ref"][k].abs().max() + 1e-6))
-                   for k in grads["ref"])
+    def errors(name):
+        return {k: float((grads[name][k] - grads["ref"][k]).abs().max() / (grads["ref"][k].abs().max() + 1e-6))
+                for k in grads["ref"]}
 
-    return losses, worst("fused"), worst("eager"), fused
+    err_fused, err_eager = errors("fused"), errors("eager")
+    for k in sorted(err_fused, key=err_fused.get, reverse=True)[:4]:
+        print(f"  worst fused parameter gradients: {k}: fused {err_fused[k]:.3e} eager {err_eager[k]:.3e} "
+              f"(max |ref| {float(grads['ref'][k].abs().max()):.3e})")
+    import statistics
+    keys = sorted(err_fused)
+    stats = {"mean_fused": statistics.fmean(err_fused[k] for k in keys), "mean_eager": statistics.fmean(err_eager[k] for k in keys),
+             "median_fused": statistics.median(err_fused[k] for k in keys), "median_eager": statistics.median(err_eager[k] for k in keys),
+             "fused_better": sum(err_fused[k] <= err_eager[k] for k in keys), "count": len(keys)}
+    print("  parameter-gradient errors over all parameters:", {k: (round(v, 5) if isinstance(v, float) else v) for k, v in stats.items()})
+    losses["stats"] = stats
+    return losses, max(err_fused.values()), max(err_eager.values()), fused
 
 
 @pytest.mark.gpu
@@ -394,8 +405,16 @@ def test_model_of_the_end_to_end_benchmark_gpu():
     assert shifts == [0, 8, 0, 8] + [0] * 8          # the 16 x 16 and 8 x 8 grids are one window: no shift
     print(f"C5 batch 4: loss ref {losses['ref']:.6f} fused {losses['fused']:.6f} eager {losses['eager']:.6f}; "
           f"worst parameter-gradient error fused {fused:.4e} eager {eager:.4e}")
+    # The operator alone is 3 - 6 x closer to fp32 than the eager bf16 path (tests/test_gpu_parity.py); inside the
+    # model the bf16 rounding of every other layer is the same in both runs and dominates most parameters, so the
+    # two runs are held against each other where that can be told apart from noise: the loss, the majority of the
+    # parameters, and the mean error; the single worst parameter (a nearly cancelling sum with a gradient of
+    # 1e-4 .. 1e-3) within a factor of two.
+    stats = losses["stats"]
     assert abs(losses["fused"] - losses["ref"]) < 3e-2
-    assert abs(losses["fused"] - losses["ref"]) <= max(2.0 * abs(losses["eager"] - losses["ref"]), 1e-2)
+    assert abs(losses["fused"] - losses["ref"]) <= abs(losses["eager"] - losses["ref"])
+    assert 2 * stats["fused_better"] >= stats["count"], stats
+    assert stats["mean_fused"] <= 1.1 * stats["mean_eager"], stats
     assert fused < max(2.0 * eager, 5e-2), (fused, eager)
 
 
