@@ -29,10 +29,12 @@ if ROOT not in sys.path:
 METRIC = "fwd+bwd ms & TFLOPS (% MFMA peak), B64 nW64 H3 d32 N256 bf16, 1 GPU"
 MFMA_BF16_PEAK_TFLOPS = 2500.0     # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0              # MI355X HBM3E
-# HBM bytes per launch of the key-side backward kernel at the benchmark shape, from
+# HBM bytes per launch of the backward kernel at the benchmark shape, from
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a copy kernel of known size
 # (profiles/kernels_C3_fwd_bwd.txt: FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0).
 BWD_KERNEL_TRAFFIC_BYTES = 1.630e9
+# device memory the library holds on every GPU whether or not it is used (the scratch of fwa2_backward_static)
+STATIC_SCRATCH_MB = 128.0
 
 
 def log(*a):
@@ -300,34 +302,64 @@ def main():
             dev[name].requires_grad_(True)
         return dev
 
-    def make_step(dev, events=None):
+    def make_step(dev):
         leaves = [dev[n] for n in ("q", "k", "v", "bias", "logit_scale")]
 
         def step(i):
-            if events is not None and i >= 0:
-                lib.fwa2_set_kernel_events(*events.pairs[i])
             o = flash_win_attn_v2_func(dev["q"], dev["k"], dev["v"], dev["logit_scale"], dev["bias"], dev["mask"])
             o.backward(dev["do"])
-            if events is not None:
-                lib.fwa2_set_kernel_events(None, None)
             for t in leaves:
                 t.grad = None
         return step
+
+    def kernel_times(dev, steps, warmup):
+        """The main kernels of one step, each between a pair of HIP events that the library records on the launch
+        stream around them (fwa2_problem.ev_start / ev_stop): the same two library calls a step makes, issued
+        through the launchers under the reference's names.  Returns (forward ms list, backward-kernel ms list)."""
+        from flash_window_attention_v2_amd.kernels import _flash_attn_backward, _flash_attn_forward
+        q, k, v, ls, bias, mask, do = (dev[n].detach() for n in ("q", "k", "v", "logit_scale", "bias", "mask", "do"))
+        dq, dk, dv = (torch.empty_like(x) for x in (q, k, v))
+        ds, db = torch.empty_like(ls), torch.empty_like(bias)
+        ev_f, ev_b = HipEvents(steps), HipEvents(steps)
+        for i in range(-warmup, steps):
+            o, lse, _ = _flash_attn_forward(q, k, v, ls, bias=bias, mask=mask, scale_type="tensor",
+                                            _events=ev_f.pairs[i] if i >= 0 else None)
+            _flash_attn_backward(do, q, k, v, ls, o, lse, dq, dk, dv, ds, db, bias=bias, mask=mask, scale_type="tensor",
+                                 _events=ev_b.pairs[i] if i >= 0 else None)
+        torch.cuda.synchronize()
+        return ev_f.elapsed_ms(), ev_b.elapsed_ms()
 
     cfg = CONFIGS["C3"]
     bw = cfg["batch"] * cfg["n_windows"]
     log(f"[bench] building inputs {cfg}")
     dev = setup(cfg)
-    events = HipEvents(args.steps)
     log("[bench] timing forward+backward")
-    ms = time_steps(make_step(dev, events), args.steps, args.warmup, torch)
-    kern_ms = events.elapsed_ms()
-    kern_avg = sum(kern_ms) / len(kern_ms)
+    ms = time_steps(make_step(dev), args.steps, args.warmup, torch)
+    log("[bench] timing the kernels of a step")
+    fwd_kern_ms, bwd_kern_ms = kernel_times(dev, args.steps, min(args.warmup, 5))
+    kern_avg = sum(bwd_kern_ms) / len(bwd_kern_ms)
     fl_all = flops_matmul(bw, cfg["heads"], cfg["n"], cfg["d"])
-    # the dominant kernel (key-side backward: S recompute, dP, dV, dK) does 8 N^2 d flops per unit
-    fl_bwd = 8 * cfg["n"] * cfg["n"] * cfg["d"] * bw * cfg["heads"]
+    # the dominant kernel is the whole backward in one pass (S recomputed once, dP, dV, dK, dQ): 10 N^2 d flops
+    # per unit; its algorithmic bytes are the backward's (q, k, v, o, dO in; dq, dk, dv, dbias out; lse, bias, mask)
+    fl_bwd = flops_matmul(bw, cfg["heads"], cfg["n"], cfg["d"], fwd=False)
+    by_bwd = bytes_min(bw, cfg["heads"], cfg["n"], cfg["d"], cfg["n_windows"], fwd=False)
     tflops = fl_all / (ms * 1e-3) * 1e-12
     achieved = fl_bwd / (kern_avg * 1e-3) * 1e-12
+
+    def kernel_row(name, ms_list, flops, nbytes):
+        avg = sum(ms_list) / len(ms_list)
+        med = sorted(ms_list)[len(ms_list) // 2]
+        return {"kernel": name, "ms": round(avg, 4), "ms_median": round(med, 4), "flops": flops, "bytes": nbytes,
+                "tflops": round(flops / avg * 1e-9, 1), "frac_mfma_peak": round(flops / avg * 1e-9 / MFMA_BF16_PEAK_TFLOPS, 4),
+                "gbs": round(nbytes / avg * 1e-6, 1), "frac_hbm_peak": round(nbytes / avg * 1e-6 / HBM_PEAK_GBS, 4)}
+
+    kernels = [
+        kernel_row("forward: fwd_resident_kernel, unmasked + masked launch", fwd_kern_ms,
+                   flops_matmul(bw, cfg["heads"], cfg["n"], cfg["d"], bwd=False),
+                   bytes_min(bw, cfg["heads"], cfg["n"], cfg["d"], cfg["n_windows"], bwd=False)),
+        kernel_row("backward: bwd_one_kernel (dq, dk, dv, dbias partials, dlogit_scale terms in one pass)", bwd_kern_ms,
+                   fl_bwd, by_bwd),
+    ]
 
     result = {
         "metric": METRIC, "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
@@ -336,12 +368,12 @@ def main():
         "config": {"workload": "C3: B64 x 64 windows, H3, N256, d32, bf16, shift-8 mask, fwd+bwd", "bw": bw,
                    "heads": cfg["heads"], "n": cfg["n"], "head_dim": cfg["d"]},
         "pct_mfma_peak": round(100 * tflops / MFMA_BF16_PEAK_TFLOPS, 2),
-        "roofline": {"bound": "mfma", "kernel": "bwd_key_kernel (dk, dv, dbias, delta; one launch)", "achieved": round(achieved, 2),
-                     "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+        "roofline": {"bound": "mfma", "kernel": "bwd_one_kernel (the whole backward in one pass, one launch)",
+                     "achieved": round(achieved, 2), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": BWD_KERNEL_TRAFFIC_BYTES,
                      "kernel_ms": round(kern_avg, 4),
-                     "hbm_frac_of_8TBs": round(bw * cfg["heads"] * (7 * cfg["n"] * cfg["d"] * 2 + 4 * cfg["n"])
-                                               / (kern_avg * 1e-3) / (HBM_PEAK_GBS * 1e9), 4)},
+                     "hbm_frac_of_8TBs": round(by_bwd / (kern_avg * 1e-3) / (HBM_PEAK_GBS * 1e9), 4),
+                     "kernels": kernels},
     }
 
     if not args.no_extras:
@@ -363,6 +395,8 @@ def main():
         base = torch.cuda.memory_allocated()
         step(-1); torch.cuda.synchronize()
         extras["peak_mem_mb_new"] = round((torch.cuda.max_memory_allocated() - base) / 2**20, 1)
+        extras["static_scratch_mb"] = STATIC_SCRATCH_MB
+        extras["peak_mem_mb_new_with_static_scratch"] = round(extras["peak_mem_mb_new"] + STATIC_SCRATCH_MB, 1)
         from flash_window_attention_v2_amd import win_attention_torch
         torch.cuda.empty_cache(); torch.cuda.reset_peak_memory_stats()
         base = torch.cuda.memory_allocated()
@@ -372,16 +406,21 @@ def main():
         del o
         for n_ in ("q", "k", "v", "bias", "logit_scale"):
             dev[n_].grad = None
-        extras["peak_mem_ratio"] = round(extras["peak_mem_mb_new"] / extras["peak_mem_mb_classic_bf16"], 4)
+        extras["peak_mem_ratio"] = round(extras["peak_mem_mb_new_with_static_scratch"] / extras["peak_mem_mb_classic_bf16"], 4)
         del dev
         torch.cuda.empty_cache()
         # N = 64 (config 2) is bandwidth-bound: report achieved HBM GB/s
         log("[bench] config 2 (N=64)")
         c2 = CONFIGS["C2"]
         dev2 = setup(c2)
-        ms2 = time_steps(make_step(dev2), args.steps, args.warmup, torch)
+        # one event pair per call, caches flushed before every call (the step touches 0.6 GB against a 256 MB
+        # memory-side cache), median and mean
+        step2 = make_step(dev2)
+        ms2, ms2_mean = timed_calls(torch, lambda: step2(0), args.steps, args.warmup, L2Flush(torch))
         bw2 = c2["batch"] * c2["n_windows"]
         extras["c2_fwd_bwd_ms"] = round(ms2, 4)
+        extras["c2_fwd_bwd_ms_mean"] = round(ms2_mean, 4)
+        extras["c2_timing"] = "per-call event pairs, 512 MiB flush before each call, median (and mean)"
         extras["c2_hbm_gbs"] = round(bytes_min(bw2, c2["heads"], c2["n"], c2["d"], c2["n_windows"]) / ms2 * 1e-6, 1)
         extras["c2_hbm_frac"] = round(extras["c2_hbm_gbs"] / HBM_PEAK_GBS, 4)
         extras["c2_tflops"] = round(flops_matmul(bw2, c2["heads"], c2["n"], c2["d"]) / ms2 * 1e-9, 2)

@@ -9,7 +9,7 @@ import ctypes
 import os
 import threading
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 OK, ERR_INVALID_ARGUMENT, ERR_UNSUPPORTED, ERR_HIP, ERR_NO_DEVICE = range(5)
 F16, BF16, F32 = 0, 1, 2
@@ -31,7 +31,6 @@ EXPORTS = (
     "fwa2_backward_static",
     "fwa2_cpb_bias_forward",
     "fwa2_cpb_bias_backward",
-    "fwa2_set_kernel_events",
 )
 
 
@@ -64,6 +63,7 @@ class Problem(ctypes.Structure):
         ("shift_h", ctypes.c_int32), ("shift_w", ctypes.c_int32),
         ("n_keys", ctypes.c_int32), ("scale_head_dim", ctypes.c_int32),
         ("mask_regions", ctypes.c_void_p),
+        ("ev_start", ctypes.c_void_p), ("ev_stop", ctypes.c_void_p),
     ]
 
 
@@ -116,8 +116,6 @@ def load():
         lib.fwa2_cpb_bias_backward.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                                ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
         lib.fwa2_cpb_bias_backward.restype = ctypes.c_int
-        lib.fwa2_set_kernel_events.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
-        lib.fwa2_set_kernel_events.restype = None
         if lib.fwa2_abi_version() != ABI_VERSION:
             raise Fwa2Error(f"libfwa2 ABI {lib.fwa2_abi_version()} != binding ABI {ABI_VERSION}")
         _lib = lib

@@ -29,8 +29,6 @@ hipError_t launch_cpb_bias_backward(const void* table, const void* dbias, int dt
 namespace {
 
 thread_local char g_err[512] = "";
-// measurement hook: process-wide, because autograd runs backward on its own thread
-std::atomic<void*> g_ev_start{nullptr}, g_ev_stop{nullptr};
 
 int fail(int code, const char* fmt, ...) {
     va_list ap;
@@ -163,6 +161,8 @@ int validate(const fwa2_problem* p, int backward) {
             return fail(FWA2_ERR_UNSUPPORTED, "window map: windows of more than %d tokens (or wider than 64) are not supported",
                         fwa2::kMapMaxN);
     }
+    if ((p->ev_start == nullptr) != (p->ev_stop == nullptr))
+        return fail(FWA2_ERR_INVALID_ARGUMENT, "ev_start and ev_stop: give both events or neither");
     if (p->lse == nullptr) return fail(FWA2_ERR_INVALID_ARGUMENT, "lse: null pointer");
     if (p->lse_stride_h < p->n) return fail(FWA2_ERR_INVALID_ARGUMENT, "lse: head stride %lld < n", (long long)p->lse_stride_h);
     if (backward) {
@@ -289,17 +289,15 @@ int fwa2_cpb_bias_backward(const void* table, const void* dbias, int dtype, int 
     return FWA2_OK;
 }
 
-void fwa2_set_kernel_events(void* start, void* stop) {
-    g_ev_start.store(start);
-    g_ev_stop.store(stop);
-}
-
 int fwa2_forward(const fwa2_problem* p) {
     g_err[0] = 0;
     int rc = validate(p, 0);
     if (rc) return rc;
+    const bool timed = p->ev_start != nullptr && p->ev_stop != nullptr;
     if (fwa2::generic_problem(p->head_dim, p->n, p->n_keys > 0 ? p->n_keys : p->n)) {
+        if (timed) (void)hipEventRecord((hipEvent_t)p->ev_start, (hipStream_t)p->stream);
         hipError_t eg = fwa2::launch_generic(p, false);
+        if (timed) (void)hipEventRecord((hipEvent_t)p->ev_stop, (hipStream_t)p->stream);
         if (eg != hipSuccess) return fail(FWA2_ERR_HIP, "forward launch: %s", hipGetErrorString(eg));
         return FWA2_OK;
     }
@@ -322,8 +320,10 @@ int fwa2_forward(const fwa2_problem* p) {
     k.side_vec_rows = (!p->bias.ptr || row_groups_ok(p->bias.ptr, p->bias.stride_a, p->bias.stride_n, p->n)) &&
                       (!p->mask.ptr || row_groups_ok(p->mask.ptr, p->mask.stride_a, p->mask.stride_n, p->n));
     k.cus = cu_count();
+    if (timed) (void)hipEventRecord((hipEvent_t)p->ev_start, (hipStream_t)p->stream);
     hipError_t e = fwa2::launch_forward(k, p->dtype, p->bias.ptr != nullptr, p->mask.ptr ? p->mask_dtype : -1,
                                         (hipStream_t)p->stream);
+    if (timed) (void)hipEventRecord((hipEvent_t)p->ev_stop, (hipStream_t)p->stream);
     if (e != hipSuccess) return fail(FWA2_ERR_HIP, "forward launch: %s", hipGetErrorString(e));
     return FWA2_OK;
 }
@@ -358,8 +358,10 @@ static int run_backward(const fwa2_problem* p) {
                       (!p->mask.ptr || row_groups_ok(p->mask.ptr, p->mask.stride_a, p->mask.stride_n, p->n));
     k.workspace = p->workspace;
     k.cus = cu_count();
-    k.ev_start = (hipEvent_t)g_ev_start.load();
-    k.ev_stop = (hipEvent_t)g_ev_stop.load();
+    if (p->ev_start != nullptr && p->ev_stop != nullptr) {
+        k.ev_start = (hipEvent_t)p->ev_start;
+        k.ev_stop = (hipEvent_t)p->ev_stop;
+    }
     hipError_t e = fwa2::launch_backward(k, p->dtype, p->bias.ptr != nullptr, p->mask.ptr ? p->mask_dtype : -1,
                                          (hipStream_t)p->stream);
     if (e != hipSuccess) return fail(FWA2_ERR_HIP, "backward launch: %s", hipGetErrorString(e));

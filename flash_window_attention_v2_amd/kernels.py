@@ -213,16 +213,19 @@ def _pad8(x):
     return torch.nn.functional.pad(x, (0, -x.shape[-1] % 8))
 
 
-def _flash_attn_forward(q, k, v, logit_scale, bias=None, mask=None, scale_type="scalar", _scale_dim=0):
+def _flash_attn_forward(q, k, v, logit_scale, bias=None, mask=None, scale_type="scalar", _scale_dim=0, _events=None):
     """(o, lse, logit_scale) as the reference's launcher returns them (attn_kernel_forward.py:261-345):
     o like q, lse fp32 [BW, H, ceil(N / 64) * 64] holding the natural-log normaliser of every query row.
     A head dimension that is not a multiple of 8 runs on zero-padded copies (the reference pads inside its
     kernels, attn_kernel_forward.py:267,298): zero columns change neither the norms nor the products, and the
-    default scale keeps referring to the true dimension."""
+    default scale keeps referring to the true dimension.
+    `_events`: an optional pair of raw hipEvent_t handles that the library records on the stream around the
+    kernels of this call (a measurement hook without a counterpart in the reference)."""
     _check_inputs(q, k, v, logit_scale, bias, mask, scale_type)
     d = q.shape[-1]
     if d % 8:
-        o, lse, logit_scale = _flash_attn_forward(_pad8(q), _pad8(k), _pad8(v), logit_scale, bias, mask, scale_type, d)
+        o, lse, logit_scale = _flash_attn_forward(_pad8(q), _pad8(k), _pad8(v), logit_scale, bias, mask, scale_type, d,
+                                                  _events)
         return o[..., :d].contiguous(), lse, logit_scale
     q, k, v = (_kernel_ready(x) for x in (q, k, v))
     if scale_type == "tensor" and not logit_scale.is_contiguous():
@@ -241,6 +244,8 @@ def _flash_attn_forward(q, k, v, logit_scale, bias=None, mask=None, scale_type="
     if not _rows_16b_aligned(o):
         o = torch.empty(q.shape, device=q.device, dtype=q.dtype)
     p = _describe(q, k, v, o, lse, logit_scale, bias, mask, _flags_for(mask), scale_type, scale_dim=_scale_dim)
+    if _events is not None:
+        p.ev_start, p.ev_stop = _events
     with _on_device(q.device) as stream:
         p.stream = stream
         _abi.check(lib.fwa2_forward(p), "fwa2_forward")
@@ -248,9 +253,10 @@ def _flash_attn_forward(q, k, v, logit_scale, bias=None, mask=None, scale_type="
 
 
 def _flash_attn_backward(do, q, k, v, logit_scale, o, lse, dq, dk, dv, dscale, db, bias=None, mask=None,
-                         scale_type="scalar", _scale_dim=0):
+                         scale_type="scalar", _scale_dim=0, _events=None):
     """Fills dq, dk, dv (and dscale, db when given) in place, as the reference's launcher does
-    (attn_kernel_backward.py:567-711); dscale already carries the clamp mask (l <= ln 100)."""
+    (attn_kernel_backward.py:567-711); dscale already carries the clamp mask (l <= ln 100).
+    `_events`: an optional pair of raw hipEvent_t handles recorded around the main backward kernel of this call."""
     if q.shape[0] == 0:     # an empty batch: the sums over units are empty
         for t in (db, dscale):
             if t is not None:
@@ -261,7 +267,7 @@ def _flash_attn_backward(do, q, k, v, logit_scale, o, lse, dq, dk, dv, dscale, d
         padded = [_pad8(x) for x in (do, q, k, v, o)]
         grads = [torch.empty_like(padded[i]) for i in (1, 2, 3)]
         _flash_attn_backward(padded[0], padded[1], padded[2], padded[3], logit_scale, padded[4], lse, *grads, dscale, db,
-                             bias=bias, mask=mask, scale_type=scale_type, _scale_dim=d)
+                             bias=bias, mask=mask, scale_type=scale_type, _scale_dim=d, _events=_events)
         for given, used in zip((dq, dk, dv), grads):
             given.copy_(used[..., :d])
         return
@@ -285,6 +291,8 @@ def _flash_attn_backward(do, q, k, v, logit_scale, o, lse, dq, dk, dv, dscale, d
         p.dbias = db_k.data_ptr()
     if ds_k is not None and scale_type == "tensor":
         p.dscale = ds_k.data_ptr()
+    if _events is not None:
+        p.ev_start, p.ev_stop = _events
     with _on_device(q.device) as stream:
         need = lib.fwa2_backward_workspace_bytes(p)
         ws = torch.empty(max(need, 1), dtype=torch.uint8, device=q.device)

@@ -40,7 +40,7 @@
 extern "C" {
 #endif
 
-#define FWA2_ABI_VERSION 3
+#define FWA2_ABI_VERSION 4
 
 typedef enum fwa2_status {
     FWA2_OK = 0,
@@ -160,6 +160,16 @@ typedef struct fwa2_problem {
                                 as having region form is then computed from its record (N bytes) instead of its
                                 N x N mask entries, by the kernels for windows of up to 256 tokens at head
                                 dimension 32; everywhere else the record is ignored and the mask is read */
+
+    /*
+     * Optional measurement hook, no counterpart in the reference: two hipEvent_t handles (both or neither) that
+     * THIS call records on `stream`.  fwa2_forward records them around its kernels; fwa2_backward and
+     * fwa2_backward_static right before and after the main backward kernel (the table / transposing pre-pass and
+     * the partial-sum reduction stay outside), so a benchmark can time that kernel alone without a profiler.
+     * NULL = nothing is recorded.  The handles belong to the caller; nothing outlives the call.
+     */
+    void* ev_start;
+    void* ev_stop;
 } fwa2_problem;
 
 /* Library / ABI identification.  Returns FWA2_ABI_VERSION. */
@@ -281,16 +291,6 @@ int fwa2_cpb_bias_forward(const void* table, int dtype, int heads, int wh, int w
  */
 int fwa2_cpb_bias_backward(const void* table, const void* dbias, int dtype, int heads, int wh, int ww, void* dtable,
                            void* stream);
-
-/*
- * Measurement hook, no counterpart in the reference: when both are non-NULL the
- * next fwa2_backward calls (from any thread of the process) record the two hipEvent_t on the
- * problem's stream immediately before and after the main backward kernel (the
- * transposing pre-pass and the partial-sum reduction stay outside), so a
- * benchmark can time that kernel alone without a profiler.  Pass NULLs to
- * switch it off.
- */
-void fwa2_set_kernel_events(void* start_event, void* stop_event);
 
 #ifdef __cplusplus
 }

@@ -250,8 +250,8 @@ def test_problem_filled_the_way_a_binding_fills_it(lib):
                   q=t4(), k=t4(), v=t4(), o=t4(), logit_scale=0x10000, bias=t3(), mask=t3(), lse=0x10000,
                   lse_stride_bw=h * n, lse_stride_h=n, stream=None)
     p = _abi.Problem(abi_version=lib.fwa2_abi_version(), **fields)
-    assert lib.fwa2_abi_version() == 3
+    assert lib.fwa2_abi_version() == 4
     assert lib.fwa2_validate(ctypes.byref(p), 0) == _abi.OK, lib.fwa2_last_error()
     p = _abi.Problem(abi_version=1, **fields)
     assert lib.fwa2_validate(ctypes.byref(p), 0) == _abi.ERR_INVALID_ARGUMENT
-    assert b"abi 1, library 464 bytes / abi 3" in lib.fwa2_last_error()
+    assert b"abi 1, library 480 bytes / abi 4" in lib.fwa2_last_error()

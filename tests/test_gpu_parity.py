@@ -430,9 +430,13 @@ def test_full_benchmark_shapes(cfg):
         plain = {k: (None if v is None else v.detach()) for k, v in dev.items()}
     ref = _classic_on_gpu_fp32(plain, chunk=256 if cfg == "C3" else 1024)
     err = float((o.detach().float() - ref["o"]).abs().max())
-    assert err <= 2e-2, f"{cfg} forward max abs err {err}"
+    full = [("o", err)]
     for gname, tname in GRADS:
-        r = float((dev[tname].grad.float() - ref[gname]).abs().max() / ref[gname].abs().max())
+        full.append((gname, float((dev[tname].grad.float() - ref[gname]).abs().max() / ref[gname].abs().max())))
+    print(f"\n{cfg} at full size ({dev['q'].shape[0]} x {dev['q'].shape[1]} units): error against fp32 classic (bars 2e-2 on o, "
+          "5e-2 on the gradients): " + ", ".join(f"{n} {e:.2e}" for n, e in full))
+    assert err <= 2e-2, f"{cfg} forward max abs err {err}"
+    for gname, r in full[1:]:
         assert r <= 5e-2, f"{cfg} {gname} rel err {r}"
     # size-independent properties at full size: gradients orthogonal to q and k, dbias rows sum to 0
     qf, kf = dev["q"].detach().float(), dev["k"].detach().float()
