@@ -190,7 +190,7 @@ __global__ void __launch_bounds__(one256::NT) bwd_one_kernel(const BwdParams p) 
 
     const int h = blockIdx.x / p.groups;
     const int grp = blockIdx.x - h * p.groups;
-    const int N = p.n;
+    const int N = PLAIN ? R : p.n;      // whole 256-token windows: a compile-time constant
 
     // landing slots (block X & 1): 32 rows of q, dO, o as they are in memory, and their lse
     // (per slot: q, dO, o rows, 2 KB each, then 1 KB for the lse values: what wavefront w copies lands 2 KB x w

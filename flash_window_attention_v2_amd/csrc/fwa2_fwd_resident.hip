@@ -45,7 +45,9 @@ namespace fwa2 {
 // MAPPED: rows are addressed through the window map (cyclic shift + window partition done here).
 // SUB: 16-row query tiles per wavefront.  Two tiles share every K / V operand read from LDS and leave the
 // wavefront 256 registers, half as many wavefronts per workgroup.
-template <int DT, bool HAS_BIAS, int MASK_DT, int NT, bool VEC, bool MASKED, bool MAPPED, int SUB = 1>
+// FULL: the window has exactly 16 NT tokens (64, 128, 256), so the window length is a compile-time constant and
+// every bounds check, clamp and per-tile branch on it folds away.
+template <int DT, bool HAS_BIAS, int MASK_DT, int NT, bool VEC, bool MASKED, bool MAPPED, int SUB = 1, bool FULL = false>
 __global__ void __launch_bounds__(64 * NT / SUB) fwd_resident_kernel(const FwdParams p) {
     typedef typename Elem<DT>::E E;
     typedef typename Elem<DT>::V8 V8;
@@ -74,7 +76,10 @@ __global__ void __launch_bounds__(64 * NT / SUB) fwd_resident_kernel(const FwdPa
     __shared__ uint16_t lds_list[kLiveCache];      // windows of this launch's class, ascending
     __shared__ int lds_count;
 
-    const int N = p.n;
+    const int N = FULL ? 16 * NT : p.n;
+    // the per-group guards of the tile loops stay run-time tests even when N is a constant: they are what keeps
+    // the scheduler to one key group at a time (merged into one block, the groups' loads are hoisted and spill)
+    const int n_groups = p.n;
     const int tid = threadIdx.x;
     const int nthreads = blockDim.x;
     const int lane = tid & 63;
@@ -430,7 +435,7 @@ __global__ void __launch_bounds__(64 * NT / SUB) fwd_resident_kernel(const FwdPa
             if (use_fast) {
 #pragma unroll
                 for (int kp = 0; kp < NT / 2; kp++) {
-                    if (32 * kp < N) {
+                    if (32 * kp < n_groups) {
                         progress_priority(kp, NT / 2);
                         f32x4 s0[SUB], s1[SUB];
                         scores(kp, s0, s1, with_regions);
@@ -453,7 +458,7 @@ __global__ void __launch_bounds__(64 * NT / SUB) fwd_resident_kernel(const FwdPa
                 for (int u = 0; u < SUB; u++) bm[u] = -INFINITY;
 #pragma unroll
                 for (int kp = 0; kp < NT / 2; kp++) {
-                    if (32 * kp < N) {
+                    if (32 * kp < n_groups) {
                         f32x4 s0[SUB], s1[SUB];
                         scores(kp, s0, s1, with_regions);
 #pragma unroll
@@ -471,7 +476,7 @@ __global__ void __launch_bounds__(64 * NT / SUB) fwd_resident_kernel(const FwdPa
                 }
 #pragma unroll
                 for (int kp = 0; kp < NT / 2; kp++) {
-                    if (32 * kp < N) {
+                    if (32 * kp < n_groups) {
                         f32x4 s0[SUB], s1[SUB];
                         scores(kp, s0, s1, with_regions);
 #pragma unroll
@@ -530,15 +535,15 @@ constexpr int kRegionMaxImages = 32;     // images per window up to which region
 
 // SUBP: 16-row query tiles per wavefront in the launch over the unmasked units (the masked launch keeps one:
 // its tile rebuilds want the registers).
-template <int DT, bool HAS_BIAS, int MASK_DT, int NT, bool VEC, bool MAPPED, int SUBP>
+template <int DT, bool HAS_BIAS, int MASK_DT, int NT, bool VEC, bool MAPPED, int SUBP, bool FULL>
 static hipError_t launch_map(FwdParams p, hipStream_t st) {
     const int waves_plain = (p.n + 16 * SUBP - 1) / (16 * SUBP);
     const int waves_masked = (p.n + 15) / 16;
     // the runtime's figure is for full groups; smaller groups only fit better
     static std::atomic<int> fit_plain_by_device[kFitDevices], fit_masked_by_device[kFitDevices];
-    const int fit_plain = resident_per_cu_cached(fwd_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, false, MAPPED, SUBP>,
+    const int fit_plain = resident_per_cu_cached(fwd_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, false, MAPPED, SUBP, FULL>,
                                                  64 * NT / SUBP, fit_plain_by_device);
-    const int fit_masked = MASK_DT >= 0 ? resident_per_cu_cached(fwd_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, true, MAPPED, 1>,
+    const int fit_masked = MASK_DT >= 0 ? resident_per_cu_cached(fwd_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, true, MAPPED, 1, FULL>,
                                                                  64 * NT, fit_masked_by_device)
                                         : 1;
     auto groups_for = [&](int fit) {
@@ -555,13 +560,13 @@ static hipError_t launch_map(FwdParams p, hipStream_t st) {
     // units with an all-zero mask (or every unit when there is no mask) ...
     if (MASK_DT < 0 || p.mask_live != nullptr) {
         p.groups = groups_for(fit_plain);
-        hipLaunchKernelGGL((fwd_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, false, MAPPED, SUBP>), dim3(p.heads * p.groups),
+        hipLaunchKernelGGL((fwd_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, false, MAPPED, SUBP, FULL>), dim3(p.heads * p.groups),
                            dim3(64 * waves_plain), 0, st, p);
     }
     // ... and the units whose mask is live
     if (MASK_DT >= 0) {
         p.groups = groups_for(fit_masked);
-        hipLaunchKernelGGL((fwd_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, true, MAPPED, 1>), dim3(p.heads * p.groups),
+        hipLaunchKernelGGL((fwd_resident_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, true, MAPPED, 1, FULL>), dim3(p.heads * p.groups),
                            dim3(64 * waves_masked), 0, st, p);
     }
     return hipGetLastError();
@@ -570,8 +575,16 @@ static hipError_t launch_map(FwdParams p, hipStream_t st) {
 template <int DT, bool HAS_BIAS, int MASK_DT, int NT, bool VEC>
 static hipError_t launch_nt(const FwdParams& p, hipStream_t st) {
     constexpr int SUBP = NT == 16 ? kFwdSub : 1;       // the 256-token form; smaller tiles keep 16 rows per wavefront
-    if (p.map.nw > 0) return launch_map<DT, HAS_BIAS, MASK_DT, NT, VEC, true, SUBP>(p, st);
-    return launch_map<DT, HAS_BIAS, MASK_DT, NT, VEC, false, SUBP>(p, st);
+    // whole tiles of 16 tokens get the form with a compile-time window length; such windows have rows of a
+    // multiple of 8 entries, so they only exist with VEC
+    if constexpr (VEC) {
+        if (p.n == 16 * NT) {
+            if (p.map.nw > 0) return launch_map<DT, HAS_BIAS, MASK_DT, NT, VEC, true, SUBP, true>(p, st);
+            return launch_map<DT, HAS_BIAS, MASK_DT, NT, VEC, false, SUBP, true>(p, st);
+        }
+    }
+    if (p.map.nw > 0) return launch_map<DT, HAS_BIAS, MASK_DT, NT, VEC, true, SUBP, false>(p, st);
+    return launch_map<DT, HAS_BIAS, MASK_DT, NT, VEC, false, SUBP, false>(p, st);
 }
 
 template <int DT, bool HAS_BIAS, int MASK_DT>
