@@ -114,7 +114,7 @@ __device__ __forceinline__ void vm_store16_if_below(E* dst, V8 v, int idx, int l
     asm volatile("v_cmp_lt_i32 vcc, %3, %4\n\ts_and_saveexec_b64 %0, vcc\n\tglobal_store_dwordx4 %1, %2, off nt\n\ts_nop 1\n\ts_mov_b64 exec, %0"
                  : "=&s"(saved)
                  : "v"(dst), "v"(v), "v"(idx), "s"(limit)
-                 : "memory", "vcc");
+                 : "memory", "vcc", "scc");
 }
 __device__ __forceinline__ void vm_store4(float* dst, float v) {
     asm volatile("global_store_dword %0, %1, off" ::"v"(dst), "v"(v) : "memory");

@@ -130,7 +130,7 @@ __device__ __forceinline__ void vm_store16_if_below(E* dst, V8 v, int idx, int l
     asm volatile("v_cmp_lt_i32 vcc, %3, %4\n\ts_and_saveexec_b64 %0, vcc\n\tglobal_store_dwordx4 %1, %2, off nt\n\ts_nop 1\n\ts_mov_b64 exec, %0"
                  : "=&s"(saved)
                  : "v"(dst), "v"(v), "v"(idx), "s"(limit)
-                 : "memory", "vcc");
+                 : "memory", "vcc", "scc");
 }
 template <class V4, class E>
 __device__ __forceinline__ void vm_store8_if_below(E* dst, V4 v, int idx, int limit) {
@@ -138,21 +138,9 @@ __device__ __forceinline__ void vm_store8_if_below(E* dst, V4 v, int idx, int li
     asm volatile("v_cmp_lt_i32 vcc, %3, %4\n\ts_and_saveexec_b64 %0, vcc\n\tglobal_store_dwordx2 %1, %2, off nt\n\ts_nop 1\n\ts_mov_b64 exec, %0"
                  : "=&s"(saved)
                  : "v"(dst), "v"(v), "v"(idx), "s"(limit)
-                 : "memory", "vcc");
+                 : "memory", "vcc", "scc");
 }
 
-// 16 bytes per lane from base + voff (base: wavefront-uniform).  The result registers are only valid after a wait
-// that the caller places (tables_arrived below): the compiler neither sees the load nor waits for it.
-__device__ __forceinline__ f32x4 vm_load16(const float* base, uint32_t voff) {
-    f32x4 r;
-    asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(r) : "v"(voff), "s"(base) : "memory");
-    return r;
-}
-// At most `n` loads outstanding from here on; a and b (loaded earlier) may be used behind this point.
-template <int N_OUT>
-__device__ __forceinline__ void tables_arrived(f32x4& a, f32x4& b) {
-    asm volatile("s_waitcnt vmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N_OUT) : "memory");
-}
 // 16 bytes per lane at base + voff (base: wavefront-uniform); two wait states before the data registers may change
 template <class V8>
 __device__ __forceinline__ void vm_store16(void* base, uint32_t voff, V8 v) {
@@ -297,7 +285,7 @@ __global__ void __launch_bounds__(one256::NT) bwd_one_kernel(const BwdParams p) 
         const int slot = live ? p.heads + (b % p.n_windows) * p.heads + h : h;
         return p.tab + (int64_t)slot * (R * R) + ((wave * KT * NQB * 2) << 8);     // wavefront-uniform; the lane adds 4 * lane
     };
-    const uint32_t lane16 = 16u * (uint32_t)lane;
+    const int lane4 = 4 * lane;
 
     // Wavefront-uniform start of unit b inside a tensor whose head offset is already part of `base`.
     auto unit_start = [&](const char* base, int64_t sb, int b) -> const char* {
@@ -493,7 +481,7 @@ __global__ void __launch_bounds__(one256::NT) bwd_one_kernel(const BwdParams p) 
 #pragma unroll
             for (int kt = 0; kt < KT; kt++)
 #pragma unroll
-                for (int tt = 0; tt < 2; tt++) tb[kt][tt] = vm_load16(cur.tab + (((kt * NQB) * 2 + tt) << 8), lane16);
+                for (int tt = 0; tt < 2; tt++) tb[kt][tt] = *reinterpret_cast<const f32x4*>(cur.tab + lane4 + (((kt * NQB) * 2 + tt) << 8));
         }
         dma_block(source_of(cur.b), cur.b, 0, 0);
         dma_block(source_of(cur.b), cur.b, 1, 1);
@@ -653,10 +641,10 @@ __global__ void __launch_bounds__(one256::NT) bwd_one_kernel(const BwdParams p) 
 #pragma unroll
             for (int kt = 0; kt < KT; kt++) {
                 f32x4 sacc[2], pacc[2];
-                // The table values of this key tile were requested a block ago.  Loads return in order, and the
-                // loads issued since are the 6 of the other key tiles and the 2 row copies of this iteration (more
-                // where a unit began in between), so "at most 8 outstanding" covers them, whatever the stores do.
-                if (HAS_TAB) tables_arrived<8>(tb[kt][0], tb[kt][1]);
+                // (The table values of this key tile were requested a block ago by ordinary loads, which the compiler
+                // waits for by count.  They must stay ordinary loads: a load hidden in inline assembly delivers into
+                // registers the compiler believes written already, and it is free to move such a value elsewhere
+                // -- into an accumulator register, say -- before the data has arrived.)
 #pragma unroll
                 for (int tt = 0; tt < 2; tt++) {
                     // (S + bias + mask) * log2e with the table as the C operand; dP - delta
@@ -668,7 +656,7 @@ __global__ void __launch_bounds__(one256::NT) bwd_one_kernel(const BwdParams p) 
                 if (HAS_TAB) {
                     const float* src = qb + 1 < NQB ? tab + (((kt * NQB + qb + 1) * 2) << 8) : tab_next + (((kt * NQB) * 2) << 8);
 #pragma unroll
-                    for (int tt = 0; tt < 2; tt++) tb[kt][tt] = vm_load16(src + (tt << 8), lane16);
+                    for (int tt = 0; tt < 2; tt++) tb[kt][tt] = *reinterpret_cast<const f32x4*>(src + lane4 + (tt << 8));
                 }
                 if (kt == KT - 1) load_rows((qb + 1) & 7);
                 // the dbias accumulators of the last blocks come out of LDS: requested here, used behind the exponentials
