@@ -8,11 +8,14 @@ synthetic batch (benchmark configuration 3: B=64 images x 64 windows of N=256 to
 logit_scale = ln 10), inputs already resident in HBM.  One JSON line goes to
 stdout; progress goes to stderr.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extras | --basic-extras] [--sweep]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extras | --basic-extras]
+                    [--sweep [--sweep-n N ...]] [--copy-bytes B]
 
 `extras` carries the forward-only and N = 64 figures, peak memory, the window-size sweep of the reference's
 operator benchmark as HIP graph replays and one end-to-end model step; `--sweep` prints the sweep alone, with
-the eager timings beside the replays.
+the eager timings beside the replays (`--sweep-n`: only those window lengths, replays only, for a profiler);
+`--copy-bytes` adds a plain device copy of that size, timed, as the reference point for HBM counters and for the
+time the step's bytes would take at copy speed.
 """
 import argparse
 import ctypes
@@ -32,7 +35,7 @@ HBM_PEAK_GBS = 8000.0              # MI355X HBM3E
 # HBM bytes per launch of the backward kernel at the benchmark shape, from
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a copy kernel of known size
 # (profiles/kernels_C3_fwd_bwd.txt: FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0).
-BWD_KERNEL_TRAFFIC_BYTES = 1.630e9
+BWD_KERNEL_TRAFFIC_BYTES = 1.812e9
 # device memory the library holds on every GPU whether or not it is used (the scratch of fwa2_backward_static)
 STATIC_SCRATCH_MB = 128.0
 
@@ -276,6 +279,8 @@ def main():
                     help="extras without the window-size sweep and the model step (forward-only, N=64 and memory figures only)")
     ap.add_argument("--sweep", action="store_true",
                     help="instead of the benchmark line, print the window-size sweep (TFLOP/s versus N) as one JSON line")
+    ap.add_argument("--sweep-n", type=int, nargs="+", default=None,
+                    help="with --sweep: only these window lengths (tokens), graph replays only")
     ap.add_argument("--copy-bytes", type=int, default=0,
                     help="also run one plain device copy of this many bytes (reference point for HBM counters)")
     args = ap.parse_args()
@@ -292,7 +297,11 @@ def main():
     lib = _abi.load()
     torch.cuda.set_device(0)
     if args.sweep:
-        print(json.dumps(window_sweep(torch, min(args.steps, 30), min(args.warmup, 5))), flush=True)
+        if args.sweep_n:
+            out = window_sweep(torch, min(args.steps, 30), min(args.warmup, 5), eager=False, windows=tuple(args.sweep_n))
+        else:
+            out = window_sweep(torch, min(args.steps, 30), min(args.warmup, 5))
+        print(json.dumps(out), flush=True)
         return
 
     def setup(cfg):
@@ -440,6 +449,14 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
         result["copy_bytes"] = args.copy_bytes
+        # The same copy timed: what the HBM gives a kernel that only reads and writes (read + written bytes per second).
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(10):
+            dst.copy_(src)
+        e1.record()
+        torch.cuda.synchronize()
+        result["copy_gbs"] = round(2 * args.copy_bytes * 10 / e0.elapsed_time(e1) * 1e-6, 1)
         del src, dst
 
     if not args.no_cpu:

@@ -609,31 +609,38 @@ __global__ void __launch_bounds__(256) transpose_pad_kernel(const T* src, int64_
 }
 
 // dbias[h][q][k] = sum_g part[h][g][k][q]; dscale[h] = gate * sum_g part_dscale[h][g].
-// One workgroup per (32 queries, key row, head): 8 groups of 32 threads each sum every 8th partial
-// tile, then the 8 sums are added in a fixed order, so results are bit-reproducible.
+// A partial tile is npk x r floats, key-major; a workgroup sums 256 consecutive floats of it (64 lanes x 16 bytes:
+// every load of a wavefront is one contiguous KB) over the partial tiles of a head.  Each of its 4 wavefronts takes
+// every 4th tile, and the 4 sums are added in a fixed order, so results are bit-reproducible.
 template <int DT>
 __global__ void __launch_bounds__(256) reduce_kernel(const BwdParams p, int npk, int r, bool has_bias) {
     typedef typename Elem<DT>::E E;
-    __shared__ float part[8][32];
+    __shared__ f32x4 part[3][64];
     const int h = blockIdx.z;
-    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
     if (has_bias) {
-        const int q = blockIdx.x * 32 + tx, k = blockIdx.y;
-        float acc = 0.f;
-        const float* src = p.part_dbias + (((int64_t)h * p.db_parts) * npk + k) * r + q;
+        const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
         const int64_t gs = (int64_t)npk * r;
-#pragma unroll 4
-        for (int gi = ty; gi < p.db_parts; gi += 8) acc += src[gi * gs];
-        part[ty][tx] = acc;
+        const int64_t flat = 4 * ((int64_t)blockIdx.x * 64 + lane);
+        const float* src = p.part_dbias + ((int64_t)h * p.db_parts) * gs + flat;
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        if (flat < gs) {
+#pragma unroll 8
+            for (int gi = wave; gi < p.db_parts; gi += 4) acc += *reinterpret_cast<const f32x4*>(src + gi * gs);
+        }
+        if (wave) part[wave - 1][lane] = acc;
         __syncthreads();
-        if (ty == 0 && q < p.n && k < p.n) {
-            float tot = 0.f;
+        if (wave == 0 && flat < gs) {
+            acc = ((acc + part[0][lane]) + part[1][lane]) + part[2][lane];
+            const int k = (int)(flat / r), q = (int)(flat % r);
+            if (k < p.n) {
+                E* dst = reinterpret_cast<E*>(p.dbias) + ((int64_t)h * p.n + q) * p.n + k;
 #pragma unroll
-            for (int j = 0; j < 8; j++) tot += part[j][tx];
-            reinterpret_cast<E*>(p.dbias)[((int64_t)h * p.n + q) * p.n + k] = (E)tot;
+                for (int i = 0; i < 4; i++)
+                    if (q + i < p.n) dst[(int64_t)i * p.n] = (E)acc[i];
+            }
         }
     }
-    if (p.scale_kind == FWA2_SCALE_TENSOR && blockIdx.x == 0 && blockIdx.y == 0) {
+    if (p.scale_kind == FWA2_SCALE_TENSOR && blockIdx.x == 0) {
         float v = 0.f;
         for (int gi = threadIdx.x; gi < p.ds_parts; gi += 256) v += p.part_dscale[(int64_t)h * p.ds_parts + gi];
         __shared__ float red[256];
@@ -667,28 +674,16 @@ hipError_t launch_backward_fused(const BwdParams& p, int dtype, bool has_bias, i
 hipError_t launch_backward_dq_resident(const BwdParams& p, int dtype, bool has_bias, int mask_dt, hipStream_t st,
                                        int max_groups, int* ds_parts_out);
 
-// Largest set of score tables bwd_key_kernel may ask for (one 256 KB table per head and per (window, head) of a
-// masked call); calls beyond it stay on bwd_kernel, which streams bias and mask from key-major copies.
+// Largest set of score tables the one-pass kernel may ask for (one 256 KB table per head and per (window, head) of
+// a masked call); calls beyond it stay on bwd_kernel + the dq kernel, which stream bias and mask from key-major copies.
 constexpr size_t kTableBudget = (size_t)96 << 20;
 
-hipError_t launch_backward_key(const BwdParams& p, int dtype, bool has_bias, int mask_dt, hipStream_t st, int max_groups,
-                               int* groups_out);
 hipError_t launch_backward_one(const BwdParams& p, int dtype, bool has_bias, int mask_dt, hipStream_t st, int max_groups,
                                int* groups_out);
-#if FWA2_HALF != 2
-// FWA2_BWD_TWO_PASS=1 in the environment keeps windows of 161 .. 256 tokens on the key-side + query-side pair of
-// kernels instead of the one-pass kernel (read once per process; for comparing the two).
-bool backward_two_pass() {
-    static const bool two = [] { const char* e = getenv("FWA2_BWD_TWO_PASS"); return e && e[0] == '1'; }();
-    return two;
-}
-#else
-bool backward_two_pass();
-#endif
 
 struct BwdPlan {
     int waves, groups, npk, r, nqb_t, kt, dq_waves, dq_chunks, ds_parts, dq_max_groups;
-    bool key256;    // 161 .. 256 tokens: bwd_key_kernel (fwa2_bwd_key.hip) is the key-side kernel
+    bool one_pass;  // 161 .. 256 tokens: bwd_one_kernel (fwa2_bwd_one.hip) is the whole backward
     size_t off_tab;
     int n_chunks;   // > 1: windows of more than 256 tokens, cut into 256 x 256 or 192 x 192 super-tiles
     size_t off_dbias, off_dscale, off_bias_t, off_mask_t, off_delta, off_dk, off_dv, total;
@@ -699,7 +694,7 @@ static BwdPlan make_plan(int heads, int n, int bw, bool has_bias, bool has_mask,
     BwdPlan pl;
     const int nqb = (n + 31) / 32;
     pl.n_chunks = (n + 255) / 256;
-    pl.key256 = false;
+    pl.one_pass = false;
     int wg_per_cu;
     if (pl.n_chunks > 1) {
         // every workgroup is a full super-tile kernel of 256 x 256, or of 192 x 192 where that pads the
@@ -727,7 +722,7 @@ static BwdPlan make_plan(int heads, int n, int bw, bool has_bias, bool has_mask,
         const size_t slots = (size_t)heads * (1 + (has_mask ? n_windows : 0));
         if (pl.nqb_t == 8 && slots * 256 * 256 * 4 <= kTableBudget) {
             // four wavefronts of four key tiles on 256 x 256 tiles whatever the window length
-            pl.key256 = true;
+            pl.one_pass = true;
             pl.kt = 4;
             pl.waves = 4;
             pl.npk = 256;
@@ -739,8 +734,8 @@ static BwdPlan make_plan(int heads, int n, int bw, bool has_bias, bool has_mask,
     pl.groups = groups;
     size_t off = 0;
     pl.off_dbias = off;
-    // one partial tile per workgroup and launch: two launches (masked / unmasked units) except for bwd_key_kernel
-    if (has_bias) off += align256((size_t)heads * (pl.key256 ? 1 : 2) * groups * pl.npk * pl.r * 4);
+    // one partial tile per workgroup and launch: two launches (masked / unmasked units) except for the one-pass kernel
+    if (has_bias) off += align256((size_t)heads * (pl.one_pass ? 1 : 2) * groups * pl.npk * pl.r * 4);
     dq_geometry(n, &pl.dq_waves, &pl.dq_chunks);
     pl.ds_parts = bw * pl.dq_chunks;
     // the resident dq kernel writes one partial per workgroup: at most this many per head and launch
@@ -750,17 +745,17 @@ static BwdPlan make_plan(int heads, int n, int bw, bool has_bias, bool has_mask,
     pl.off_dscale = off;
     off += align256((size_t)heads * ds_slots * 4);
     pl.off_delta = off;
-    if (pl.n_chunks == 1) off += align256((size_t)bw * heads * pl.r * 4);
+    if (pl.n_chunks == 1 && !pl.one_pass) off += align256((size_t)bw * heads * pl.r * 4);
     pl.off_dk = off;
     if (pl.n_chunks > 1) off += align256((size_t)pl.n_chunks * bw * heads * pl.npk * 32 * 4);
     pl.off_dv = off;
     if (pl.n_chunks > 1) off += align256((size_t)pl.n_chunks * bw * heads * pl.npk * 32 * 4);
     pl.off_bias_t = off;
-    if (has_bias && !pl.key256) off += align256((size_t)heads * pl.npk * pl.r * 2);
+    if (has_bias && !pl.one_pass) off += align256((size_t)heads * pl.npk * pl.r * 2);
     pl.off_mask_t = off;
-    if (has_mask && !pl.key256) off += align256((size_t)n_windows * pl.npk * pl.r * 4);
+    if (has_mask && !pl.one_pass) off += align256((size_t)n_windows * pl.npk * pl.r * 4);
     pl.off_tab = off;
-    if (pl.key256) off += align256((size_t)heads * (1 + (has_mask ? n_windows : 0)) * 256 * 256 * 4);
+    if (pl.one_pass) off += align256((size_t)heads * (1 + (has_mask ? n_windows : 0)) * 256 * 256 * 4);
     pl.total = off;
     pl.smem = 0;   // the kernels use static LDS
     return pl;
@@ -869,7 +864,7 @@ static hipError_t launch_bwd_dt(BwdParams p, bool has_bias, int mask_dt, hipStre
         p.db_parts = parts;
         p.ds_parts = parts;
         if (has_bias || p.scale_kind == FWA2_SCALE_TENSOR) {
-            dim3 gr(has_bias ? pl.r / 32 : 1, has_bias ? pl.npk : 1, p.heads);
+            dim3 gr(has_bias ? (pl.npk * pl.r + 255) / 256 : 1, 1, p.heads);
             hipLaunchKernelGGL(reduce_kernel<DT>, gr, dim3(256), 0, st, p, pl.npk, pl.r, has_bias);
             ef = hipGetLastError();
         }
@@ -877,13 +872,13 @@ static hipError_t launch_bwd_dt(BwdParams p, bool has_bias, int mask_dt, hipStre
     }
     p.tab = reinterpret_cast<const float*>(ws + pl.off_tab);
     const dim3 tgrid(pl.r / 32, (pl.npk + 31) / 32, 1);
-    if (has_bias && !pl.key256) {
+    if (has_bias && !pl.one_pass) {
         dim3 gr(tgrid.x, tgrid.y, p.heads);
         hipLaunchKernelGGL(transpose_pad_kernel<E>, gr, dim3(256), 0, st, reinterpret_cast<const E*>(p.bias), p.bias_sh,
                            p.bias_sn, p.n, pl.npk, pl.r, (const uint8_t*)nullptr,
                            reinterpret_cast<E*>(const_cast<void*>(p.bias_t)), -INFINITY);
     }
-    if (mask_dt >= 0 && !pl.key256) {
+    if (mask_dt >= 0 && !pl.one_pass) {
         dim3 gr(tgrid.x, tgrid.y, p.n_windows);
         if (mask_dt == FWA2_F32)
             hipLaunchKernelGGL(transpose_pad_kernel<float>, gr, dim3(256), 0, st, reinterpret_cast<const float*>(p.mask),
@@ -897,23 +892,20 @@ static hipError_t launch_bwd_dt(BwdParams p, bool has_bias, int mask_dt, hipStre
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     int gr_out[2] = {pl.groups, pl.groups};
-    const bool one_pass = pl.key256 && !backward_two_pass();
-    if (one_pass) {
+    if (pl.one_pass) {
         e = launch_backward_one(p, DT, has_bias, mask_dt, st, pl.groups, gr_out);
         if (e != hipSuccess) return e;
         p.groups = gr_out[0];
         p.db_parts = gr_out[1];
         p.ds_parts = gr_out[0];
         if (has_bias || p.scale_kind == FWA2_SCALE_TENSOR) {
-            dim3 gr(has_bias ? pl.r / 32 : 1, has_bias ? pl.npk : 1, p.heads);
+            dim3 gr(has_bias ? (pl.npk * pl.r + 255) / 256 : 1, 1, p.heads);
             hipLaunchKernelGGL(reduce_kernel<DT>, gr, dim3(256), 0, st, p, pl.npk, pl.r, has_bias);
             e = hipGetLastError();
         }
         return e;
     }
-    if (pl.key256) {
-        e = launch_backward_key(p, DT, has_bias, mask_dt, st, pl.groups, gr_out);
-    } else if (has_bias) {
+    if (has_bias) {
         if (mask_dt < 0) e = launch_nqb<DT, true, -1>(p, pl, st, gr_out);
         else if (mask_dt == FWA2_F32) e = launch_nqb<DT, true, FWA2_F32>(p, pl, st, gr_out);
         else e = launch_nqb<DT, true, DT>(p, pl, st, gr_out);
@@ -935,7 +927,7 @@ static hipError_t launch_bwd_dt(BwdParams p, bool has_bias, int mask_dt, hipStre
     }
     if (e != hipSuccess) return e;
     if (has_bias || p.scale_kind == FWA2_SCALE_TENSOR) {
-        dim3 gr(has_bias ? pl.r / 32 : 1, has_bias ? pl.npk : 1, p.heads);
+        dim3 gr(has_bias ? (pl.npk * pl.r + 255) / 256 : 1, 1, p.heads);
         hipLaunchKernelGGL(reduce_kernel<DT>, gr, dim3(256), 0, st, p, pl.npk, pl.r, has_bias);
         e = hipGetLastError();
     }

@@ -5,14 +5,22 @@
 // (flash_win_attn_v2/kernels/attn_kernel_backward.py:6-51, 84-353), which also recomputes every score once
 // (:246-336) but sums dq and dbias with fp32 atomics; here nothing is atomic and every sum has a fixed order.
 //
-// One workgroup of four wavefronts (one per SIMD, 512 registers each) is persistent for one head and keeps the
-// head's whole dbias tile in accumulator registers, as bwd_key_kernel does: every wavefront owns 64 keys and the
-// queries stream past them in blocks of 32.  What is new is that the blocks are a software pipeline over ALL the
-// units the workgroup walks, with one barrier per block and no per-unit staging phase:
+// One workgroup of four wavefronts (one per SIMD, 512 registers each) is persistent for one head, walks over many
+// (batch*window) units and keeps the head's whole dbias tile on chip: every wavefront owns 64 keys (four MFMA tiles
+// of 16) and the unit's queries stream past them in blocks of 32.  The dbias accumulators of a lane (256 floats)
+// sit in AGPRs, the last quarter of them in LDS, and are only ever touched by the matrix pipe (dbias += I * dZ, an
+// MFMA against a one-hot operand).  Bias and mask come as ONE fp32 table per head (per (window, head) where the
+// window's mask is live; fwa2_score_tables.hip) that holds (bias + mask) * log2e in the order of the score
+// accumulators, so the values of a block are loaded straight into the C operand of S = Q_hat K_hat^T, one block
+// ahead, into the registers the running block has just read; masked and unmasked units run the same code in one
+// launch.  Per score the VALU does: add -lse, exp2, multiply by (dP - delta), two half conversions.
+//
+// The blocks are a software pipeline over ALL the units the workgroup walks, with one barrier per block and no
+// per-unit staging phase:
 //
 //   iteration of block X:   rows of block X+3      global memory -> landing slot (global_load_lds, 2 slots)
 //                           block X+2              landing slot -> tiles (q_hat s log2e, dO, -delta, -lse log2e, 1/|q|; 4 slots)
-//                           block X                S, dP, exp2, dZ, dbias, dV, dK_hat as in bwd_key_kernel; the
+//                           block X                S, dP, exp2, dZ, dbias, dV, dK_hat against the wavefront's keys; the
 //                                                  wavefront's dZ (32 queries x 64 keys, fp16) also goes to its own
 //                                                  LDS slab and comes back transposed (ds_read_b64_tr_b16) as the
 //                                                  B operand of dQ_hat^T += K_hat^T dZ^T over its 64 keys
@@ -35,7 +43,7 @@
 
 namespace fwa2 {
 
-hipError_t launch_key_tables(const BwdParams& p, int dtype, bool has_bias, int mask_dt, hipStream_t st);
+hipError_t launch_score_tables(const BwdParams& p, int dtype, bool has_bias, int mask_dt, hipStream_t st);
 
 namespace one256 {
 
@@ -45,7 +53,12 @@ constexpr int NQB = 8;        // query blocks of 32
 constexpr int KT = 4;         // key tiles of 16 per wavefront
 constexpr int WAVES = 4;
 constexpr int NT = 64 * WAVES;
-constexpr int kLdsQb = 2;     // query blocks whose dbias accumulators live in LDS (see bwd_key_kernel)
+// The 256 dbias accumulators of a lane are exactly the AGPR file, and the compiler needs a few AGPRs of its own (what
+// it cannot hold in 256 VGPRs, it parks there with a register move; without room it spills to scratch, and a scratch
+// reload queues behind every fetch in flight).  The accumulators of the last query blocks therefore live in LDS, in
+// a private 16-byte slot per lane, and visit registers once per unit (two blocks: with one, some instantiations
+// still spill).
+constexpr int kLdsQb = 2;
 __host__ __device__ constexpr bool db_in_lds(int qb) { return qb >= NQB - kLdsQb; }
 constexpr int kLive = 256;    // windows whose mask flags are listed in LDS (more: every window counts as live)
 constexpr int kLandE = 3 * 32 * 32 + 512;   // elements of a landing slot: three tensors' rows and 1 KB for lse
@@ -105,7 +118,8 @@ __device__ __forceinline__ float oct_add(float x) {
     return x + y;
 }
 
-// Vector-memory instructions the compiler's wait-count bookkeeping must not see (see bwd_key_kernel): the copies
+// Vector-memory instructions the compiler's wait-count bookkeeping must not see (it would guard every LDS read it
+// cannot tell from the copies' targets with a wait for all of them): the copies
 // into LDS and the output stores are issued from inline assembly, and whoever reads what the copies wrote waits
 // with an explicit s_waitcnt.  Loads return in order, so "at most n loads outstanding" means everything older
 // than the youngest n loads has arrived; outstanding stores only make such a wait stricter.
@@ -824,7 +838,7 @@ static hipError_t launch_one_dt(const BwdParams& p, bool has_bias, int mask_dt, 
     const bool masked = mask_dt >= 0;
     const bool has_tab = has_bias || masked || p.n < one256::R;
     const bool mapped = p.map.nw > 0;
-    hipError_t e = launch_key_tables(p, DT, has_bias, mask_dt, st);
+    hipError_t e = launch_score_tables(p, DT, has_bias, mask_dt, st);
     if (e != hipSuccess) return e;
     if (p.ev_start) (void)hipEventRecord(p.ev_start, st);
 #define FWA2_ONE_CASE(B, T, M)                                                                                       \

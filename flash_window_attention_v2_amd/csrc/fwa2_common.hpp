@@ -481,7 +481,7 @@ struct BwdParams {
     bool side_vec_rows;  // ... or n % 8 != 0 but every row is at least n rounded up to 8 entries long (resident kernels)
     const void* bias_t;  // [H, NP, NQ] input dtype: bias transposed to key-major, zero padded
     const void* mask_t;  // [nW, NP, NQ] mask dtype: mask transposed to key-major, zero padded
-    const float* tab;    // table mode of the key-side kernel: (bias + mask) * log2e in accumulator order, slot h for
+    const float* tab;    // score tables of the one-pass kernel: (bias + mask) * log2e in accumulator order, slot h for
                          // head h alone and slot heads + w * heads + h for window w with a live mask
 };
 

@@ -54,7 +54,7 @@ CASES = [
     (1, (12, 8), (4, 4), (1, 3), 4, True),
     (2, (8, 8), (8, 8), (0, 0), 3, False),          # one window covers the grid
     (2, (6, 9), (3, 3), (1, 1), 2, True),           # 9 tokens
-    (2, (32, 32), (16, 16), (8, 8), 3, True),       # 256 tokens: forward, dq and key-side kernels
+    (2, (32, 32), (16, 16), (8, 8), 3, True),       # 256 tokens: forward and one-pass backward kernels
     (2, (32, 16), (16, 16), (0, 0), 3, False),
     (2, (24, 36), (12, 12), (6, 6), 3, True),       # 144 tokens: one 16-key tile per wavefront
     (1, (20, 40), (10, 20), (5, 10), 2, True),      # 200 tokens, not a multiple of 16

@@ -137,7 +137,7 @@ def test_more_windows_than_the_flag_cache_and_no_flags(monkeypatch):
 
 
 def test_more_windows_than_the_key_side_kernel_lists():
-    """Windows of 161 .. 256 tokens with more windows than the key-side backward lists in LDS (256) and one
+    """Windows of 161 .. 256 tokens with more windows than the one-pass backward lists in LDS (256) and one
     head, so that the score tables still fit the table budget: every window then counts as live in that kernel
     and the table of a window whose mask is all zero must have been built too (dk, dv, dbias read it)."""
     n_w, n = 260, 192
