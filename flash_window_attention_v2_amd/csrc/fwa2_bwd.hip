@@ -580,8 +580,9 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
                     f32x4 a, c;
 #pragma unroll
                     for (int j = 0; j < 4; j++) { a[j] = w.dbacc[qb][kt][j]; c[j] = w.dbacc[qb][kt][4 + j]; }
-                    __builtin_nontemporal_store(a, reinterpret_cast<f32x4*>(dst + 32 * qb + 8 * g));
-                    __builtin_nontemporal_store(c, reinterpret_cast<f32x4*>(dst + 32 * qb + 8 * g + 4));
+                    // (plain stores: the reduction that follows then finds the tiles in the memory-side cache)
+                    *reinterpret_cast<f32x4*>(dst + 32 * qb + 8 * g) = a;
+                    *reinterpret_cast<f32x4*>(dst + 32 * qb + 8 * g + 4) = c;
                 }
             }
         }

@@ -810,7 +810,8 @@ __global__ void __launch_bounds__(one256::NT) bwd_one_kernel(const BwdParams p) 
                     const f32x4 acc = db_in_lds(qb) ? *reinterpret_cast<const f32x4*>(
                                                           lds_db + ((((qb - (NQB - kLdsQb)) * KT + kt) * 2 + hf) * NT + tid) * 4)
                                                     : dbq[qb][kt][hf];
-                    __builtin_nontemporal_store(acc, reinterpret_cast<f32x4*>(dst + 32 * qb + 16 * hf + 4 * g));
+                    // (a plain store: the reduction that follows then finds the tiles in the memory-side cache)
+                    *reinterpret_cast<f32x4*>(dst + 32 * qb + 16 * hf + 4 * g) = acc;
                 }
         }
     }

@@ -84,9 +84,14 @@ __device__ __forceinline__ V8 ld8(const E* p) { return *reinterpret_cast<const V
 template <class V8, class E>
 __device__ __forceinline__ void st8(E* p, V8 v) { *reinterpret_cast<V8*>(p) = v; }
 
-// 16-byte store of an output row chunk that nobody re-reads soon: non-temporal, like the row fetches.
-template <class V8, class E>
-__device__ __forceinline__ void st8_stream(E* p, V8 v) { __builtin_nontemporal_store(v, reinterpret_cast<V8*>(p)); }
+// 16-byte store of an output row chunk that nobody re-reads soon: non-temporal, like the row fetches.  (STREAM =
+// false: a plain store, for kernels whose whole problem fits the memory-side cache often enough that the next
+// kernel finds the rows there.)
+template <class V8, class E, bool STREAM = true>
+__device__ __forceinline__ void st8_stream(E* p, V8 v) {
+    if (STREAM) __builtin_nontemporal_store(v, reinterpret_cast<V8*>(p));
+    else *reinterpret_cast<V8*>(p) = v;
+}
 
 template <class V8>
 __device__ __forceinline__ V8 zero8() {

@@ -16,48 +16,39 @@ constexpr int kTableLive = 256;     // windows whose mask flags the backward lis
 // tab[slot][key tile j][query block qb][t][lane][i] = (bias[h][q][key] + mask[w][q][key]) * log2e with key = 16 j +
 // lane % 16 and q = 32 qb + 8 (lane / 16) + 4 t + i; -inf for padded keys, 0 for padded queries.  Slot h < heads: the
 // bias of head h alone; slot heads + w * heads + h: with the mask of window w (built only for windows whose mask is
-// live; every window without flags).  One workgroup per (query block, slot): the 32 rows are read a row at a time
-// (consecutive lanes, consecutive keys), summed into an LDS tile, and written out in table order, 16 bytes a lane.
+// live; every window without flags).  One thread per 16 bytes of table: eight independent 2-byte loads (16 lanes read
+// 32 consecutive bytes of a row), one 16-byte store.  (A form that reads whole rows through an LDS tile, one workgroup
+// per query block and slot, has too few workgroups in flight and measured twice as slow.)
 template <class E, class ME>
 __global__ void __launch_bounds__(256) build_table_kernel(const E* bias, int64_t bias_sh, int64_t bias_sn, const ME* mask,
                                                           int64_t mask_sw, int64_t mask_sn, const uint8_t* live, int n,
                                                           int heads, float* tab) {
-    __shared__ float tile[32][kTableRows + 1];
-    const int slot = blockIdx.y, qb = blockIdx.x;
+    const int slot = blockIdx.y;
     int h = slot, wnd = -1;
     if (slot >= heads) {
         wnd = (slot - heads) / heads;
         h = (slot - heads) - wnd * heads;
         if (live && !live[wnd]) return;
     }
-    const int key = threadIdx.x;
-    const E* bcol = bias ? bias + h * bias_sh + key : nullptr;
-    const ME* mcol = wnd >= 0 ? mask + wnd * mask_sw + key : nullptr;
-#pragma unroll 8
-    for (int r = 0; r < 32; r++) {
-        const int q = 32 * qb + r;
+    const int idx = blockIdx.x * 256 + threadIdx.x;        // (j, qb, t, lane)
+    const int lane = idx & 63, t = (idx >> 6) & 1, rest = idx >> 7;
+    const int qb = rest % kTableBlocks, j = rest / kTableBlocks;
+    const int key = 16 * j + (lane & 15), q0 = 32 * qb + 8 * (lane >> 4) + 4 * t;
+    f32x4 v;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int q = q0 + i;
         float x = 0.f;
         if (key >= n) {
             x = -INFINITY;
         } else if (q < n) {
-            if (bcol) x = (float)bcol[(int64_t)q * bias_sn];
-            if (mcol) x += (float)mcol[(int64_t)q * mask_sn];
+            if (bias) x = (float)bias[h * bias_sh + (int64_t)q * bias_sn + key];
+            if (wnd >= 0) x += (float)mask[wnd * mask_sw + (int64_t)q * mask_sn + key];
             x *= kLog2e;
         }
-        tile[r][key] = x;
+        v[i] = x;
     }
-    __syncthreads();
-    float* dst = tab + (int64_t)slot * (kTableRows * kTableRows);
-#pragma unroll
-    for (int it = 0; it < 8; it++) {
-        const int idx = it * 256 + threadIdx.x;          // (j, t, lane)
-        const int lane = idx & 63, t = (idx >> 6) & 1, j = idx >> 7;
-        const int col = 16 * j + (lane & 15), r0 = 8 * (lane >> 4) + 4 * t;
-        f32x4 v;
-#pragma unroll
-        for (int i = 0; i < 4; i++) v[i] = tile[r0 + i][col];
-        *reinterpret_cast<f32x4*>(dst + ((int64_t)((j * kTableBlocks + qb) * 2 + t) * 64 + lane) * 4) = v;
-    }
+    *reinterpret_cast<f32x4*>(tab + (int64_t)slot * (kTableRows * kTableRows) + (int64_t)idx * 4) = v;
 }
 
 template <int DT>
@@ -67,7 +58,7 @@ static hipError_t build_tables(const BwdParams& p, bool has_bias, int mask_dt, h
     const bool has_tab = has_bias || masked || p.n < kTableRows;
     if (!has_tab) return hipSuccess;
     const int slots = p.heads * (1 + (masked ? p.n_windows : 0));
-    const dim3 gr(kTableBlocks, slots);
+    const dim3 gr(kTableRows * kTableRows / 4 / 256, slots);
     float* tab = const_cast<float*>(p.tab);
     const E* bias = has_bias ? reinterpret_cast<const E*>(p.bias) : nullptr;
     // The backward lists the flags of up to kTableLive windows; with more it treats every window as live and reads
