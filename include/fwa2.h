@@ -252,11 +252,12 @@ int fwa2_backward(const fwa2_problem* p);
  * Has no counterpart in the reference (whose launcher allocates dq_accum, db_accum, dscale_accum and delta with
  * torch on every call, attn_kernel_backward.py:582-626).
  *   - a problem whose fwa2_backward_workspace_bytes() exceeds FWA2_STATIC_SCRATCH_BYTES is refused with
- *     FWA2_ERR_UNSUPPORTED.  The need grows with the batch (one fp32 delta value per query row), with the
- *     device's compute-unit count (one N x N fp32 dbias tile per persistent workgroup) and, for windows of 161
- *     to 256 tokens with a mask, with the number of windows per image (one N x N fp32 table slot per window and
- *     head): 3 heads of 256-token windows with a 64-window mask need 124.5 MiB at 4 096 windows per call (the
- *     reference's benchmark shape; fits), 80 MiB with a 16-window mask at 1 024 windows per call, 36 MiB for
+ *     FWA2_ERR_UNSUPPORTED.  The need grows with the batch (one fp32 delta value per query row, except for
+ *     windows of 161 to 256 tokens, whose delta never leaves the chip), with the device's compute-unit count
+ *     (one N x N fp32 dbias tile per persistent workgroup) and, for windows of 161 to 256 tokens with a mask,
+ *     with the number of windows per image (one N x N fp32 table slot per window and head): 3 heads of
+ *     256-token windows with a 64-window mask need 112.5 MiB whatever the batch (the reference's benchmark
+ *     shape; fits), 76.5 MiB with a 16-window mask, 36 MiB for
  *     64-token windows at 4 096 per call; windows of 576 tokens and more need their fp32 dk / dv partials here
  *     too (0.7 GiB at 256 windows of 6 heads) and do not fit: use fwa2_backward there;
  *   - the device that is current at the call must be the one the tensors and the stream belong to; the address

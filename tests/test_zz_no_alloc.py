@@ -64,7 +64,7 @@ def _case(lib, batch, n_windows, heads, n, resolution, window, shift, dtype, see
 def test_static_scratch_backward_matches_workspace_backward_twice():
     lib = _abi.load()
     # first windows of 256 tokens with a 16-window mask (the one-pass backward with its score tables; about
-    # 80 MiB of scratch on a 256-CU part) ...
+    # 77 MiB of scratch on a 256-CU part) ...
     _case(lib, batch=4, n_windows=16, heads=3, n=256, resolution=64, window=16, shift=8, dtype=torch.bfloat16, seed=11)
     # ... then a smaller problem on the fused kernel, which finds the first call's leftovers in the scratch
     _case(lib, batch=2, n_windows=4, heads=2, n=64, resolution=16, window=8, shift=4, dtype=torch.float16, seed=12)
