@@ -363,7 +363,7 @@ def main():
                 "gbs": round(nbytes / avg * 1e-6, 1), "frac_hbm_peak": round(nbytes / avg * 1e-6 / HBM_PEAK_GBS, 4)}
 
     kernels = [
-        kernel_row("forward: fwd_resident_kernel, unmasked + masked launch", fwd_kern_ms,
+        kernel_row("forward: fwd_resident_kernel (masked and unmasked units in one launch)", fwd_kern_ms,
                    flops_matmul(bw, cfg["heads"], cfg["n"], cfg["d"], bwd=False),
                    bytes_min(bw, cfg["heads"], cfg["n"], cfg["d"], cfg["n_windows"], bwd=False)),
         kernel_row("backward: bwd_one_kernel (dq, dk, dv, dbias partials, dlogit_scale terms in one pass)", bwd_kern_ms,
