@@ -25,9 +25,12 @@
 
 namespace fwa2 {
 
+// The walk of one workgroup (head h, workgroup grp of the `groups` its class of windows has for that head) over its
+// units; its dbias tile and dscale partial go to slot `slot` of the head.
+// MASKED: the class of windows whose mask is live (the resident tile then holds bias + the window's mask).
 // MAPPED: rows are addressed through the window map (cyclic shift + window partition done here).
 template <int DT, bool HAS_BIAS, int MASK_DT, int NT, bool VEC, bool MASKED, bool MAPPED>
-__global__ void __launch_bounds__(64 * NT, 3) bwd_fused_kernel(const BwdParams p) {
+__device__ __forceinline__ void bwd_fused_body(const BwdParams& p, const int h, const int grp, const int groups, const int slot) {
     typedef typename Elem<DT>::E E;
     typedef typename Elem<DT>::V8 V8;
     typedef typename Elem<DT>::V4 V4;
@@ -39,17 +42,18 @@ __global__ void __launch_bounds__(64 * NT, 3) bwd_fused_kernel(const BwdParams p
     constexpr int S = kLdsStride;         // row stride of the 32-column tiles
     constexpr int PS = ROWS + 8;          // row stride of the [query][key] tiles
 
-    __shared__ __attribute__((aligned(16))) SE lds_K[ROWS * S];        // k_hat of the current unit
-    __shared__ __attribute__((aligned(16))) E lds_V[ROWS * S];
-    __shared__ __attribute__((aligned(16))) float lds_kinv[ROWS];      // 1 / max(|k|, eps), negated when |k| <= eps
-    __shared__ __attribute__((aligned(16))) SE lds_Qs[ROWS * S];       // q_hat s log2e of the current unit
-    __shared__ __attribute__((aligned(16))) E lds_dOs[ROWS * S];       // dO (times w when folded) of the current unit
-    __shared__ __attribute__((aligned(16))) E lds_Pt[ROWS * PS];       // e,  [query][key]
-    __shared__ __attribute__((aligned(16))) SE lds_Zt[ROWS * PS];      // dZ, [query][key]
-    __shared__ uint8_t lds_live[kLiveCache];
-    __shared__ uint16_t lds_list[kLiveCache];
-    __shared__ int lds_count;
-    __shared__ float lds_red[NT];
+    // (arrays shared by the two bodies a kernel may run, one per class of windows)
+    SE* lds_K = shared_array<SE, ROWS * S, 0>();           // k_hat of the current unit
+    E* lds_V = shared_array<E, ROWS * S, 1>();
+    float* lds_kinv = shared_array<float, ROWS, 2>();      // 1 / max(|k|, eps), negated when |k| <= eps
+    SE* lds_Qs = shared_array<SE, ROWS * S, 3>();          // q_hat s log2e of the current unit
+    E* lds_dOs = shared_array<E, ROWS * S, 4>();           // dO (times w when folded) of the current unit
+    E* lds_Pt = shared_array<E, ROWS * PS, 5>();           // e,  [query][key]
+    SE* lds_Zt = shared_array<SE, ROWS * PS, 6>();         // dZ, [query][key]
+    uint8_t* lds_live = shared_array<uint8_t, kLiveCache, 7>();
+    uint16_t* lds_list = shared_array<uint16_t, kLiveCache, 8>();
+    int& lds_count = *shared_array<int, 4, 9>();
+    float* lds_red = shared_array<float, NT, 10>();
 
     const int N = p.n;
     const int tid = threadIdx.x;
@@ -58,10 +62,6 @@ __global__ void __launch_bounds__(64 * NT, 3) bwd_fused_kernel(const BwdParams p
     const int wave = tid >> 6;
     const int l16 = lane & 15;
     const int g = lane >> 4;
-
-    const int groups = p.dq_groups;
-    const int h = blockIdx.x / groups;
-    const int grp = blockIdx.x - h * groups;
 
     float s_true;
     if (p.scale_kind == FWA2_SCALE_TENSOR) {
@@ -148,30 +148,25 @@ __global__ void __launch_bounds__(64 * NT, 3) bwd_fused_kernel(const BwdParams p
     auto window_at = [&](int wi) -> int {
         return listed ? __builtin_amdgcn_readfirstlane((int)lds_list[wi]) : wi;
     };
-    int wi_step = 1, img0 = 0, img_step = 1, wi0 = grp;
-    if (MASKED) {
-        if (groups >= cnt && cnt > 0) {
-            const int per = groups / cnt;         // workgroups per window
-            wi0 = grp / per;                      // (>= cnt for the few left over: they idle)
-            img0 = grp - wi0 * per;
-            img_step = per;
-            wi_step = cnt;                        // one window only
-        } else {
-            wi_step = groups;
-        }
-    }
-    struct Cursor { int wi, img; };
-    auto valid = [&](const Cursor& c) -> bool { return MASKED ? c.wi < cnt : c.img < n_img; };
+    // MASKED: the units in window-major order, t = wi * n_img + img, are cut into one stretch per workgroup (lengths
+    // differ by at most one), so a workgroup changes its window once or twice at most
+    const int64_t units_m = (int64_t)cnt * n_img;
+    const int t_first = MASKED ? (int)(units_m * grp / groups) : 0;
+    const int t_count = MASKED ? (int)(units_m * (grp + 1) / groups) - t_first : 0;
+    struct Cursor { int wi, img, left; };
+    auto valid = [&](const Cursor& c) -> bool { return MASKED ? c.left > 0 : c.img < n_img; };
     auto first = [&]() -> Cursor {
         Cursor c;
-        if (MASKED) { c.wi = wi0; c.img = img0; if (img0 >= n_img) c.wi = cnt; }
+        c.left = t_count;
+        if (MASKED) { c.wi = t_first / n_img; c.img = t_first - c.wi * n_img; }
         else { c.img = cnt > 0 ? grp / cnt : n_img; c.wi = cnt > 0 ? grp - c.img * cnt : 0; }
         return c;
     };
     auto next = [&](Cursor c) -> Cursor {
         if (MASKED) {
-            c.img += img_step;
-            if (c.img >= n_img) { c.img = img0; c.wi += wi_step; }
+            c.left -= 1;
+            c.img += 1;
+            if (c.img >= n_img) { c.img = 0; c.wi += 1; }
         } else {
             const int t = c.img * cnt + c.wi + groups;
             c.img = t / cnt;
@@ -432,7 +427,7 @@ __global__ void __launch_bounds__(64 * NT, 3) bwd_fused_kernel(const BwdParams p
         int ln = lane;
         asm volatile("" : "+v"(ln));
         const int q = wave * 16 + (ln & 15), gg = ln >> 4;
-        float* dst = p.part_dbias + ((int64_t)h * p.db_parts + p.db_slot0 + grp) * p.npk_tot * p.r_tot;
+        float* dst = p.part_dbias + ((int64_t)h * p.db_parts + slot) * p.npk_tot * p.r_tot;
 #pragma unroll
         for (int kp = 0; kp < NT / 2; kp++)
 #pragma unroll
@@ -448,50 +443,78 @@ __global__ void __launch_bounds__(64 * NT, 3) bwd_fused_kernel(const BwdParams p
         if (tid == 0) {
             float tot = 0.f;
             for (int i = 0; i < (nthreads >> 6); i++) tot += lds_red[i];
-            p.part_dscale[(int64_t)h * p.ds_parts + p.ds_slot0 + grp] = tot * s_true;
+            p.part_dscale[(int64_t)h * p.ds_parts + slot] = tot * s_true;
         }
     }
+}
+
+// One launch for all the units of a call: without a mask every workgroup runs the plain body; with one, the workgroups
+// of a head are split between the windows whose mask is all zero and the others in proportion to their numbers (every
+// window has the same number of images) and run side by side.  Without mask flags every window counts as masked.
+// Every workgroup owns slot grp of its head's partial tiles.  With a single workgroup per head it runs one class
+// after the other and writes two slots.
+template <int DT, bool HAS_BIAS, int MASK_DT, int NT, bool VEC, bool MAPPED>
+__global__ void __launch_bounds__(64 * NT, 3) bwd_fused_kernel(const BwdParams p) {
+    const int groups = p.dq_groups;
+    const int h = blockIdx.x / groups;
+    const int grp = blockIdx.x - h * groups;
+#define FWA2_FUSED_BODY(M, G0, GN, SLOT) bwd_fused_body<DT, HAS_BIAS, MASK_DT, NT, VEC, M, MAPPED>(p, h, G0, GN, SLOT)
+    if constexpr (MASK_DT < 0) {
+        FWA2_FUSED_BODY(false, grp, groups, grp);
+    } else {
+        if (groups < 2) {
+            FWA2_FUSED_BODY(false, 0, 1, 0);
+            __syncthreads();
+            FWA2_FUSED_BODY(true, 0, 1, 1);
+            return;
+        }
+        const int nw = p.n_windows;
+        int n_masked = nw;
+        if (p.mask_live != nullptr) {
+            const int lane = threadIdx.x & 63;
+            n_masked = 0;
+            for (int base = 0; base < nw; base += 64) {
+                const int w = base + lane;
+                const uint8_t f = w < nw ? p.mask_live[w] : (uint8_t)0;
+                n_masked += __popcll(__ballot(f != 0));
+            }
+            n_masked = __builtin_amdgcn_readfirstlane(n_masked);
+        }
+        if (n_masked == 0) {
+            FWA2_FUSED_BODY(false, grp, groups, grp);
+        } else if (n_masked == nw) {
+            FWA2_FUSED_BODY(true, grp, groups, grp);
+        } else {
+            int g_masked = (int)(((int64_t)groups * n_masked + nw / 2) / nw);
+            g_masked = g_masked < 1 ? 1 : (g_masked > groups - 1 ? groups - 1 : g_masked);
+            const int g_plain = groups - g_masked;
+            if (grp < g_plain) FWA2_FUSED_BODY(false, grp, g_plain, grp);
+            else FWA2_FUSED_BODY(true, grp - g_plain, g_masked, grp);
+        }
+    }
+#undef FWA2_FUSED_BODY
 }
 
 // ---- host side -----------------------------------------------------------------
 int backward_fused_supported(int n) { return n >= 1 && n <= 64; }
 
-// Launches the kernel(s); reports how many partial tiles / dscale partials per head they wrote.
+// Launches the kernel; reports how many partial tiles / dscale partials per head it wrote.
 template <int DT, bool HAS_BIAS, int MASK_DT, bool VEC, bool MAPPED>
 static hipError_t launch_map(BwdParams p, hipStream_t st, int max_groups, int* parts_out) {
     constexpr int NT = 4;
     // wavefront pairs share a 32-key group in phase B, so there is always an even number of them
     const int waves = 2 * ((p.n + 31) / 32);
-    static std::atomic<int> fit_plain_by_device[kFitDevices], fit_masked_by_device[kFitDevices];
-    const int fit_plain =
-        resident_per_cu_cached(bwd_fused_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, false, MAPPED>, 64 * NT, fit_plain_by_device);
-    const int fit_masked =
-        MASK_DT >= 0 ? resident_per_cu_cached(bwd_fused_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, true, MAPPED>, 64 * NT, fit_masked_by_device)
-                     : 1;
-    auto groups_for = [&](int fit) {
-        int groups = (p.cus * fit) / p.heads;
-        if (groups < 1) groups = 1;
-        if (groups > p.bw) groups = p.bw;
-        if (groups > max_groups) groups = max_groups;
-        return groups;
-    };
-    const bool two = MASK_DT >= 0 && p.mask_live != nullptr;
-    const int g_plain = (MASK_DT < 0 || two) ? groups_for(fit_plain) : 0;
-    const int g_masked = MASK_DT >= 0 ? groups_for(fit_masked) : 0;
-    p.ds_parts = p.db_parts = g_plain + g_masked;
+    static std::atomic<int> fit_by_device[kFitDevices];
+    const int fit = resident_per_cu_cached(bwd_fused_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, MAPPED>, 64 * NT, fit_by_device);
+    int groups = (p.cus * fit) / p.heads;
+    if (groups < 1) groups = 1;
+    if (groups > p.bw) groups = p.bw;
+    if (groups > max_groups) groups = max_groups;
+    p.dq_groups = groups;
+    p.ds_parts = p.db_parts = (MASK_DT >= 0 && groups < 2) ? 2 : groups;
+    p.ds_slot0 = p.db_slot0 = 0;
     if (p.ev_start) (void)hipEventRecord(p.ev_start, st);
-    if (g_plain) {
-        p.dq_groups = g_plain;
-        p.ds_slot0 = p.db_slot0 = 0;
-        hipLaunchKernelGGL((bwd_fused_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, false, MAPPED>), dim3(p.heads * g_plain),
-                           dim3(64 * waves), 0, st, p);
-    }
-    if (g_masked) {
-        p.dq_groups = g_masked;
-        p.ds_slot0 = p.db_slot0 = g_plain;
-        hipLaunchKernelGGL((bwd_fused_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, true, MAPPED>), dim3(p.heads * g_masked),
-                           dim3(64 * waves), 0, st, p);
-    }
+    hipLaunchKernelGGL((bwd_fused_kernel<DT, HAS_BIAS, MASK_DT, NT, VEC, MAPPED>), dim3(p.heads * groups), dim3(64 * waves), 0, st, p);
     if (p.ev_stop) (void)hipEventRecord(p.ev_stop, st);
     *parts_out = p.ds_parts;
     return hipGetLastError();

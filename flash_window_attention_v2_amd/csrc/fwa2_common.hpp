@@ -101,6 +101,14 @@ __device__ __forceinline__ V8 zero8() {
     return z;
 }
 
+// An LDS array that every function instantiated with the same arguments shares: the two bodies a kernel may run
+// (one per class of windows) name the same arrays this way, so the kernel's LDS is that of one body.
+template <class T, int COUNT, int TAG>
+__device__ __forceinline__ __attribute__((returns_nonnull)) T* shared_array() {
+    __shared__ __attribute__((aligned(16))) T a[COUNT];
+    return a;
+}
+
 // Two transposing LDS reads glued into one 8-element MFMA operand.
 template <int DT>
 __device__ __forceinline__ typename Elem<DT>::V8 lds_tr8(const typename Elem<DT>::E* lo,

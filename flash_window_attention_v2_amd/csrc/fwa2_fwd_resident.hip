@@ -49,15 +49,7 @@ namespace fwa2 {
 // wavefront 256 registers, half as many wavefronts per workgroup.
 // FULL: the window has exactly 16 NT tokens (64, 128, 256), so the window length is a compile-time constant and
 // every bounds check, clamp and per-tile branch on it folds away.
-// An LDS array that every function instantiated with the same arguments shares: the two bodies a kernel may run
-// (one per class of windows) name the same arrays this way, so the kernel's LDS is that of one body.
-template <class T, int COUNT, int TAG>
-__device__ __forceinline__ __attribute__((returns_nonnull)) T* shared_array() {
-    __shared__ __attribute__((aligned(16))) T a[COUNT];
-    return a;
-}
-
-// LDS address (a scalar) of a wavefront-uniform pointer into one of those arrays: the low half of its flat address.
+// LDS address (a scalar) of a wavefront-uniform pointer into one of the shared_array() arrays: the low half of its flat address.
 // (Cast to the LDS address space instead, the pointer would be checked for null at run time wherever the compiler
 // has moved the cast behind a readfirstlane and no longer knows where the pointer came from.)
 __device__ __forceinline__ uint32_t lds_offset(const void* p) {
