@@ -150,6 +150,23 @@ def test_more_windows_than_the_key_side_kernel_lists():
     _run_and_check(inp, torch.bfloat16, tag="260 windows of 192 tokens")
 
 
+@pytest.mark.parametrize("n,heads", [(256, 260), (256, 90), (64, 900)])
+def test_more_heads_than_workgroups(n, heads):
+    """With more heads than the device has room for persistent workgroups, every head gets a single workgroup, which
+    then walks the windows without a live mask and the masked ones one class after the other (forward and the fused
+    backward write two partial tiles per head in that case).  260 heads of 256 tokens: one workgroup per head (their
+    score tables exceed the table budget, so the backward is the key-side + dq pair); 90 heads: two workgroups per head,
+    one per class, and the one-pass backward; 900 heads of 64 tokens: one workgroup per head in the fused backward."""
+    n_w = 3
+    inp = make_inputs(batch=2, n_windows=n_w, heads=heads, n=n, dtype=torch.bfloat16, seed=300 + n, with_mask=False)
+    g = torch.Generator().manual_seed(301 + n)
+    mask = torch.where(torch.rand(n_w, n, n, generator=g) < 0.25, -100.0, 0.0)
+    mask[1] = 0.0                                   # one window without a live mask
+    mask[:, torch.arange(n), torch.arange(n)] = 0.0
+    inp["mask"] = mask.to(torch.bfloat16)
+    _run_and_check(inp, torch.bfloat16, tag=f"{heads} heads of {n}-token windows", dscale_l1_frac=0.1)
+
+
 @pytest.mark.parametrize("n", [1, 7, 17, 31, 33, 47, 63, 65, 100, 129, 196, 200, 225, 255])
 def test_ragged_window_sizes(n):
     """Window sizes that are no multiple of 8, 16 or 32 (bias and mask rows padded to 8 entries above 64 tokens
