@@ -35,7 +35,7 @@ HBM_PEAK_GBS = 8000.0              # MI355X HBM3E
 # HBM bytes per launch of the backward kernel at the benchmark shape, from
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a copy kernel of known size
 # (profiles/kernels_C3_fwd_bwd.txt: FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0).
-BWD_KERNEL_TRAFFIC_BYTES = 1.812e9
+BWD_KERNEL_TRAFFIC_BYTES = 1.805e9
 # device memory the library holds on every GPU whether or not it is used (the scratch of fwa2_backward_static)
 STATIC_SCRATCH_MB = 128.0
 
