@@ -109,6 +109,30 @@ __device__ __forceinline__ __attribute__((returns_nonnull)) T* shared_array() {
     return a;
 }
 
+// Sum of the squares of 8 packed elements on the dot unit (two products per instruction, fp32 accumulation).
+__device__ __forceinline__ float sumsq8(bf16x8 a) {
+    typedef __bf16 v2 __attribute__((ext_vector_type(2)));
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        v2 x;
+        x[0] = a[2 * j]; x[1] = a[2 * j + 1];
+        s = __builtin_amdgcn_fdot2_f32_bf16(x, x, s, false);
+    }
+    return s;
+}
+__device__ __forceinline__ float sumsq8(f16x8 a) {
+    typedef _Float16 v2 __attribute__((ext_vector_type(2)));
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        v2 x;
+        x[0] = a[2 * j]; x[1] = a[2 * j + 1];
+        s = __builtin_amdgcn_fdot2(x, x, s, false);
+    }
+    return s;
+}
+
 // Two transposing LDS reads glued into one 8-element MFMA operand.
 template <int DT>
 __device__ __forceinline__ typename Elem<DT>::V8 lds_tr8(const typename Elem<DT>::E* lo,

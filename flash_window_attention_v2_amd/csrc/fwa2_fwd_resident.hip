@@ -311,10 +311,7 @@ __device__ __forceinline__ void fwd_resident_body(const FwdParams& p, const int 
             const V8 vv = ld8<V8>(lds_rawV + frow * 32 + fc8);
             float x[8];
             unpack8(kk, x);
-            float ss = 0.f;
-#pragma unroll
-            for (int j = 0; j < 8; j++) ss += x[j] * x[j];
-            ss = quad_add(ss);
+            const float ss = quad_add(sumsq8(kk));
             const float inv = inv_norm(ss);
             SV8 kn;
 #pragma unroll
@@ -355,10 +352,7 @@ __device__ __forceinline__ void fwd_resident_body(const FwdParams& p, const int 
             const V8 qq = ld8<V8>(lds_rawQ + (wave * WR + 16 * u + l16) * 32 + 8 * g);
             float x[8];
             unpack8(qq, x);
-            float ss = 0.f;
-#pragma unroll
-            for (int j = 0; j < 8; j++) ss += x[j] * x[j];
-            ss = col_add(ss);
+            const float ss = col_add(sumsq8(qq));
             const float sc = scale2 * inv_norm(ss);
 #pragma unroll
             for (int j = 0; j < 8; j++) bq[u][j] = (SE)(x[j] * sc);
