@@ -735,7 +735,7 @@ static BwdPlan make_plan(int heads, int n, int bw, bool has_bias, bool has_mask,
     pl.groups = groups;
     size_t off = 0;
     pl.off_dbias = off;
-    // one partial tile per workgroup and launch: two launches (masked / unmasked units) except for the one-pass kernel
+    // one partial tile per workgroup and launch: two launches (masked / unmasked units) of bwd_kernel, one of the others
     if (has_bias) off += align256((size_t)heads * (pl.one_pass ? 1 : 2) * groups * pl.npk * pl.r * 4);
     dq_geometry(n, &pl.dq_waves, &pl.dq_chunks);
     pl.ds_parts = bw * pl.dq_chunks;

@@ -124,7 +124,7 @@ __device__ __forceinline__ void bwd_fused_body(const BwdParams& p, const int h, 
     // the bf16 range
     const bool fold = (DT == FWA2_BF16) && (2.f * scale2 <= kGapLimit);
 
-    // ---- which units belong to this launch (same dealing as in fwa2_fwd_resident.hip) ----
+    // ---- which units belong to this class of windows (same dealing as in fwa2_fwd_resident.hip) ----
     const int nw = MASK_DT >= 0 ? p.n_windows : 1;
     const bool listed = MASK_DT >= 0 && p.mask_live != nullptr;
     if (listed) {
