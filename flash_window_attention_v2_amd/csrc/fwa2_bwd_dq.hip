@@ -49,23 +49,30 @@ __global__ void __launch_bounds__(512) bwd_dq_kernel(const BwdParams p) {
     const int li = lane & 15;        // lane inside its 16-lane block (transpose reads)
     const int blk1 = (lane >> 4) & 1;
 
-    int idx = blockIdx.x;
+    // Workgroups go to the 8 XCDs in turn, each with an L2 of its own; a group of 8 consecutive workgroups (one per
+    // XCD) does one kind of work.
+    //  - Some groups sum the fp32 dk / dv partials of the key-side kernel (bound by HBM, while the dq work is bound by
+    //    compute).  They are spread evenly among the others: with D dq groups out of T, group g does dq work iff
+    //    floor((g + 1) D / T) > floor(g D / T), as dq group floor(g D / T).
+    //  - dq group j on XCD x takes query chunk j % chunks of unit (j / chunks) * 8 + x: the chunks of one unit run on
+    //    one XCD, which fetches the unit's K and V once for all of them; and the units run head by head, so that the
+    //    workgroups in flight share one head's bias rows in the L2s.
+    const int xcd = blockIdx.x & 7;
+    int64_t j = blockIdx.x >> 3;
     if (p.dkv_blocks > 0) {
-        // Some workgroups of this launch sum the fp32 dk / dv partials of the key-side kernel instead (bound by HBM,
-        // while the dq work is bound by compute).  They are spread evenly among the others: with D dq workgroups out
-        // of T, workgroup i does dq work iff floor((i + 1) D / T) > floor(i D / T), as dq workgroup floor(i D / T).
-        const int64_t total = gridDim.x, dq_blocks = total - p.dkv_blocks;
-        const int64_t before = (int64_t)idx * dq_blocks / total, upto = ((int64_t)idx + 1) * dq_blocks / total;
+        const int64_t total = gridDim.x >> 3, dq_groups = total - p.dkv_blocks;
+        const int64_t before = j * dq_groups / total, upto = (j + 1) * dq_groups / total;
         if (upto == before) {
-            dkv_reduce_rows<DT>(p, idx - before, (int)blockDim.x, (int)threadIdx.x);
+            dkv_reduce_rows<DT>(p, (j - before) * 8 + xcd, (int)blockDim.x, (int)threadIdx.x);
             return;
         }
-        idx = (int)before;
+        j = before;
     }
-    const int qc = idx % p.dq_chunks;
-    idx /= p.dq_chunks;
-    const int h = idx % p.heads;
-    const int b = idx / p.heads;
+    const int qc = (int)(j % p.dq_chunks);
+    const int64_t unit = (j / p.dq_chunks) * 8 + xcd;
+    if (unit >= (int64_t)p.bw * p.heads) return;
+    const int h = (int)(unit / p.bw);
+    const int b = (int)(unit - (int64_t)h * p.bw);
 
     // rows are addressed through the window map when there is one (cyclic shift + window partition done here)
     const E* qptr = reinterpret_cast<const E*>(p.q.ptr) + unit_off_any(p.q, p.map, b, h);
@@ -303,12 +310,14 @@ hipError_t launch_backward_dq(const BwdParams& p_in, int dtype, bool has_bias, i
     const int chunk_rows = ((p.n < kKeyChunk ? p.n : kKeyChunk) + 63) & ~63;
     const size_t smem = (size_t)2 * chunk_rows * kLdsStride * 2 + 8 * sizeof(float);
     const dim3 block(64 * p.dq_waves);
-    const int64_t dq_blocks = (int64_t)p.bw * p.heads * p.dq_chunks;
-    // the fp32 dk / dv partials of the super-tiled key-side kernel are summed by extra workgroups of this launch
+    // groups of 8 workgroups: dq groups cover (unit, chunk) for the units rounded up to a multiple of 8 ...
+    const int64_t dq_groups = (((int64_t)p.bw * p.heads + 7) / 8) * p.dq_chunks;
+    // ... and the fp32 dk / dv partials of the super-tiled key-side kernel are summed by extra groups of this launch
     const int64_t rows_per_block = block.x / 4, rows = (int64_t)p.bw * p.heads * p.n;
-    p.dkv_blocks = p.n_chunks > 1 ? (int)((rows + rows_per_block - 1) / rows_per_block) : 0;
-    if (dq_blocks + p.dkv_blocks > 0x7fffffffLL) return hipErrorInvalidValue;
-    dim3 grid((unsigned)(dq_blocks + p.dkv_blocks));
+    const int64_t dkv_blocks = p.n_chunks > 1 ? (rows + rows_per_block - 1) / rows_per_block : 0;
+    p.dkv_blocks = (int)((dkv_blocks + 7) / 8);        // (counted in groups)
+    if ((dq_groups + p.dkv_blocks) * 8 > 0x7fffffffLL) return hipErrorInvalidValue;
+    dim3 grid((unsigned)((dq_groups + p.dkv_blocks) * 8));
     if (dtype == FWA2_BF16) return launch_dt<FWA2_BF16>(p, has_bias, mask_dt, grid, block, smem, st);
     return launch_dt<FWA2_F16>(p, has_bias, mask_dt, grid, block, smem, st);
 }

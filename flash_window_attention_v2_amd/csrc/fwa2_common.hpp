@@ -513,7 +513,7 @@ struct BwdParams {
     float* part_dv;
     int dq_waves;        // wavefronts per workgroup of the dq kernel
     int dq_chunks;       // dq workgroups per (bw, head)
-    int dkv_blocks;      // windows of more than 256 tokens: workgroups of the dq launch that sum the dk / dv partials instead
+    int dkv_blocks;      // dq launch for windows beyond 256 tokens: groups of 8 workgroups that sum dk / dv partials
     bool side_vec;       // rows of bias and mask (query-major) may be read with 16-byte loads, n % 8 == 0
     bool side_vec_rows;  // ... or n % 8 != 0 but every row is at least n rounded up to 8 entries long (resident kernels)
     const void* bias_t;  // [H, NP, NQ] input dtype: bias transposed to key-major, zero padded

@@ -54,11 +54,22 @@ __global__ void __launch_bounds__(512) fwd_kernel(const FwdParams p) {
     const int li = lane & 15;        // lane inside its 16-lane block (transpose reads)
     const int blk1 = (lane >> 4) & 1;
 
-    int idx = blockIdx.x;
-    const int qc = idx % p.q_chunks;
-    idx /= p.q_chunks;
-    const int h = idx % p.heads;
-    const int b = idx / p.heads;
+    // Workgroup -> (query chunk, unit).  Workgroups go to the 8 XCDs in turn, each with an L2 of its own, so the
+    // chunks of one unit are given to workgroups 8 apart (one XCD fetches the unit's K and V once for all of them),
+    // and the units run head by head, so that the workgroups in flight share one head's bias rows in those L2s.
+    const int units = p.bw * p.heads, units8 = units & ~7;
+    int qc, unit;
+    if ((int)blockIdx.x < units8 * p.q_chunks) {
+        const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
+        qc = j % p.q_chunks;
+        unit = (j / p.q_chunks) * 8 + xcd;
+    } else {
+        const int r = blockIdx.x - units8 * p.q_chunks;
+        qc = r % p.q_chunks;
+        unit = units8 + r / p.q_chunks;
+    }
+    const int h = unit / p.bw;
+    const int b = unit - h * p.bw;
 
     // rows are addressed through the window map when there is one (cyclic shift + window partition done here)
     const E* qptr = reinterpret_cast<const E*>(p.q.ptr) + unit_off_any(p.q, p.map, b, h);
