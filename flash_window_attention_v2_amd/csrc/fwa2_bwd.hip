@@ -230,11 +230,26 @@ __global__ void __launch_bounds__(NQB * 128 / KT) bwd_kernel(const BwdParams p) 
     // ---- which head (and, for BIG, which super-tile) this workgroup owns ----
     int h, grp, q_off = 0, k_off = 0, qs = 0;
     if (BIG) {
-        int idx = blockIdx.x;
-        grp = idx % p.groups; idx /= p.groups;
-        const int ks = idx % p.n_chunks; idx /= p.n_chunks;
-        qs = idx % p.n_chunks;
-        h = idx / p.n_chunks;
+        // Workgroups go to the 8 XCDs in turn, each with an L2 of its own.  The super-tiles of one (head, group) --
+        // workgroups that walk the same units at the same pace -- are given to workgroups 8 apart, so one XCD fetches
+        // a unit's rows once for all of them.
+        // (Only when the (head, group) pairs divide evenly among the XCDs: otherwise some XCDs would hold one pair's
+        // workgroups more than others, which costs more than the shared fetches save -- +2 % at 1024 tokens, where
+        // 12 pairs of 16 super-tiles would fill four XCDs and half-fill the other four.)
+        const int tiles = p.n_chunks * p.n_chunks;
+        int tile, sid;
+        if (p.big_xcd) {
+            const int pos = blockIdx.x >> 3;
+            tile = pos % tiles;
+            sid = (pos / tiles) * 8 + (blockIdx.x & 7);
+        } else {
+            tile = (blockIdx.x / p.groups) % tiles;
+            sid = (blockIdx.x / (p.groups * tiles)) * p.groups + blockIdx.x % p.groups;
+        }
+        h = sid / p.groups;
+        grp = sid - h * p.groups;
+        qs = tile / p.n_chunks;
+        const int ks = tile - qs * p.n_chunks;
         q_off = qs * R;
         k_off = ks * NPk;
     } else {
@@ -796,6 +811,7 @@ static hipError_t launch_main(BwdParams p, const BwdPlan& pl, hipStream_t st, in
     const bool two = !kOneLaunch && MASK_DT >= 0 && p.mask_live != nullptr;
     p.db_parts = two ? 2 * groups : groups;
     p.db_slot0 = 0;
+    p.big_xcd = BIG && (p.heads * groups) % 8 == 0;       // super-tiles of a (head, group) pair on one XCD, see the kernel
     const dim3 grid(p.heads * tiles * groups), block(64 * pl.waves);
     if (p.ev_start) (void)hipEventRecord(p.ev_start, st);
     if constexpr (kOneLaunch) {

@@ -513,6 +513,7 @@ struct BwdParams {
     float* part_dv;
     int dq_waves;        // wavefronts per workgroup of the dq kernel
     int dq_chunks;       // dq workgroups per (bw, head)
+    int big_xcd;         // super-tiled key-side kernel: workgroup order that keeps a (head, group) pair on one XCD
     int dkv_blocks;      // dq launch for windows beyond 256 tokens: groups of 8 workgroups that sum dk / dv partials
     bool side_vec;       // rows of bias and mask (query-major) may be read with 16-byte loads, n % 8 == 0
     bool side_vec_rows;  // ... or n % 8 != 0 but every row is at least n rounded up to 8 entries long (resident kernels)
